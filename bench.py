@@ -1,0 +1,389 @@
+#!/usr/bin/env python3
+"""Benchmark of the torch_webgpu op path on one MI355X: achieved HBM GB/s.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n 28]
+
+One "step" is one pass of the three ops the headline metric names, each on 2^28
+fp32 elements already resident in HBM:
+    add.Tensor   two contiguous vectors                      12 B/elem
+    gelu         approximate='none' on [16384, 16384]          8 B/elem
+    masked_select  Bernoulli(0.5) mask, count read back        5 B/elem + 4 B/selected
+`value` is the algorithmic bytes of one step divided by the wall time of one step.
+After the timed steps every other configuration (silu, relu, row-bias and
+transposed add, eq / ne / bitwise_and, masked_select at p = 0.01 / 0.99 /
+clustered) is timed per launch with HIP events and listed under "ops".
+
+Kernels are launched through the C ABI of libtwg_hip.so (ctypes); durations come
+from hipEvents recorded on the library's own stream.  The CPU baseline legs time
+(a) the single-threaded C oracle and (b) PyTorch's CPU kernels on the box's cores,
+on bounded samples.  Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "torch-webgpu_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--log2n", type=int, default=28, help="log2 of the element count (28 = the named config)")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-op sweep of the other configs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--only", default="", help="comma list of op names to run in the sweep")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this op path is single-GPU (no collectives, nothing to shard in one "
+            "process); run with --gpus 1.  How it would shard is described in DESIGN.md.")
+        sys.exit(2)
+
+    import torch
+    import twg_capi as capi
+    import twg_workloads as W
+
+    L = capi.load()
+    capi.init()
+    dev_name, cus, mem = capi.device_info()
+    log(f"device: {dev_name}  CUs={cus}  mem={mem / 2**30:.0f} GiB")
+    n = 1 << args.log2n
+    K, Wm = args.steps, args.warmup
+
+    def ev_pair():
+        return capi.Event(), capi.Event()
+
+    def time_launches(fn, warm, reps):
+        """Per-launch durations (ms) from events recorded around each call."""
+        for _ in range(warm):
+            fn()
+        capi.sync()
+        evs = [ev_pair() for _ in range(reps)]
+        for s, e in evs:
+            s.record()
+            fn()
+            e.record()
+        capi.sync()
+        return [s.elapsed_ms(e) for s, e in evs]
+
+    def summarize(name, kernel, nbytes, ms_list, nelem, extra=None):
+        avg = sum(ms_list) / len(ms_list)
+        med = statistics.median(ms_list)
+        d = {
+            "op": name, "kernel": kernel, "elements": nelem, "bytes": nbytes,
+            "avg_ms": round(avg, 5), "median_ms": round(med, 5), "min_ms": round(min(ms_list), 5),
+            "GBps": round(nbytes / avg / 1e6, 1),
+            "GBps_median": round(nbytes / med / 1e6, 1),
+            "Gelem_per_s": round(nelem / avg / 1e6, 2),
+            "pct_hbm_peak": round(nbytes / avg / 1e6 / HBM_PEAK_GBS * 100, 2),
+        }
+        if extra:
+            d.update(extra)
+        log(f"  {name:28s} {d['avg_ms']:9.4f} ms  {d['GBps']:8.1f} GB/s  {d['pct_hbm_peak']:6.2f}% of peak")
+        return d
+
+    f32 = ctypes.c_float
+
+    # ------------------------------------------------------------ headline inputs
+    t0 = time.time()
+    log(f"generating inputs for n = 2^{args.log2n} ...")
+    rows = 1 << (args.log2n // 2)
+    cols = n // rows
+    a_h, b_h = W.add_contiguous(n, seed=0)
+    x_h = W.activation_input(rows, cols, seed=1).view(-1)
+    src_h = W.select_source(n, seed=4)
+    m50_h = W.bernoulli_mask(n, 0.5)
+    k50 = int(m50_h.sum())
+    d_a, d_b, d_x, d_src, d_m = (capi.to_device(t) for t in (a_h, b_h, x_h, src_h, m50_h))
+    d_out = capi.DeviceBuffer(4 * n)
+    d_cnt = capi.DeviceBuffer(8)
+    scratch_bytes = L.twg_masked_select_scratch_bytes(n)
+    d_scratch = capi.DeviceBuffer(scratch_bytes)
+    it = capi.dense_iter(n)
+    cnt_host = torch.zeros(1, dtype=torch.int64)
+    capi.sync()
+    log(f"  inputs ready in {time.time() - t0:.1f} s")
+
+    def run_add():
+        capi.check(L.twg_add_f32(d_out.ptr, d_a.ptr, d_b.ptr, f32(1.0), ctypes.byref(it), None))
+
+    def run_gelu():
+        capi.check(L.twg_unary_f32(capi.UNARY_GELU_ERF, d_out.ptr, d_x.ptr, ctypes.byref(it), None))
+
+    def launch_ms(mask_buf):
+        capi.check(L.twg_masked_select_f32(d_out.ptr, d_cnt.ptr, d_src.ptr, mask_buf.ptr,
+                                           ctypes.byref(it), d_scratch.ptr, scratch_bytes, None))
+
+    def read_count():
+        capi.check(L.twg_memcpy_d2h(cnt_host.data_ptr(), d_cnt.ptr, 8, None))
+        return int(cnt_host[0])
+
+    def run_ms():
+        launch_ms(d_m)
+        return read_count()
+
+    bytes_add = W.BYTES_PER_ELEM["add"] * n
+    bytes_gelu = W.BYTES_PER_ELEM["gelu"] * n
+    bytes_ms = W.masked_select_bytes(n, k50)
+    step_bytes = bytes_add + bytes_gelu + bytes_ms
+
+    # ------------------------------------------------------------ timed steps
+    log(f"timing {K} steps after {Wm} warm-up steps ...")
+    for _ in range(Wm):
+        run_add(); run_gelu(); assert run_ms() == k50
+    capi.sync()
+    ev = [[capi.Event() for _ in range(5)] for _ in range(K)]
+    t_start = time.perf_counter()
+    for i in range(K):
+        e = ev[i]
+        e[0].record(); run_add()
+        e[1].record(); run_gelu()
+        e[2].record(); launch_ms(d_m)
+        e[3].record(); got = read_count()
+        e[4].record()
+        if got != k50:
+            raise RuntimeError(f"masked_select count {got} != {k50}")
+    capi.sync()
+    t_stop = time.perf_counter()
+    ms_per_step = (t_stop - t_start) * 1e3 / K
+    value = step_bytes / (ms_per_step * 1e6)  # GB/s
+
+    ops = []
+    add_ms = [e[0].elapsed_ms(e[1]) for e in ev]
+    gelu_ms = [e[1].elapsed_ms(e[2]) for e in ev]
+    msk_ms = [e[2].elapsed_ms(e[3]) for e in ev]   # scratch clear + compaction kernel
+    mso_ms = [e[2].elapsed_ms(e[4]) for e in ev]   # ... plus the 8-byte count read-back
+    head = [
+        summarize("add", "ew_contig<AddOp>", bytes_add, add_ms, n),
+        summarize("gelu", "ew_contig<GeluErfOp>", bytes_gelu, gelu_ms, n),
+        summarize("masked_select_p0.50", "ms_compact<4>", bytes_ms, msk_ms, n,
+                  {"selected": k50, "op_ms_with_count_readback": round(sum(mso_ms) / K, 5)}),
+    ]
+    ops += head
+    dominant = max(head, key=lambda d: d["avg_ms"])
+    roofline = {
+        "bound": "hbm", "kernel": dominant["kernel"], "op": dominant["op"],
+        "achieved": dominant["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(dominant["GBps"] / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "algorithmic_bytes_per_launch": dominant["bytes"],
+        "avg_launch_ms": dominant["avg_ms"],
+    }
+    tr = os.path.join(ROOT, "profiles", "hbm_traffic_bytes.json")
+    if os.path.exists(tr):  # measured FETCH_SIZE + WRITE_SIZE per launch, scaled by a copy kernel
+        with open(tr) as f:
+            traffic = json.load(f)
+        roofline["traffic"] = traffic.get(dominant["op"] + f"@2^{args.log2n}")
+
+    # ------------------------------------------------------------ sweep of the other configs
+    del a_h, b_h
+    only = set(filter(None, args.only.split(",")))
+
+    def want(name):
+        return not only or name in only
+
+    result_sweep = []
+    if not args.no_sweep:
+        log("sweep of the remaining configurations ...")
+        result_sweep = sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summarize,
+                             d_out, d_cnt, d_scratch, scratch_bytes, d_src, d_x, it, cnt_host, want)
+    ops += result_sweep
+
+    # ------------------------------------------------------------ CPU baselines
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(torch, W, n, x_h, src_h, m50_h, step_bytes, bytes_add, bytes_gelu, bytes_ms)
+
+    out = {
+        "metric": "HBM GB/s (% of peak) for add/gelu/masked_select at 2^28 fp32, 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": Wm,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"one step = add.Tensor + gelu(approximate='none') + masked_select"
+                               f"(Bernoulli 0.5) on 2^{args.log2n} fp32 elements resident in HBM "
+                               "(configs[1] shape [16384,16384] for gelu; configs[0]/[4] shapes for "
+                               "add and masked_select at the same element count)",
+                   "elements": n, "step_bytes": step_bytes},
+        "pct_hbm_peak": round(value / HBM_PEAK_GBS * 100, 2),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "ops": ops,
+        "device": {"name": dev_name, "compute_units": cus},
+    }
+    print(json.dumps(out), flush=True)
+
+
+def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summarize,
+          d_out, d_cnt, d_scratch, scratch_bytes, d_src, d_x, it, cnt_host, want):
+    f32 = ctypes.c_float
+    res = []
+    by = W.BYTES_PER_ELEM
+
+    # config 2: silu, relu on the gelu input
+    for name, op in (("silu", capi.UNARY_SILU), ("relu", capi.UNARY_RELU),
+                     ("gelu_tanh", capi.UNARY_GELU_TANH)):
+        if want(name):
+            ms = time_launches(lambda: capi.check(L.twg_unary_f32(op, d_out.ptr, d_x.ptr,
+                                                                   ctypes.byref(it), None)), Wm, K)
+            res.append(summarize(name, f"ew_contig<{name}>", 8 * n, ms, n))
+
+    # config 3: row-bias add and transposed add
+    if want("add_rowbias") or want("add_transposed"):
+        r3, c3 = (1 << (args.log2n // 2 - 1)), 0
+        c3 = n // r3  # 8192 x 32768 at 2^28
+        a_h, bias_h, c_h = W.broadcast_add_inputs(r3, c3, seed=2)
+        d_a3, d_bias, d_c3 = capi.to_device(a_h), capi.to_device(bias_h), capi.to_device(c_h)
+        del a_h, c_h
+        if want("add_rowbias"):
+            it_rb = capi.make_iter((r3, c3), (c3, 1), (c3, 1), (0, 1))
+            ms = time_launches(lambda: capi.check(L.twg_add_f32(d_out.ptr, d_a3.ptr, d_bias.ptr, f32(1.0),
+                                                                ctypes.byref(it_rb), None)), Wm, K)
+            res.append(summarize("add_rowbias", "ew_rows<AddOp>", by["add_rowbias"] * n + 4 * c3, ms, n,
+                                 {"shape": [r3, c3]}))
+        if want("add_transposed"):
+            # A viewed as (c3, r3) with strides (1, c3) + contiguous C[c3, r3]; at::TensorIterator
+            # gives the output the first input's layout, so dimension 0 of the iterator is the
+            # logical dimension 0 (stride 1 for out and A, stride r3 for C).
+            it_t = capi.Iter()
+            it_t.ndim = 2
+            it_t.numel = n
+            it_t.shape[0], it_t.shape[1] = c3, r3
+            for slot, st in ((capi.OUT, (1, c3)), (capi.A, (1, c3)), (capi.B, (r3, 1))):
+                it_t.stride[slot][0], it_t.stride[slot][1] = st
+            ms = time_launches(lambda: capi.check(L.twg_add_f32(d_out.ptr, d_a3.ptr, d_c3.ptr, f32(1.0),
+                                                                ctypes.byref(it_t), None)), Wm, K)
+            res.append(summarize("add_transposed", "ew_tile<AddOp>", by["add_transposed"] * n, ms, n,
+                                 {"logical_shape": [c3, r3], "out_strides": [1, c3]}))
+        del d_a3, d_bias, d_c3
+
+    # config 4: eq, ne.Scalar, bitwise_and
+    if want("eq") or want("ne_scalar") or want("bitwise_and"):
+        p_h, q_h, z_h = W.mask_inputs(n, seed=3)
+        d_p, d_q, d_z = capi.to_device(p_h), capi.to_device(q_h), capi.to_device(z_h)
+        del p_h, q_h, z_h
+        d_m1, d_m2, d_m3 = capi.DeviceBuffer(n), capi.DeviceBuffer(n), capi.DeviceBuffer(n)
+        ms = time_launches(lambda: capi.check(L.twg_eq_f32(d_m1.ptr, d_p.ptr, d_q.ptr, ctypes.byref(it), None)), Wm, K)
+        res.append(summarize("eq", "ew_contig<EqOp>", by["eq"] * n, ms, n))
+        ms = time_launches(lambda: capi.check(L.twg_ne_scalar_f32(d_m2.ptr, d_z.ptr, f32(0.0), ctypes.byref(it), None)), Wm, K)
+        res.append(summarize("ne_scalar", "ew_contig<NeScalarOp>", by["ne_scalar"] * n, ms, n))
+        ms = time_launches(lambda: capi.check(L.twg_and_u8(d_m3.ptr, d_m1.ptr, d_m2.ptr, ctypes.byref(it), None)), Wm, K)
+        res.append(summarize("bitwise_and", "ew_contig<AndOp>", by["bitwise_and"] * n, ms, n))
+        del d_p, d_q, d_z, d_m1, d_m2, d_m3
+
+    # config 5: the other masks
+    for name, make in (("masked_select_p0.01", lambda: W.bernoulli_mask(n, 0.01)),
+                       ("masked_select_p0.99", lambda: W.bernoulli_mask(n, 0.99)),
+                       ("masked_select_clustered", lambda: W.clustered_mask(n, 4096))):
+        if not want(name):
+            continue
+        m_h = make()
+        k = int(m_h.sum())
+        d_mask = capi.to_device(m_h)
+        del m_h
+
+        def launch():
+            capi.check(L.twg_masked_select_f32(d_out.ptr, d_cnt.ptr, d_src.ptr, d_mask.ptr,
+                                               ctypes.byref(it), d_scratch.ptr, scratch_bytes, None))
+
+        def full():
+            launch()
+            capi.check(L.twg_memcpy_d2h(cnt_host.data_ptr(), d_cnt.ptr, 8, None))
+
+        ms_kernel = time_launches(launch, Wm, K)
+        ms_full = time_launches(full, 1, K)
+        if int(cnt_host[0]) != k:
+            raise RuntimeError(f"{name}: count {int(cnt_host[0])} != {k}")
+        res.append(summarize(name, "ms_compact<4>", W.masked_select_bytes(n, k), ms_kernel, n,
+                             {"selected": k,
+                              "op_ms_with_count_readback": round(sum(ms_full) / len(ms_full), 5)}))
+        del d_mask
+    return res
+
+
+def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu, bytes_ms):
+    """Times the same three ops on the host: (a) the C oracle, one thread, on samples;
+    (b) PyTorch's CPU kernels on all cores at full size."""
+    from oracle import oracle
+    import torch.nn.functional as F
+
+    OL = oracle.lib()
+    ns_add = min(n, 1 << 26)
+    ns_gelu = min(n, 1 << 24)
+    ns_ms = min(n, 1 << 26)
+    a = torch.rand(ns_add) * 8 - 4
+    b = torch.rand(ns_add) * 8 - 4
+    o = torch.empty(ns_add)
+
+    def best(fn, reps=3):
+        ts = []
+        for _ in range(reps):
+            t = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t)
+        return statistics.median(ts)
+
+    log("CPU baseline: C oracle, 1 thread ...")
+    t_add = best(lambda: OL.oracle_dense_add_f32(o.data_ptr(), a.data_ptr(), b.data_ptr(), 1.0, ns_add))
+    xs = x_h[:ns_gelu].contiguous()
+    og = torch.empty(ns_gelu)
+    t_gelu = best(lambda: OL.oracle_dense_unary_f32(oracle.GELU_ERF, og.data_ptr(), xs.data_ptr(), ns_gelu))
+    ss, msk = src_h[:ns_ms].contiguous(), m_h[:ns_ms].contiguous()
+    om = torch.empty(ns_ms)
+    t_ms = best(lambda: OL.oracle_dense_masked_select_f32(om.data_ptr(), ss.data_ptr(), msk.data_ptr(), ns_ms))
+    g_add = 12 * ns_add / t_add / 1e9
+    g_gelu = 8 * ns_gelu / t_gelu / 1e9
+    g_ms = (5 * ns_ms + 4 * int(msk.sum())) / t_ms / 1e9
+    step_s = bytes_add / g_add / 1e9 + bytes_gelu / g_gelu / 1e9 + bytes_ms / g_ms / 1e9
+    port = {"add_GBps": round(g_add, 2), "gelu_GBps": round(g_gelu, 3), "masked_select_GBps": round(g_ms, 2)}
+
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    log(f"CPU baseline: PyTorch CPU kernels, {threads} threads ...")
+    nt = min(n, 1 << 27)
+    a = torch.rand(nt) * 8 - 4
+    b = torch.rand(nt) * 8 - 4
+    o = torch.empty(nt)
+    xt, st, mt = x_h[:nt], src_h[:nt], m_h[:nt]
+    ta = best(lambda: torch.add(a, b, out=o), 5)
+    tg = best(lambda: F.gelu(xt), 5)
+    tm = best(lambda: torch.masked_select(st, mt), 5)
+    kt = int(mt.sum())
+    ga, gg, gm = 12 * nt / ta / 1e9, 8 * nt / tg / 1e9, (5 * nt + 4 * kt) / tm / 1e9
+    step_t = bytes_add / ga / 1e9 + bytes_gelu / gg / 1e9 + bytes_ms / gm / 1e9
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = [l.split(":", 1)[1].strip() for l in f if l.startswith("model name")][0]
+    except Exception:
+        model = "unknown"
+    return {
+        "value": round(step_bytes / step_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"C oracle (oracle/twg_oracle.c), 1 thread: add on 2^{ns_add.bit_length() - 1}, "
+                  f"gelu on 2^{ns_gelu.bit_length() - 1}, masked_select on 2^{ns_ms.bit_length() - 1} "
+                  "elements, median of 3; per-op GB/s combined into the time of one 2^28 step",
+        "per_op": port,
+        "torch_cpu": {
+            "value": round(step_bytes / step_t / 1e9, 2), "unit": "GB/s", "cores": threads,
+            "cpu_model": model,
+            "sample": f"torch.add / F.gelu / torch.masked_select on 2^{nt.bit_length() - 1} elements, "
+                      "median of 5 (ATen's CPU kernel is the reference's own masked_select)",
+            "per_op": {"add_GBps": round(ga, 2), "gelu_GBps": round(gg, 2),
+                       "masked_select_GBps": round(gm, 2)},
+        },
+    }
+
+
+if __name__ == "__main__":
+    main()

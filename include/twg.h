@@ -1,0 +1,214 @@
+/*
+ * twg.h - C ABI of libtwg_hip.so, the gfx950 (MI355X) kernel library that sits
+ * underneath the "webgpu" PrivateUse1 backend of torch_webgpu.
+ *
+ * The reference (jmaczan/torch-webgpu) has no FFI of its own: its op layer talks
+ * to Google Dawn through C++ objects.  Every entry point below therefore cites the
+ * reference C++ function whose work it takes over.  No torch and no HIP types
+ * cross this line: plain pointers, sizes and POD structs only, so the same
+ * library is driven from the torch extension (csrc/torch), from ctypes, or from
+ * any other host language with a C FFI.
+ *
+ * Conventions
+ *  - Every function returns 0 on success.  A positive value is a hipError_t, a
+ *    negative value is one of the TWG_E_* codes; twg_error_string() decodes both.
+ *  - Device pointers are real device addresses, already advanced by the tensor's
+ *    storage offset (the reference instead passes whole buffers plus element
+ *    offsets: csrc/ops/binary.h:101-103, csrc/ops/unary.h:82-83).
+ *  - `stream` is a hipStream_t passed as an opaque pointer; NULL selects the
+ *    library's own in-order stream (the stand-in for the reference's single Dawn
+ *    queue, csrc/core/webgpu_context.cpp:44).  Launches are asynchronous.
+ *  - Iteration geometry travels in twg_iter_t, the 64-bit widening of the
+ *    reference's uniform `Params` blocks (csrc/ops/binary.h:108-124,
+ *    csrc/ops/unary.h:88-101).  Dimension 0 is the fastest-moving one, which is
+ *    the order at::TensorIterator presents.  Strides are in elements, may be 0
+ *    (broadcast) and may be negative.
+ */
+#ifndef TWG_H_
+#define TWG_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TWG_MAX_DIMS 8 /* csrc/ops/binary.h:105 (MAX_DIMS) */
+
+/* negative (library) error codes */
+#define TWG_E_INVALID_ARG (-1)   /* bad ndim / negative extent / numel mismatch / null pointer */
+#define TWG_E_UNSUPPORTED (-2)   /* valid request this build has no kernel for */
+#define TWG_E_SCRATCH_SMALL (-3) /* masked_select scratch buffer too small */
+#define TWG_E_OVERLAP (-4)       /* reserved */
+
+typedef struct ihipStream_t *twg_stream_t; /* == hipStream_t */
+typedef struct ihipEvent_t *twg_event_t;   /* == hipEvent_t  */
+
+/* Operand slots of twg_iter_t.stride */
+#define TWG_OUT 0
+#define TWG_A 1
+#define TWG_B 2
+
+typedef struct twg_iter {
+  int32_t ndim;  /* 0..TWG_MAX_DIMS; 0 means a single element */
+  int32_t reserved;
+  int64_t numel; /* product of shape[0..ndim) */
+  int64_t shape[TWG_MAX_DIMS];
+  int64_t stride[3][TWG_MAX_DIMS]; /* [TWG_OUT|TWG_A|TWG_B][dim], elements */
+} twg_iter_t;
+
+/* Unary functor selector: the reference's UnaryOp enum (csrc/ops/unary.h:20-26)
+ * with GeLU split into the formula the reference actually evaluates (tanh,
+ * csrc/ops/unary.cpp:93-95) and the exact erf form ATen means by
+ * approximate='none'. */
+enum twg_unary_op {
+  TWG_UNARY_COPY = 0,      /* csrc/ops/unary.cpp:88-89 */
+  TWG_UNARY_RELU = 1,      /* csrc/ops/unary.cpp:90-92 */
+  TWG_UNARY_GELU_ERF = 2,  /* aten gelu(approximate='none') */
+  TWG_UNARY_GELU_TANH = 3, /* csrc/ops/unary.cpp:93-95 */
+  TWG_UNARY_SILU = 4       /* csrc/ops/unary.cpp:96-98 */
+};
+
+/* ---------------------------------------------------------------- runtime */
+
+/* Bind device 0, create the library stream.  Idempotent, thread safe.  Replaces
+ * the lazy Dawn instance/adapter/device/queue singleton
+ * (csrc/core/webgpu_context.cpp:9-68); unlike it, failure is returned, never
+ * exit(1). */
+int twg_init(void);
+/* 1 once twg_init has succeeded (python/torch_webgpu/webgpu/__init__.py:4-5). */
+int twg_is_initialized(void);
+const char *twg_error_string(int code);
+/* Name, compute-unit count and memory of the bound device (diagnostics, bench). */
+int twg_device_info(char *name, size_t name_cap, int32_t *compute_units,
+                    int64_t *total_mem_bytes);
+/* The library's in-order stream. */
+twg_stream_t twg_default_stream(void);
+int twg_stream_sync(twg_stream_t stream);
+int twg_device_sync(void);
+
+/* Event timing on a given stream (used by the benchmark for the roofline
+ * figures; no reference counterpart: the reference has no timing code). */
+int twg_event_create(twg_event_t *ev);
+int twg_event_destroy(twg_event_t ev);
+int twg_event_record(twg_event_t ev, twg_stream_t stream);
+int twg_event_sync(twg_event_t ev);
+int twg_event_elapsed_ms(float *ms, twg_event_t start, twg_event_t stop);
+
+/* -------------------------------------------------------------- allocator */
+
+/* Caching device allocator.  Replaces WebGPUAllocator::allocate /
+ * WebGPUCachingHostDeleter (csrc/core/webgpu_allocator.cpp:10-29), which create
+ * and destroy one Dawn buffer per tensor.  Blocks are rounded up (512 B below
+ * 1 MiB, 2 MiB above), kept on per-size free lists when freed and handed out
+ * again without touching hipMalloc.  Reuse is safe without events because all
+ * work runs in order on one stream.  n == 0 yields *p == NULL and success
+ * (csrc/core/webgpu_allocator.cpp:33-38). */
+int twg_malloc(void **p, size_t n);
+int twg_free(void *p);
+/* Return every cached (unused) block to the driver. */
+int twg_empty_cache(void);
+
+typedef struct twg_mem_stats {
+  int64_t bytes_in_use;   /* handed out, rounded sizes */
+  int64_t bytes_cached;   /* sitting on free lists */
+  int64_t n_device_mallocs; /* hipMalloc calls so far */
+  int64_t n_cache_hits;   /* twg_malloc calls served from a free list */
+  int64_t n_allocs;       /* twg_malloc calls with n > 0 */
+} twg_mem_stats_t;
+int twg_mem_stats(twg_mem_stats_t *out);
+
+/* ----------------------------------------------------------------- copies */
+
+/* Host -> device.  Replaces queue.WriteBuffer in copy_ (csrc/ops/copy.cpp:74-92).
+ * Pageable host memory is staged through a ring of pinned buffers so the CPU
+ * memcpy of chunk k+1 overlaps the DMA of chunk k; the host range may be reused
+ * as soon as the call returns. */
+int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_stream_t stream);
+/* Device -> host, blocking: on return the bytes are in dst_host.  Replaces the
+ * staging-buffer + MapAsync + WaitAny + memcpy sequence of cpu_copy_with_webgpu
+ * (csrc/ops/copy.cpp:33-56). */
+int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_stream_t stream);
+/* Device -> device, contiguous.  Replaces CopyBufferToBuffer in copy_
+ * (csrc/ops/copy.cpp:95-122).  Ranges must not overlap. */
+int twg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes, twg_stream_t stream);
+/* Fill nbytes with a byte value (kernel, not hipMemset, so it is safe to record
+ * into a HIP graph). */
+int twg_fill_bytes(void *dst_dev, int value, size_t nbytes, twg_stream_t stream);
+
+/* ------------------------------------------------------------ elementwise */
+
+/* out = a + alpha * b in binary32, product and sum rounded separately.
+ * Replaces binary_kernel<BinaryOp::Add> and its WGSL
+ * (csrc/ops/binary.h:29-215, csrc/ops/binary.cpp:55-98), as reached from
+ * add_out_webgpu (csrc/ops/arithmetic.cpp:24-43).  Full broadcasting and
+ * arbitrary strides through `it`. */
+int twg_add_f32(float *out, const float *a, const float *b, float alpha,
+                const twg_iter_t *it, twg_stream_t stream);
+/* out = a + alpha * s for a host scalar s.  The reference lets a CPU scalar
+ * tensor into the iterator and then misreads its storage as a device buffer
+ * (csrc/ops/arithmetic.cpp:37, csrc/ops/binary.h:95); here the scalar is passed
+ * by value.  Uses it->stride[TWG_OUT] and it->stride[TWG_A]. */
+int twg_add_scalar_f32(float *out, const float *a, float s, float alpha,
+                       const twg_iter_t *it, twg_stream_t stream);
+/* out = a * b.  Replaces binary_kernel<BinaryOp::Mul> (csrc/ops/binary.cpp:99-101),
+ * whose registration the reference leaves commented out
+ * (csrc/ops/arithmetic.cpp:45-63,396). */
+int twg_mul_f32(float *out, const float *a, const float *b, const twg_iter_t *it,
+                twg_stream_t stream);
+int twg_mul_scalar_f32(float *out, const float *a, float s, const twg_iter_t *it,
+                       twg_stream_t stream);
+/* out = max(0, a + b).  Replaces binary_kernel<BinaryOp::FusedAddRelu>
+ * (csrc/ops/binary.cpp:102-104, csrc/ops/webgpu_ops.cpp:26-44). */
+int twg_add_relu_f32(float *out, const float *a, const float *b, const twg_iter_t *it,
+                     twg_stream_t stream);
+
+/* out = f(in), f from enum twg_unary_op.  Replaces unary_kernel<Op> and its WGSL
+ * (csrc/ops/unary.h:30-181, csrc/ops/unary.cpp:49-98), as reached from relu/
+ * gelu/silu(_out) (csrc/ops/activation_functions.cpp:27-114) and from the
+ * strided device-to-device branch of copy_ (csrc/ops/copy.cpp:123-134).  Uses
+ * it->stride[TWG_OUT] and it->stride[TWG_A]. */
+int twg_unary_f32(int op, float *out, const float *in, const twg_iter_t *it,
+                  twg_stream_t stream);
+/* Strided gather/scatter copy for 1-, 2-, 4- and 8-byte elements (bool masks
+ * are 1 byte).  Same role as TWG_UNARY_COPY for non-float dtypes, which the
+ * reference rejects (csrc/ops/unary.h:34). */
+int twg_copy_strided(void *out, const void *in, int32_t elem_size,
+                     const twg_iter_t *it, twg_stream_t stream);
+
+/* out[i] = (a[i] == b[i]) as a 0/1 byte, IEEE semantics (NaN != NaN, -0 == +0).
+ * Replaces the boxed CPU fallback registered for eq.Tensor / eq.Tensor_out
+ * (csrc/bindings.cpp:38-39). */
+int twg_eq_f32(uint8_t *out, const float *a, const float *b, const twg_iter_t *it,
+               twg_stream_t stream);
+/* out[i] = (a[i] != s).  Replaces the fallback for ne.Scalar / ne.Scalar_out
+ * (csrc/bindings.cpp:36-37). */
+int twg_ne_scalar_f32(uint8_t *out, const float *a, float s, const twg_iter_t *it,
+                      twg_stream_t stream);
+/* out[i] = a[i] & b[i] on 0/1 bytes.  Replaces the fallback for
+ * bitwise_and.Tensor / bitwise_and.Tensor_out (csrc/bindings.cpp:40-41) for bool
+ * (and uint8/int8) tensors. */
+int twg_and_u8(uint8_t *out, const uint8_t *a, const uint8_t *b, const twg_iter_t *it,
+               twg_stream_t stream);
+
+/* ---------------------------------------------------------- masked_select */
+
+/* Bytes of device scratch twg_masked_select_f32 needs for `numel` elements. */
+size_t twg_masked_select_scratch_bytes(int64_t numel);
+/* Single-pass ordered stream compaction: writes src[i] for every i with
+ * mask[i] != 0, in increasing logical index i, to out[0..K) and K to *d_count
+ * (device memory).  `out` must hold it->numel floats.  Replaces the boxed CPU
+ * fallback registered for masked_select (csrc/bindings.cpp:42).  `it` describes
+ * the broadcast logical shape: stride[TWG_A] addresses src, stride[TWG_B]
+ * addresses mask, stride[TWG_OUT] is ignored; dim 0 fastest, so logical index i
+ * is the row-major index of the broadcast shape reversed.  Asynchronous: read
+ * *d_count with twg_memcpy_d2h. */
+int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
+                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                          size_t scratch_bytes, twg_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TWG_H_ */

@@ -1,0 +1,109 @@
+"""Drive libtwg_hip.so through its C ABI from CPU tensors (GPU tests only).
+
+Operands are uploaded storage-and-all, so storage offsets and arbitrary strides
+are exercised exactly as the torch extension would pass them: the pointer handed
+to the kernel is storage base + offset, the strides go into twg_iter_t.
+"""
+import ctypes
+
+import torch
+
+import twg_capi as capi
+
+
+def _expanded(shape, *ts):
+    return [t.expand(shape) for t in ts]
+
+
+def _iter_for(shape, out, ops, sort_by_out=True):
+    """twg_iter_t over `shape` for out + up to two inputs.  With sort_by_out the
+    dimensions are ordered by ascending output stride (what at::TensorIterator does),
+    otherwise the logical order is kept (last dimension fastest)."""
+    nd = len(shape)
+    dims = list(range(nd - 1, -1, -1))  # fastest first
+    if sort_by_out and out is not None:
+        dims.sort(key=lambda d: (abs(out.stride(d)) if shape[d] != 1 else 0))
+    it = capi.Iter()
+    it.ndim = nd
+    numel = 1
+    for k, d in enumerate(dims):
+        it.shape[k] = shape[d]
+        numel *= shape[d]
+        it.stride[capi.OUT][k] = out.stride(d) if out is not None else 0
+        for slot, t in zip((capi.A, capi.B), ops):
+            it.stride[slot][k] = t.stride(d)
+    it.numel = numel
+    return it
+
+
+class Uploaded:
+    """A CPU tensor's whole storage on the device."""
+
+    def __init__(self, t):
+        self.t = t
+        self.buf, self.off = capi.upload_storage(t)
+
+    @property
+    def ptr(self):
+        return ctypes.c_void_p(self.buf.ptr + self.off)
+
+    def fetch(self):
+        """Download the storage and return a tensor with the original geometry."""
+        st_bytes = self.t.untyped_storage().nbytes()
+        raw = self.buf.download((st_bytes,), torch.uint8)
+        out = torch.empty(0, dtype=self.t.dtype)
+        out.set_(raw.untyped_storage(), self.t.storage_offset(), self.t.shape, self.t.stride())
+        return out
+
+
+def binary(fn_name, a, b, out=None, out_dtype=torch.float32, extra=(), sort_by_out=True):
+    """out = fn(a, b) on the GPU.  `out` may be a CPU tensor giving the output layout."""
+    L = capi.load()
+    shape = torch.broadcast_shapes(a.shape, b.shape)
+    if out is None:
+        out = torch.zeros(shape, dtype=out_dtype)
+    ae, be = _expanded(shape, a, b)
+    ua, ub, uo = Uploaded(a), Uploaded(b), Uploaded(out)
+    it = _iter_for(shape, out, (ae, be), sort_by_out)
+    rc = getattr(L, fn_name)(uo.ptr, ua.ptr, ub.ptr, *extra, ctypes.byref(it), None)
+    capi.check(rc)
+    return uo.fetch()
+
+
+def unary(fn_name, a, out=None, out_dtype=torch.float32, pre=(), extra=(), sort_by_out=True):
+    L = capi.load()
+    shape = tuple(a.shape)
+    if out is None:
+        out = torch.zeros(shape, dtype=out_dtype)
+    ua, uo = Uploaded(a), Uploaded(out)
+    it = _iter_for(shape, out, (a,), sort_by_out)
+    rc = getattr(L, fn_name)(*pre, uo.ptr, ua.ptr, *extra, ctypes.byref(it), None)
+    capi.check(rc)
+    return uo.fetch()
+
+
+def add(a, b, alpha=1.0, out=None):
+    return binary("twg_add_f32", a, b, out=out, extra=(ctypes.c_float(alpha),))
+
+
+def masked_select(x, mask, scratch_bytes=None):
+    """Returns (values, count) from twg_masked_select_f32."""
+    L = capi.load()
+    shape = torch.broadcast_shapes(x.shape, mask.shape)
+    xe, me = _expanded(shape, x, mask)
+    n = 1
+    for s in shape:
+        n *= s
+    ux, um = Uploaded(x), Uploaded(mask)
+    out = capi.DeviceBuffer(max(4 * n, 4))
+    cnt = capi.DeviceBuffer(8)
+    need = L.twg_masked_select_scratch_bytes(n)
+    scratch = capi.DeviceBuffer(need if scratch_bytes is None else max(scratch_bytes, 8))
+    it = _iter_for(shape, None, (xe, me), sort_by_out=False)
+    rc = L.twg_masked_select_f32(out.ptr, cnt.ptr, ux.ptr, um.ptr, ctypes.byref(it),
+                                 scratch.ptr, scratch.nbytes if scratch_bytes is None else scratch_bytes,
+                                 None)
+    capi.check(rc)
+    k = int(cnt.download((1,), torch.int64)[0])
+    vals = out.download((k,), torch.float32) if k else torch.empty(0, dtype=torch.float32)
+    return vals, k

@@ -1,0 +1,393 @@
+"""Parity of the HIP kernels, driven through the C ABI of libtwg_hip.so, against the
+CPU oracle (and ATen's CPU kernels where those are the reference's implementation).
+
+Bars: bit-exact for add (alpha = 1 and alpha != 1, same two roundings as the
+oracle), relu, copy, eq, ne, bitwise_and and masked_select (length and order);
+|got - ref| <= 2e-6*|ref| + 4 subnormal steps for gelu and silu against the
+closed form.
+"""
+import ctypes
+import itertools
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import capi_helpers as H
+import twg_workloads as W
+from oracle import oracle
+from util import (FLOOR, bit_equal, closed_form64, load_activation_golden, rel_err_ok, ulp_diff)
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ----------------------------------------------------------------- runtime
+
+def test_device_is_mi355x(twg):
+    name, cus, mem = twg.device_info()
+    _say(f"device: {name}, {cus} CUs, {mem / 2**30:.0f} GiB")
+    assert "gfx950" in name
+    assert cus >= 200
+
+
+def test_allocator_caches_and_handles_zero(twg):
+    L = twg.load()
+    p = ctypes.c_void_p(1)
+    twg.check(L.twg_malloc(ctypes.byref(p), 0))
+    assert not p.value  # zero bytes -> NULL, success
+    before = twg.mem_stats()
+    a = twg.DeviceBuffer(3 << 20)
+    addr = a.ptr
+    a.free()
+    b = twg.DeviceBuffer(3 << 20)
+    after = twg.mem_stats()
+    assert b.ptr == addr, "a freed block of the same size class is handed out again"
+    assert after["n_cache_hits"] >= before["n_cache_hits"] + 1
+    assert L.twg_free(ctypes.c_void_p(12345)) == twg.E_INVALID_ARG  # not ours
+    b.free()
+
+
+def test_copy_round_trip_fp32_and_bool(twg):
+    g = torch.Generator().manual_seed(1)
+    # 80 MiB crosses two 32 MiB staging chunks with a ragged tail
+    for t in (torch.randn((80 << 20) // 4 + 3, generator=g),
+              torch.rand(1000003, generator=g) < 0.5,
+              torch.randn(5, generator=g)):
+        buf = twg.to_device(t)
+        back = buf.download(t.shape, t.dtype)
+        assert bit_equal(back, t)
+    # device -> device and fill
+    t = torch.randn(4097, generator=g)
+    src = twg.to_device(t)
+    dst = twg.DeviceBuffer(t.numel() * 4 + 16)
+    L = twg.load()
+    twg.check(L.twg_fill_bytes(dst.ptr, 0xAB, dst.nbytes, None))
+    twg.check(L.twg_memcpy_d2d(dst.ptr + 8, src.ptr, t.numel() * 4, None))
+    raw = dst.download((dst.nbytes,), torch.uint8)
+    assert bool((raw[:8] == 0xAB).all()) and bool((raw[-8:] == 0xAB).all())
+    assert bit_equal(raw[8:-8].view(torch.float32), t)
+
+
+# --------------------------------------------------------------------- add
+
+def test_add_config1_contiguous(twg):
+    a, b = W.add_contiguous(1 << 20, seed=0)
+    got = H.add(a, b)
+    assert bit_equal(got, oracle.add(a, b))
+    assert bit_equal(got, a + b)
+
+
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 1023, 1024, 4095, 4096, 4097, 8191, 65536 + 13,
+                               (1 << 20) + 7])
+def test_add_ragged_sizes_and_misaligned(twg, n):
+    g = torch.Generator().manual_seed(n)
+    a = torch.randn(n + 3, generator=g)
+    b = torch.randn(n + 3, generator=g)
+    assert bit_equal(H.add(a[:n], b[:n]), a[:n] + b[:n])
+    # storage offsets 1 and 3: pointers no longer 16-byte aligned
+    out = torch.zeros(n + 2)[2:]
+    got = H.add(a[1:n + 1], b[3:n + 3], out=out)
+    assert bit_equal(got, a[1:n + 1] + b[3:n + 3])
+
+
+@pytest.mark.parametrize("alpha", [1.0, -1.0, 0.5, 1.7, 3.14159, 0.0])
+def test_add_alpha_matches_oracle_bits(twg, alpha):
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn(100003, generator=g)
+    b = torch.randn(100003, generator=g)
+    got = H.add(a, b, alpha=alpha)
+    assert bit_equal(got, oracle.add(a, b, alpha=alpha))
+    # and within 1 ulp of the exactly rounded value where nothing cancels
+    pa, pb = a.abs() + 0.5, b.abs() + 0.5
+    af = float(torch.tensor(abs(alpha), dtype=torch.float32))
+    ref = (pa.double() + af * pb.double()).float()
+    assert ulp_diff(H.add(pa, pb, alpha=abs(alpha)), ref) <= 1
+
+
+def test_add_special_values(twg):
+    s = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 1e-45, -1e-45, 3e38,
+                      1.17e-38])
+    a = s.repeat_interleave(s.numel())
+    b = s.repeat(s.numel())
+    assert ulp_diff(H.add(a, b), a + b) == 0
+    got, ref = H.add(a, b), a + b
+    ok = ~torch.isnan(ref)
+    assert torch.equal(torch.signbit(got[ok]), torch.signbit(ref[ok]))
+
+
+@pytest.mark.parametrize("rows,cols", [(256, 4096), (37, 1000), (5, 64), (3, 70001), (1, 513)])
+def test_add_row_and_column_bias(twg, rows, cols):
+    # config 3a shape family: [rows, cols] + [1, cols]; plus the column-bias and
+    # scalar-broadcast variants
+    a, bias, _ = W.broadcast_add_inputs(rows, cols, seed=rows)
+    assert bit_equal(H.add(a, bias), oracle.add(a, bias))
+    assert bit_equal(H.add(bias, a), bias + a)
+    col = bias[0, :rows].reshape(rows, 1).contiguous() if rows <= cols else a[:, :1].contiguous()
+    assert bit_equal(H.add(a, col), a + col)
+    assert bit_equal(H.add(a, a[0, 0].reshape(1, 1)), a + a[0, 0])
+    # outer-strided rows (every other row of a taller matrix)
+    tall = torch.cat([a, a * 2.0], 0)
+    assert bit_equal(H.add(tall[::2], bias), tall[::2] + bias)
+
+
+@pytest.mark.parametrize("rows,cols", [(256, 512), (100, 70), (64, 64), (65, 33), (16, 1000)])
+def test_add_transposed_operand(twg, rows, cols):
+    # config 3b shape family: A[rows, cols] viewed as (cols, rows) with strides
+    # (1, cols), plus a contiguous C[cols, rows].  TensorIterator gives the output
+    # the layout of the first input, so both output layouts are covered.
+    a, _, c = W.broadcast_add_inputs(rows, cols, seed=cols)
+    at = a.as_strided((cols, rows), (1, cols))
+    ref = oracle.add(at, c)
+    assert bit_equal(ref, at + c)
+    out_like_a = torch.zeros(rows, cols).t()  # strides (1, cols)
+    got = H.add(at, c, out=out_like_a)
+    assert bit_equal(got.contiguous(), ref)
+    got2 = H.add(at, c)  # contiguous output: now `at` is the transposed one
+    assert bit_equal(got2, ref)
+    got3 = H.add(c, at)
+    assert bit_equal(got3, ref)
+    # batched: leading dimension on top of the transposed pair
+    a3 = torch.stack([a, a + 1.0, a - 1.0])
+    at3 = a3.transpose(1, 2)
+    c3 = torch.stack([c, c * 2.0, c * 0.5])
+    assert bit_equal(H.add(at3, c3), at3 + c3)
+
+
+def test_add_generic_strides_bruteforce(twg):
+    g = torch.Generator().manual_seed(5)
+    sizes = [3, 4, 2, 5]
+    for perm in itertools.permutations(range(4)):
+        a = torch.randn(*sizes, generator=g).permute(*perm)
+        for bc in (0, 1, 6, 9, 15):
+            bshape = [1 if (bc >> d) & 1 else a.shape[d] for d in range(4)]
+            b = torch.randn(11 + int(torch.tensor(bshape).prod()), generator=g)[11:].view(*bshape)
+            ref = oracle.add(a, b, alpha=1.5)
+            assert bit_equal(H.add(a, b, alpha=1.5), ref)
+            # keep the logical dimension order too (no sorting by output stride)
+            assert bit_equal(H.binary("twg_add_f32", a, b, extra=(ctypes.c_float(1.5),),
+                                      sort_by_out=False), ref)
+    # 8 dimensions, negative stride via flip is not expressible in torch; use steps
+    a8 = torch.randn(2, 3, 2, 2, 3, 2, 2, 3, generator=g)[:, ::2, :, :, ::2]
+    b8 = torch.randn(2, 1, 2, 1, 1, 2, 1, 3, generator=g)
+    assert bit_equal(H.add(a8, b8), a8 + b8)
+
+
+def test_mul_and_fused_add_relu(twg):
+    g = torch.Generator().manual_seed(6)
+    a = torch.randn(70001, generator=g)
+    b = torch.randn(70001, generator=g)
+    assert bit_equal(H.binary("twg_mul_f32", a, b), oracle.mul(a, b))
+    assert bit_equal(H.binary("twg_add_relu_f32", a, b), oracle.add_relu(a, b))
+    # reference vectors: tests/ops/test_mul.py:30-39, tests/test_dev.py:8-18
+    assert torch.equal(H.binary("twg_mul_f32", torch.tensor([[1., 2.], [3., 4.]]),
+                                torch.tensor([10., 20.])),
+                       torch.tensor([[10., 40.], [30., 80.]]))
+    r = H.binary("twg_add_relu_f32", torch.tensor([-1.5, 2.7, 1.0, 2.0]),
+                 torch.tensor([-1.0, 0.9, 1.1, -2.1]))
+    assert torch.allclose(r, torch.tensor([0, 3.6, 2.1, 0]))
+    s = H.unary("twg_add_scalar_f32", a, extra=(ctypes.c_float(2.5), ctypes.c_float(0.5)))
+    assert bit_equal(s, oracle.add(a, torch.full_like(a, 2.5), alpha=0.5))
+    m = H.unary("twg_mul_scalar_f32", a, extra=(ctypes.c_float(2.0),))
+    assert bit_equal(m, a * 2.0)
+
+
+# ------------------------------------------------------------- activations
+
+def _unary(op, x, **kw):
+    return H.unary("twg_unary_f32", x, pre=(ctypes.c_int(op),), **kw)
+
+
+def test_relu_and_copy_bits(twg):
+    import twg_capi as C
+    x = W.activation_input(512, 1024, seed=1)
+    assert bit_equal(_unary(C.UNARY_RELU, x), oracle.relu(x))
+    assert bit_equal(_unary(C.UNARY_RELU, x), torch.relu(x))
+    assert bit_equal(_unary(C.UNARY_COPY, x), x)
+    s = torch.tensor([-0.0, 0.0, -1.0, 1.0, float("nan"), float("inf"), -float("inf"), -1e-45,
+                      1e-45, 1e-30, -1e-30])
+    got = _unary(C.UNARY_RELU, s)
+    assert ulp_diff(got, torch.relu(s)) == 0
+    assert torch.equal(torch.signbit(got), torch.signbit(torch.relu(s)))
+    # strided input, transposed output
+    xt = x.t()
+    assert bit_equal(_unary(C.UNARY_RELU, xt), torch.relu(xt))
+    assert bit_equal(_unary(C.UNARY_COPY, xt), xt.contiguous())
+    assert bit_equal(_unary(C.UNARY_COPY, x[::3, 5:900:7]), x[::3, 5:900:7].contiguous())
+
+
+@pytest.mark.parametrize("name", ["gelu_erf", "gelu_tanh", "silu"])
+def test_activation_golden_points(twg, name):
+    import twg_capi as C
+    op = {"gelu_erf": C.UNARY_GELU_ERF, "gelu_tanh": C.UNARY_GELU_TANH, "silu": C.UNARY_SILU}[name]
+    x, ref = load_activation_golden()
+    got = _unary(op, x)
+    ok, err, bound = rel_err_ok(got, ref[name], floor=FLOOR[name])
+    worst = int(torch.argmax(err / bound))
+    assert ok, f"{name}: x={x[worst].item()!r} got={got[worst].item()!r} ref={ref[name][worst].item()!r}"
+    # signed zeros and tiny inputs, as ATen's CPU kernels give them
+    z = torch.tensor([0.0, -0.0, 1e-30, -1e-30])
+    gz = _unary(op, z)
+    assert torch.equal(torch.signbit(gz), torch.tensor([False, True, False, True]))
+    assert bool((gz[:2] == 0).all())
+    assert rel_err_ok(gz[2:], torch.tensor([5.000000015855384e-31, -5.000000015855384e-31],
+                                            dtype=torch.float64))[0]
+    # NaN propagates, +inf -> +inf
+    s = _unary(op, torch.tensor([float("nan"), float("inf")]))
+    assert torch.isnan(s[0]) and s[1] == float("inf")
+
+
+@pytest.mark.parametrize("name", ["gelu_erf", "gelu_tanh", "silu"])
+def test_activation_config2_distribution(twg, name):
+    import twg_capi as C
+    op = {"gelu_erf": C.UNARY_GELU_ERF, "gelu_tanh": C.UNARY_GELU_TANH, "silu": C.UNARY_SILU}[name]
+    x = W.activation_input(1024, 2048, seed=1)  # N(0, 9) with forced 0 / +-1e-30 entries
+    # widen the tails beyond what 2^21 samples reach: 2^28 samples reach |x| ~ 18.7
+    x.view(-1)[:4096] = torch.linspace(-19.0, 19.0, 4096)
+    got = _unary(op, x)
+    ref64 = closed_form64(name, x)
+    ok, err, bound = rel_err_ok(got, ref64, floor=FLOOR[name])
+    worst = int(torch.argmax((err / bound).view(-1)))
+    assert ok, f"{name}: x={x.view(-1)[worst].item()!r} err={err.view(-1)[worst].item()}"
+    # the oracle (closed form rounded once) agrees to the same bar
+    ora = oracle.unary({"gelu_erf": oracle.GELU_ERF, "gelu_tanh": oracle.GELU_TANH,
+                        "silu": oracle.SILU}[name], x)
+    ok2, _, _ = rel_err_ok(got, ora.double(), floor=FLOOR[name])
+    assert ok2
+    # ATen's CPU kernels, at the tolerances the reference's own tests use
+    if name == "silu":
+        assert torch.allclose(got, F.silu(x), atol=1e-6)   # tests/ops/test_silu.py:13
+    else:
+        assert torch.allclose(got, F.gelu(x), atol=1e-3)   # tests/ops/test_gelu.py:14
+    if name == "gelu_erf":
+        assert torch.allclose(got, F.gelu(x), atol=2e-6, rtol=0)
+
+
+def test_activation_reference_vectors(twg):
+    import twg_capi as C
+    for data in ([-1.0, 0.0, 1.0, 2.0], [[0.5, -0.5], [1.5, -1.5]], [2.0], [0.0]):
+        t = torch.tensor(data, dtype=torch.float32)
+        assert torch.allclose(_unary(C.UNARY_GELU_ERF, t), F.gelu(t), atol=1e-3)
+        assert torch.allclose(_unary(C.UNARY_GELU_TANH, t), F.gelu(t), atol=1e-3)
+        assert torch.allclose(_unary(C.UNARY_SILU, t), F.silu(t), atol=1e-6)
+
+
+# ------------------------------------------------------------------- masks
+
+def test_mask_ops_config4(twg):
+    n = (1 << 20) + 5
+    p, q, z = W.mask_inputs(n, seed=3)
+    e = H.binary("twg_eq_f32", p, q, out_dtype=torch.bool)
+    assert e.dtype == torch.bool and bit_equal(e, oracle.eq(p, q)) and bit_equal(e, torch.eq(p, q))
+    assert 0.05 < e.float().mean().item() < 0.075  # about 1/16
+    nz = H.unary("twg_ne_scalar_f32", z, out_dtype=torch.bool, extra=(ctypes.c_float(0.0),))
+    assert bit_equal(nz, oracle.ne_scalar(z, 0.0)) and bit_equal(nz, z.ne(0.0))
+    assert 0.69 < nz.float().mean().item() < 0.71
+    both = H.binary("twg_and_u8", e, nz, out_dtype=torch.bool)
+    assert bit_equal(both, oracle.bitwise_and(e, nz)) and bit_equal(both, e & nz)
+    # bool bytes are exactly 0 or 1
+    assert set(both.view(torch.uint8).unique().tolist()) <= {0, 1}
+
+
+def test_compare_ieee_cases_and_layouts(twg):
+    a = torch.tensor([0.0, -0.0, float("nan"), float("nan"), float("inf"), 1.0, -0.0, 5.0])
+    b = torch.tensor([-0.0, 0.0, float("nan"), 1.0, float("inf"), float("nan"), -0.0, 5.0])
+    assert bit_equal(H.binary("twg_eq_f32", a, b, out_dtype=torch.bool), torch.eq(a, b))
+    for s in (0.0, -0.0, 5.0, float("nan")):
+        assert bit_equal(H.unary("twg_ne_scalar_f32", a, out_dtype=torch.bool,
+                                 extra=(ctypes.c_float(s),)), a.ne(s))
+    g = torch.Generator().manual_seed(8)
+    for n in (1, 3, 15, 16, 17, 4099):  # around the 4- and 16-element packs, misaligned
+        x = torch.randint(0, 3, (n + 1,), generator=g).float()
+        y = torch.randint(0, 3, (n + 1,), generator=g).float()
+        assert bit_equal(H.binary("twg_eq_f32", x[1:], y[:-1], out_dtype=torch.bool),
+                         torch.eq(x[1:], y[:-1]))
+        m1, m2 = x > 0, y > 1
+        assert bit_equal(H.binary("twg_and_u8", m1[1:], m2[:-1], out_dtype=torch.bool),
+                         m1[1:] & m2[:-1])
+    # broadcast and transposed compares
+    X = torch.randint(0, 4, (130, 70), generator=g).float()
+    row = torch.randint(0, 4, (1, 70), generator=g).float()
+    assert bit_equal(H.binary("twg_eq_f32", X, row, out_dtype=torch.bool), torch.eq(X, row))
+    Y = torch.randint(0, 4, (70, 130), generator=g).float()
+    assert bit_equal(H.binary("twg_eq_f32", X, Y.t(), out_dtype=torch.bool), torch.eq(X, Y.t()))
+    M = X > 1
+    assert bit_equal(H.binary("twg_and_u8", M, (Y > 0).t(), out_dtype=torch.bool), M & (Y > 0).t())
+    assert bit_equal(H.unary("twg_copy_strided", M.t(), out_dtype=torch.bool,
+                             extra=(ctypes.c_int32(1),)), M.t().contiguous())
+
+
+# ----------------------------------------------------------- masked_select
+
+@pytest.mark.parametrize("p", [0.0, 0.01, 0.5, 0.99, 1.0])
+@pytest.mark.parametrize("n", [1, 63, 64, 8191, 8192, 8193, (1 << 21) + 77])
+def test_masked_select_bernoulli(twg, n, p):
+    _say(f"masked_select n={n} p={p}")
+    x = W.select_source(n, seed=4)
+    m = W.bernoulli_mask(n, p, seed=n % 1000) if 0.0 < p < 1.0 else torch.full((n,), p == 1.0)
+    vals, k = H.masked_select(x, m)
+    ref = oracle.masked_select(x, m)
+    assert k == int(m.sum()) == ref.numel()
+    assert bit_equal(vals, ref)
+    assert bit_equal(vals, torch.masked_select(x, m))
+
+
+def test_masked_select_clustered_and_empty(twg):
+    n = (1 << 22) + 1234
+    x = W.select_source(n, seed=4)
+    m = W.clustered_mask(n, mean_run=4096, seed=6)
+    vals, k = H.masked_select(x, m)
+    assert k == int(m.sum())
+    assert bit_equal(vals, torch.masked_select(x, m))
+    # zero elements
+    vals0, k0 = H.masked_select(torch.empty(0), torch.empty(0, dtype=torch.bool))
+    assert k0 == 0 and vals0.numel() == 0
+
+
+def test_masked_select_misaligned_broadcast_strided(twg):
+    g = torch.Generator().manual_seed(9)
+    n = 50021
+    x = torch.rand(n + 3, generator=g)
+    m = torch.rand(n + 3, generator=g) < 0.4
+    # misaligned source / mask pointers (scalar variant of the kernel)
+    for xo, mo in ((1, 0), (0, 1), (3, 2)):
+        vals, k = H.masked_select(x[xo:xo + n], m[mo:mo + n])
+        assert bit_equal(vals, torch.masked_select(x[xo:xo + n], m[mo:mo + n]))
+    # reference known answers: row mask over a matrix, transposed self
+    xm = torch.tensor([[0., 1., 2.], [3., 4., 5.]])
+    rm = torch.tensor([True, False, True])
+    assert torch.equal(H.masked_select(xm, rm)[0], torch.tensor([0., 2., 3., 5.]))
+    xt = torch.arange(6.).view(3, 2).t()
+    assert torch.equal(H.masked_select(xt, rm)[0], torch.tensor([0., 4., 1., 5.]))
+    # larger broadcast / strided cases against the oracle and ATen
+    x3 = torch.rand(37, 1, 50, generator=g)
+    m3 = torch.rand(1, 11, 50, generator=g) < 0.5
+    v, _ = H.masked_select(x3, m3)
+    assert bit_equal(v, oracle.masked_select(x3, m3)) and bit_equal(v, torch.masked_select(x3, m3))
+    xs = torch.rand(300, 200, generator=g).t()[::2]
+    ms = (torch.rand(200, 300, generator=g) < 0.3)[::2]
+    v, _ = H.masked_select(xs, ms)
+    assert bit_equal(v, torch.masked_select(xs, ms))
+
+
+def test_masked_select_rejects_small_scratch(twg):
+    x = torch.rand(100000)
+    m = x > 0.5
+    with pytest.raises(H.capi.TwgError) as ei:
+        H.masked_select(x, m, scratch_bytes=64)
+    assert ei.value.code == H.capi.E_SCRATCH_SMALL
+
+
+def test_invalid_iter_is_rejected(twg):
+    L = twg.load()
+    it = twg.dense_iter(16)
+    it.numel = 17  # does not match the shape
+    buf = twg.DeviceBuffer(64)
+    assert L.twg_add_f32(buf.ptr, buf.ptr, buf.ptr, 1.0, ctypes.byref(it), None) == twg.E_INVALID_ARG
+    it = twg.dense_iter(16)
+    it.ndim = 9
+    assert L.twg_add_f32(buf.ptr, buf.ptr, buf.ptr, 1.0, ctypes.byref(it), None) == twg.E_INVALID_ARG
+    assert L.twg_unary_f32(99, buf.ptr, buf.ptr, ctypes.byref(twg.dense_iter(16)), None) == twg.E_INVALID_ARG

@@ -1,0 +1,644 @@
+// Elementwise half of libtwg_hip.so: add / mul / fused add+relu, the unary
+// activations, strided copy, eq / ne / and.  All HBM-bound: no MFMA.
+//
+// One templated family of four kernels serves every op:
+//   ew_contig  - every operand dense and equally ordered: 128-bit loads/stores,
+//                grid-stride over block-sized chunks.
+//   ew_rows    - inner dimension unit-stride (or broadcast) for every operand,
+//                outer dimensions arbitrary (row bias, column bias, slices).
+//   ew_tile    - an input whose unit stride lies along another dimension than
+//                the output's: 64x64 tiles staged through LDS so both sides of
+//                the transpose stay coalesced.
+//   ew_generic - anything else, one element per lane, div/mod index math with
+//                dimension 0 fastest.
+//
+// Replaces the two WGSL templates of the reference and their host drivers:
+//   csrc/ops/binary.cpp:23-104, csrc/ops/binary.h:29-215
+//   csrc/ops/unary.cpp:23-98,   csrc/ops/unary.h:30-181
+// and the CPU fallbacks for eq/ne/bitwise_and (csrc/bindings.cpp:36-41).
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "twg_internal.h"
+#include "twg_math.h"
+
+namespace twg {
+namespace {
+
+constexpr int kThreads = 256;  // 4 wavefronts of 64
+
+#ifndef TWG_EW_UNROLL
+#define TWG_EW_UNROLL 4
+#endif
+#ifndef TWG_EW_BLOCKS_PER_CU
+#define TWG_EW_BLOCKS_PER_CU 8
+#endif
+
+// ------------------------------------------------------------------ packs
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Pack {
+  T v[N];
+};
+
+template <typename P>
+__device__ __forceinline__ P load_pack(const P *p) {
+  return *p;
+}
+template <typename P>
+__device__ __forceinline__ void store_pack(P *p, const P &x) {
+  *p = x;
+}
+
+template <typename... Ts>
+struct MaxSize;
+template <typename T>
+struct MaxSize<T> {
+  static constexpr int value = (int)sizeof(T);
+};
+template <typename T, typename... Ts>
+struct MaxSize<T, Ts...> {
+  static constexpr int rest = MaxSize<Ts...>::value;
+  static constexpr int value = (int)sizeof(T) > rest ? (int)sizeof(T) : rest;
+};
+
+// ---------------------------------------------------------------- functors
+// Binary functors take (a, b); unary ones take (a) and are called with NIN == 1.
+
+struct AddOp {  // csrc/ops/binary.cpp:97: self + alpha * other, each op rounded
+  float alpha;
+  __device__ __forceinline__ float operator()(float a, float b) const {
+    return __fadd_rn(a, __fmul_rn(alpha, b));
+  }
+};
+struct AddScalarOp {
+  float alpha, s;
+  __device__ __forceinline__ float operator()(float a) const {
+    return __fadd_rn(a, __fmul_rn(alpha, s));
+  }
+};
+struct MulOp {  // csrc/ops/binary.cpp:100
+  __device__ __forceinline__ float operator()(float a, float b) const { return __fmul_rn(a, b); }
+};
+struct MulScalarOp {
+  float s;
+  __device__ __forceinline__ float operator()(float a) const { return __fmul_rn(a, s); }
+};
+struct AddReluOp {  // csrc/ops/binary.cpp:103
+  __device__ __forceinline__ float operator()(float a, float b) const {
+    return relu_f32(__fadd_rn(a, b));
+  }
+};
+template <typename T>
+struct CopyOp {  // csrc/ops/unary.cpp:89
+  __device__ __forceinline__ T operator()(T a) const { return a; }
+};
+struct ReluOp {  // csrc/ops/unary.cpp:91
+  __device__ __forceinline__ float operator()(float a) const { return relu_f32(a); }
+};
+struct GeluErfOp {
+  __device__ __forceinline__ float operator()(float a) const { return gelu_erf_f32(a); }
+};
+struct GeluTanhOp {  // csrc/ops/unary.cpp:94
+  __device__ __forceinline__ float operator()(float a) const { return gelu_tanh_f32(a); }
+};
+struct SiluOp {  // csrc/ops/unary.cpp:97
+  __device__ __forceinline__ float operator()(float a) const { return silu_f32(a); }
+};
+struct EqOp {
+  __device__ __forceinline__ uint8_t operator()(float a, float b) const { return a == b ? 1 : 0; }
+};
+struct NeScalarOp {
+  float s;
+  __device__ __forceinline__ uint8_t operator()(float a) const { return a != s ? 1 : 0; }
+};
+struct AndOp {
+  __device__ __forceinline__ uint8_t operator()(uint8_t a, uint8_t b) const { return a & b; }
+};
+
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+__device__ __forceinline__ TO apply(const Op &op, TA a, TB b) {
+  if constexpr (NIN == 2) {
+    return op(a, b);
+  } else {
+    return op(a);
+  }
+}
+
+// ------------------------------------------------------------- ew_contig
+
+template <int NIN, int VEC, int UNROLL, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_contig(TO *out, const TA *a, const TB *b,
+                                                      int64_t numel, Op op) {
+  using PO = Pack<TO, VEC>;
+  using PA = Pack<TA, VEC>;
+  using PB = Pack<TB, VEC>;
+  const int64_t nvec = numel / VEC;
+  constexpr int64_t kChunk = (int64_t)kThreads * UNROLL;  // packs per block step
+  const int64_t nchunk_full = nvec / kChunk;
+  const PA *pa = reinterpret_cast<const PA *>(a);
+  const PB *pb = reinterpret_cast<const PB *>(b);
+  PO *po = reinterpret_cast<PO *>(out);
+
+  for (int64_t c = blockIdx.x; c < nchunk_full; c += gridDim.x) {
+    const int64_t base = c * kChunk + threadIdx.x;
+    PA va[UNROLL];
+    PB vb[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) va[u] = load_pack(pa + base + u * kThreads);
+    if constexpr (NIN == 2) {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) vb[u] = load_pack(pb + base + u * kThreads);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      PO r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va[u].v[k], NIN == 2 ? vb[u].v[k] : TB());
+      store_pack(po + base + u * kThreads, r);
+    }
+  }
+  // Remainder packs (fewer than one chunk) and the last numel % VEC elements
+  // are swept by the first block.
+  if (blockIdx.x == 0) {
+    for (int64_t i = nchunk_full * kChunk + threadIdx.x; i < nvec; i += kThreads) {
+      PA va = load_pack(pa + i);
+      PB vb;
+      if constexpr (NIN == 2) vb = load_pack(pb + i);
+      PO r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
+      store_pack(po + i, r);
+    }
+    if constexpr (VEC > 1) {
+      const int64_t i = nvec * VEC + threadIdx.x;
+      if (i < numel) out[i] = apply<NIN, Op, TO, TA, TB>(op, a[i], NIN == 2 ? b[i] : TB());
+    }
+  }
+}
+
+// --------------------------------------------------------------- ew_rows
+
+struct RowGeom {
+  int64_t len;               // extent of dimension 0
+  uint32_t chunks_per_row;   // blocks along one row
+  int32_t nouter;            // remaining dimensions
+  int64_t oshape[TWG_MAX_DIMS - 1];
+  int64_t ostride[3][TWG_MAX_DIMS - 1];
+};
+
+template <int NIN, int VEC, int UNROLL, bool A_BC, bool B_BC, typename Op, typename TO,
+          typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
+                                                    Op op) {
+  using PO = Pack<TO, VEC>;
+  using PA = Pack<TA, VEC>;
+  using PB = Pack<TB, VEC>;
+  uint32_t row = blockIdx.x / g.chunks_per_row;
+  const uint32_t chunk = blockIdx.x - row * g.chunks_per_row;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  {
+    int64_t r = row;
+    for (int d = 0; d < g.nouter; ++d) {
+      const int64_t q = r / g.oshape[d];
+      const int64_t c = r - q * g.oshape[d];
+      r = q;
+      off_o += c * g.ostride[0][d];
+      off_a += c * g.ostride[1][d];
+      if constexpr (NIN == 2) off_b += c * g.ostride[2][d];
+    }
+  }
+  TO *orow = out + off_o;
+  const TA *arow = a + off_a;
+  const TB *brow = (NIN == 2) ? b + off_b : nullptr;
+  TA abc = TA();
+  TB bbc = TB();
+  if constexpr (A_BC) abc = arow[0];
+  if constexpr (NIN == 2 && B_BC) bbc = brow[0];
+
+  const int64_t e0 = (int64_t)chunk * (kThreads * VEC * UNROLL) + (int64_t)threadIdx.x * VEC;
+  PA va[UNROLL];
+  PB vb[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t e = e0 + (int64_t)u * kThreads * VEC;
+    if (e < g.len) {
+      if constexpr (!A_BC) va[u] = load_pack(reinterpret_cast<const PA *>(arow + e));
+      if constexpr (NIN == 2 && !B_BC) vb[u] = load_pack(reinterpret_cast<const PB *>(brow + e));
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t e = e0 + (int64_t)u * kThreads * VEC;
+    if (e < g.len) {
+      PO r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const TA x = A_BC ? abc : va[u].v[k];
+        const TB y = (NIN == 2) ? (B_BC ? bbc : vb[u].v[k]) : TB();
+        r.v[k] = apply<NIN, Op, TO, TA, TB>(op, x, y);
+      }
+      store_pack(reinterpret_cast<PO *>(orow + e), r);
+    }
+  }
+}
+
+// --------------------------------------------------------------- ew_tile
+
+constexpr int kTile = 64;
+
+struct TileGeom {
+  int64_t n0, nt;          // extents of dimension 0 and of the transposed dimension t
+  int64_t s0[3], st[3];    // strides along those two, per operand
+  uint32_t tiles0, tilest; // tile counts
+  int32_t nbatch;          // remaining dimensions
+  int64_t bshape[TWG_MAX_DIMS - 2];
+  int64_t bstride[3][TWG_MAX_DIMS - 2];
+};
+
+// Lane x (0..63) runs along dimension 0, the 4 wavefronts and 16 steps cover 64
+// positions along t.  An operand marked *_T has its unit stride along t: it is
+// read with lane x along t instead, parked in LDS and picked up transposed.
+template <int NIN, bool A_T, bool B_T, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_tile(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                    Op op) {
+  __shared__ TA sa[A_T ? kTile : 1][kTile + 1];
+  __shared__ TB sb[(NIN == 2 && B_T) ? kTile : 1][kTile + 1];
+
+  uint32_t bid = blockIdx.x;
+  const uint32_t t0i = bid % g.tiles0;
+  bid /= g.tiles0;
+  const uint32_t tti = bid % g.tilest;
+  int64_t r = bid / g.tilest;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const int64_t q = r / g.bshape[d];
+    const int64_t c = r - q * g.bshape[d];
+    r = q;
+    off_o += c * g.bstride[0][d];
+    off_a += c * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
+  }
+  const int x = threadIdx.x & 63;
+  const int y = threadIdx.x >> 6;  // 0..3
+  const int64_t base0 = (int64_t)t0i * kTile;
+  const int64_t baset = (int64_t)tti * kTile;
+
+  if constexpr (A_T) {
+    const int64_t tt = baset + x;
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) {
+      const int64_t d0 = base0 + y + 4 * k;
+      if (tt < g.nt && d0 < g.n0) sa[y + 4 * k][x] = a[off_a + d0 * g.s0[1] + tt * g.st[1]];
+    }
+  }
+  if constexpr (NIN == 2 && B_T) {
+    const int64_t tt = baset + x;
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) {
+      const int64_t d0 = base0 + y + 4 * k;
+      if (tt < g.nt && d0 < g.n0) sb[y + 4 * k][x] = b[off_b + d0 * g.s0[2] + tt * g.st[2]];
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+
+  const int64_t d0 = base0 + x;
+  if (d0 >= g.n0) return;
+#pragma unroll 4
+  for (int k = 0; k < kTile / 4; ++k) {
+    const int tl = y + 4 * k;
+    const int64_t tt = baset + tl;
+    if (tt >= g.nt) break;
+    TA va;
+    TB vb = TB();
+    if constexpr (A_T) {
+      va = sa[x][tl];
+    } else {
+      va = a[off_a + d0 * g.s0[1] + tt * g.st[1]];
+    }
+    if constexpr (NIN == 2) {
+      if constexpr (B_T) {
+        vb = sb[x][tl];
+      } else {
+        vb = b[off_b + d0 * g.s0[2] + tt * g.st[2]];
+      }
+    }
+    out[off_o + d0 * g.s0[0] + tt * g.st[0]] = apply<NIN, Op, TO, TA, TB>(op, va, vb);
+  }
+}
+
+// ------------------------------------------------------------ ew_generic
+
+template <typename UIdx, typename SIdx>
+struct GenGeom {
+  int32_t ndim;
+  UIdx numel;
+  UIdx shape[TWG_MAX_DIMS];
+  SIdx stride[3][TWG_MAX_DIMS];
+};
+
+template <int NIN, typename UIdx, typename SIdx, typename Op, typename TO, typename TA,
+          typename TB>
+__global__ __launch_bounds__(kThreads) void ew_generic(TO *out, const TA *a, const TB *b,
+                                                       GenGeom<UIdx, SIdx> g, Op op) {
+  const UIdx step = (UIdx)gridDim.x * kThreads;
+  for (UIdx i = (UIdx)blockIdx.x * kThreads + threadIdx.x; i < g.numel; i += step) {
+    UIdx rem = i;
+    SIdx oo = 0, oa = 0, ob = 0;
+    for (int d = 0; d < g.ndim; ++d) {  // dimension 0 is the fastest-moving one
+      const UIdx q = rem / g.shape[d];
+      const SIdx c = (SIdx)(rem - q * g.shape[d]);
+      rem = q;
+      oo += c * g.stride[0][d];
+      oa += c * g.stride[1][d];
+      if constexpr (NIN == 2) ob += c * g.stride[2][d];
+    }
+    out[oo] = apply<NIN, Op, TO, TA, TB>(op, a[oa], NIN == 2 ? b[ob] : TB());
+  }
+}
+
+// -------------------------------------------------------------- dispatch
+
+inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+
+inline unsigned capped_grid(int64_t blocks_wanted) {
+  int64_t cap = (int64_t)compute_units() * TWG_EW_BLOCKS_PER_CU;
+  if (cap < 1) cap = 1;
+  if (blocks_wanted < 1) blocks_wanted = 1;
+  return (unsigned)(blocks_wanted < cap ? blocks_wanted : cap);
+}
+
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_generic(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  bool fits32 = g.numel <= INT32_MAX;
+  for (int o = 0; o <= NIN && fits32; ++o) {
+    int64_t span = 0;
+    for (int d = 0; d < g.ndim; ++d) {
+      int64_t st = g.stride[o][d] < 0 ? -g.stride[o][d] : g.stride[o][d];
+      span += st * (g.shape[d] - 1);
+      if (span > INT32_MAX) { fits32 = false; break; }
+    }
+  }
+  const unsigned grid = capped_grid((g.numel + kThreads - 1) / kThreads);
+  if (fits32) {
+    GenGeom<uint32_t, int32_t> gg{};
+    gg.ndim = g.ndim;
+    gg.numel = (uint32_t)g.numel;
+    for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+      gg.shape[d] = (uint32_t)g.shape[d];
+      for (int o = 0; o < 3; ++o) gg.stride[o][d] = (int32_t)g.stride[o][d];
+    }
+    ew_generic<NIN, uint32_t, int32_t, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, gg, op);
+  } else {
+    GenGeom<uint64_t, int64_t> gg{};
+    gg.ndim = g.ndim;
+    gg.numel = (uint64_t)g.numel;
+    for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+      gg.shape[d] = (uint64_t)g.shape[d];
+      for (int o = 0; o < 3; ++o) gg.stride[o][d] = g.stride[o][d];
+    }
+    ew_generic<NIN, uint64_t, int64_t, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, gg, op);
+  }
+  return (int)hipGetLastError();
+}
+
+template <int NIN, int VEC, bool A_BC, bool B_BC, typename Op, typename TO, typename TA,
+          typename TB>
+int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  constexpr int U = TWG_EW_UNROLL;
+  RowGeom rg{};
+  rg.len = g.shape[0];
+  const int64_t per_block = (int64_t)kThreads * VEC * U;
+  const int64_t cpr = (rg.len + per_block - 1) / per_block;
+  const int64_t rows = g.numel / rg.len;
+  if (cpr * rows > INT32_MAX || cpr > UINT32_MAX) return TWG_E_UNSUPPORTED;
+  rg.chunks_per_row = (uint32_t)cpr;
+  rg.nouter = g.ndim - 1;
+  for (int d = 1; d < g.ndim; ++d) {
+    rg.oshape[d - 1] = g.shape[d];
+    for (int o = 0; o < 3; ++o) rg.ostride[o][d - 1] = g.stride[o][d];
+  }
+  ew_rows<NIN, VEC, U, A_BC, B_BC, Op, TO, TA, TB>
+      <<<(unsigned)(cpr * rows), kThreads, 0, s>>>(out, a, b, rg, op);
+  return (int)hipGetLastError();
+}
+
+template <int NIN, bool A_BC, bool B_BC, typename Op, typename TO, typename TA, typename TB>
+int launch_rows(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  constexpr int VEC = 16 / MaxSize<TO, TA, TB>::value;
+  // Packs need every row start aligned for every non-broadcast operand.
+  bool vec_ok = (g.shape[0] % VEC == 0) && aligned_to(out, sizeof(TO) * VEC) &&
+                (A_BC || aligned_to(a, sizeof(TA) * VEC)) &&
+                (NIN == 1 || B_BC || aligned_to(b, sizeof(TB) * VEC));
+  for (int d = 1; d < g.ndim && vec_ok; ++d) {
+    vec_ok = vec_ok && (g.stride[0][d] % VEC == 0) && (A_BC || g.stride[1][d] % VEC == 0) &&
+             (NIN == 1 || B_BC || g.stride[2][d] % VEC == 0);
+  }
+  if (vec_ok) return launch_rows_v<NIN, VEC, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
+  return launch_rows_v<NIN, 1, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
+}
+
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
+                hipStream_t s) {
+  TileGeom tg{};
+  tg.n0 = g.shape[0];
+  tg.nt = g.shape[t];
+  for (int o = 0; o < 3; ++o) {
+    tg.s0[o] = g.stride[o][0];
+    tg.st[o] = g.stride[o][t];
+  }
+  const int64_t tiles0 = (tg.n0 + kTile - 1) / kTile;
+  const int64_t tilest = (tg.nt + kTile - 1) / kTile;
+  int64_t batch = 1;
+  tg.nbatch = 0;
+  for (int d = 1; d < g.ndim; ++d) {
+    if (d == t) continue;
+    tg.bshape[tg.nbatch] = g.shape[d];
+    for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+    tg.nbatch++;
+    batch *= g.shape[d];
+  }
+  if (tiles0 > UINT32_MAX || tilest > UINT32_MAX) return TWG_E_UNSUPPORTED;
+  if (tiles0 * tilest > INT32_MAX || tiles0 * tilest * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+  tg.tiles0 = (uint32_t)tiles0;
+  tg.tilest = (uint32_t)tilest;
+  const unsigned grid = (unsigned)(tiles0 * tilest * batch);
+  if (a_t && b_t) {
+    if constexpr (NIN == 2)
+      ew_tile<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  } else if (a_t) {
+    ew_tile<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  } else {
+    if constexpr (NIN == 2)
+      ew_tile<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  }
+  return (int)hipGetLastError();
+}
+
+// Pick the kernel for a canonical geometry.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, twg_stream_t stream) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  Geom g;
+  if ((rc = canonicalize(it, NIN + 1, &g))) return rc;
+  if (g.numel == 0) return 0;
+  if (!out || !a || (NIN == 2 && !b)) return TWG_E_INVALID_ARG;
+  hipStream_t s = resolve_stream(stream);
+  constexpr int VEC = 16 / MaxSize<TO, TA, TB>::value;
+  constexpr int U = TWG_EW_UNROLL;
+
+  // (i) every operand dense in the same order
+  bool dense = g.ndim <= 1;
+  if (dense && g.ndim == 1)
+    dense = g.stride[0][0] == 1 && g.stride[1][0] == 1 && (NIN == 1 || g.stride[2][0] == 1);
+  if (dense) {
+    const bool vec_ok = aligned_to(out, sizeof(TO) * VEC) && aligned_to(a, sizeof(TA) * VEC) &&
+                        (NIN == 1 || aligned_to(b, sizeof(TB) * VEC));
+    if (vec_ok) {
+      const int64_t chunks = g.numel / ((int64_t)VEC * kThreads * U);
+      ew_contig<NIN, VEC, U, Op, TO, TA, TB>
+          <<<capped_grid(chunks), kThreads, 0, s>>>(out, a, b, g.numel, op);
+    } else {
+      const int64_t chunks = g.numel / ((int64_t)kThreads * U);
+      ew_contig<NIN, 1, U, Op, TO, TA, TB>
+          <<<capped_grid(chunks), kThreads, 0, s>>>(out, a, b, g.numel, op);
+    }
+    return (int)hipGetLastError();
+  }
+
+  if (g.ndim >= 1 && g.stride[0][0] == 1) {
+    const int64_t sa0 = g.stride[1][0];
+    const int64_t sb0 = (NIN == 2) ? g.stride[2][0] : 1;
+    // (ii) inner dimension unit-stride or broadcast for every input
+    if ((sa0 == 0 || sa0 == 1) && (sb0 == 0 || sb0 == 1) && !(sa0 == 0 && sb0 == 0) &&
+        g.shape[0] >= 64) {
+      int r;
+      if (sa0 == 0) {
+        r = launch_rows<NIN, true, false, Op, TO, TA, TB>(out, a, b, g, op, s);
+      } else if (NIN == 2 && sb0 == 0) {
+        r = launch_rows<NIN, false, true, Op, TO, TA, TB>(out, a, b, g, op, s);
+      } else {
+        r = launch_rows<NIN, false, false, Op, TO, TA, TB>(out, a, b, g, op, s);
+      }
+      if (r != TWG_E_UNSUPPORTED) return r;
+    }
+    // (iii) an input with its unit stride along another dimension
+    if (g.ndim >= 2 && g.shape[0] >= 16) {
+      int t = -1;
+      for (int d = 1; d < g.ndim && t < 0; ++d) {
+        if (g.shape[d] < 16) continue;
+        if ((sa0 != 0 && sa0 != 1 && g.stride[1][d] == 1) ||
+            (NIN == 2 && sb0 != 0 && sb0 != 1 && g.stride[2][d] == 1))
+          t = d;
+      }
+      if (t > 0) {
+        const bool a_t = sa0 != 0 && sa0 != 1 && g.stride[1][t] == 1;
+        const bool b_t = NIN == 2 && sb0 != 0 && sb0 != 1 && g.stride[2][t] == 1;
+        int r = launch_tile<NIN, Op, TO, TA, TB>(out, a, b, g, t, a_t, b_t, op, s);
+        if (r != TWG_E_UNSUPPORTED) return r;
+      }
+    }
+  }
+  // (iv) anything else
+  return launch_generic<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
+}
+
+}  // namespace
+}  // namespace twg
+
+using namespace twg;
+
+extern "C" {
+
+int twg_add_f32(float *out, const float *a, const float *b, float alpha, const twg_iter_t *it,
+                twg_stream_t stream) {
+  return launch_ew<2, AddOp, float, float, float>(out, a, b, it, AddOp{alpha}, stream);
+}
+
+int twg_add_scalar_f32(float *out, const float *a, float s, float alpha, const twg_iter_t *it,
+                       twg_stream_t stream) {
+  return launch_ew<1, AddScalarOp, float, float, float>(out, a, nullptr, it, AddScalarOp{alpha, s},
+                                                        stream);
+}
+
+int twg_mul_f32(float *out, const float *a, const float *b, const twg_iter_t *it,
+                twg_stream_t stream) {
+  return launch_ew<2, MulOp, float, float, float>(out, a, b, it, MulOp{}, stream);
+}
+
+int twg_mul_scalar_f32(float *out, const float *a, float s, const twg_iter_t *it,
+                       twg_stream_t stream) {
+  return launch_ew<1, MulScalarOp, float, float, float>(out, a, nullptr, it, MulScalarOp{s},
+                                                        stream);
+}
+
+int twg_add_relu_f32(float *out, const float *a, const float *b, const twg_iter_t *it,
+                     twg_stream_t stream) {
+  return launch_ew<2, AddReluOp, float, float, float>(out, a, b, it, AddReluOp{}, stream);
+}
+
+int twg_unary_f32(int op, float *out, const float *in, const twg_iter_t *it, twg_stream_t stream) {
+  const float *nb = nullptr;
+  switch (op) {
+    case TWG_UNARY_COPY:
+      return launch_ew<1, CopyOp<float>, float, float, float>(out, in, nb, it, CopyOp<float>{},
+                                                              stream);
+    case TWG_UNARY_RELU:
+      return launch_ew<1, ReluOp, float, float, float>(out, in, nb, it, ReluOp{}, stream);
+    case TWG_UNARY_GELU_ERF:
+      return launch_ew<1, GeluErfOp, float, float, float>(out, in, nb, it, GeluErfOp{}, stream);
+    case TWG_UNARY_GELU_TANH:
+      return launch_ew<1, GeluTanhOp, float, float, float>(out, in, nb, it, GeluTanhOp{}, stream);
+    case TWG_UNARY_SILU:
+      return launch_ew<1, SiluOp, float, float, float>(out, in, nb, it, SiluOp{}, stream);
+    default:
+      return TWG_E_INVALID_ARG;
+  }
+}
+
+int twg_copy_strided(void *out, const void *in, int32_t elem_size, const twg_iter_t *it,
+                     twg_stream_t stream) {
+  switch (elem_size) {
+    case 1:
+      return launch_ew<1, CopyOp<uint8_t>, uint8_t, uint8_t, uint8_t>(
+          (uint8_t *)out, (const uint8_t *)in, (const uint8_t *)nullptr, it, CopyOp<uint8_t>{},
+          stream);
+    case 2:
+      return launch_ew<1, CopyOp<uint16_t>, uint16_t, uint16_t, uint16_t>(
+          (uint16_t *)out, (const uint16_t *)in, (const uint16_t *)nullptr, it,
+          CopyOp<uint16_t>{}, stream);
+    case 4:
+      return launch_ew<1, CopyOp<uint32_t>, uint32_t, uint32_t, uint32_t>(
+          (uint32_t *)out, (const uint32_t *)in, (const uint32_t *)nullptr, it,
+          CopyOp<uint32_t>{}, stream);
+    case 8:
+      return launch_ew<1, CopyOp<uint64_t>, uint64_t, uint64_t, uint64_t>(
+          (uint64_t *)out, (const uint64_t *)in, (const uint64_t *)nullptr, it,
+          CopyOp<uint64_t>{}, stream);
+    default:
+      return TWG_E_UNSUPPORTED;
+  }
+}
+
+int twg_eq_f32(uint8_t *out, const float *a, const float *b, const twg_iter_t *it,
+               twg_stream_t stream) {
+  return launch_ew<2, EqOp, uint8_t, float, float>(out, a, b, it, EqOp{}, stream);
+}
+
+int twg_ne_scalar_f32(uint8_t *out, const float *a, float s, const twg_iter_t *it,
+                      twg_stream_t stream) {
+  return launch_ew<1, NeScalarOp, uint8_t, float, float>(out, a, nullptr, it, NeScalarOp{s},
+                                                         stream);
+}
+
+int twg_and_u8(uint8_t *out, const uint8_t *a, const uint8_t *b, const twg_iter_t *it,
+               twg_stream_t stream) {
+  return launch_ew<2, AndOp, uint8_t, uint8_t, uint8_t>(out, a, b, it, AndOp{}, stream);
+}
+
+}  // extern "C"

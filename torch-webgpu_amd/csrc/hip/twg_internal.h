@@ -1,0 +1,39 @@
+// Internal helpers shared by the .hip translation units of libtwg_hip.so.
+// Nothing here is part of the C ABI (that is include/twg.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "twg.h"
+
+namespace twg {
+
+// Resolve the stream argument of an entry point: NULL selects the library stream.
+hipStream_t resolve_stream(twg_stream_t s);
+// Number of compute units of the bound device (256 on MI355X); 0 before init.
+int compute_units();
+// Lazily run twg_init(); returns its status.
+int ensure_init();
+
+#define TWG_HIP_TRY(expr)                      \
+  do {                                         \
+    hipError_t twg_e_ = (expr);                \
+    if (twg_e_ != hipSuccess) return (int)twg_e_; \
+  } while (0)
+
+// Canonical iteration geometry derived from a caller's twg_iter_t: size-1
+// dimensions dropped and adjacent dimensions merged wherever every used operand
+// stays linear across them.  Dimension 0 remains the fastest one.
+struct Geom {
+  int ndim;
+  int64_t numel;
+  int64_t shape[TWG_MAX_DIMS];
+  int64_t stride[3][TWG_MAX_DIMS];
+};
+
+// Validate `it` and build the canonical geometry for the first `nops` operand
+// slots (2 = out + a, 3 = out + a + b).  Returns 0 or TWG_E_INVALID_ARG.
+int canonicalize(const twg_iter_t *it, int nops, Geom *g);
+
+}  // namespace twg

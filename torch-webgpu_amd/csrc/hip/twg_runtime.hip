@@ -1,0 +1,457 @@
+// Runtime half of libtwg_hip.so: device/stream bring-up, the caching device
+// allocator, pinned-staged host<->device copies and event timing.
+//
+// Takes over what the reference does through Google Dawn:
+//   csrc/core/webgpu_context.cpp:9-68     instance/adapter/device/queue singleton
+//   csrc/core/webgpu_allocator.cpp:10-55  one wgpu::Buffer per tensor storage
+//   csrc/ops/copy.cpp:12-62,74-122        WriteBuffer / CopyBufferToBuffer / MapAsync
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "twg_internal.h"
+
+namespace twg {
+namespace {
+
+struct Runtime {
+  std::once_flag once;
+  std::atomic<int> status{-1000};  // -1000 = not attempted yet
+  hipStream_t stream = nullptr;
+  int cus = 0;
+  hipDeviceProp_t prop;
+};
+
+Runtime &rt() {
+  static Runtime r;
+  return r;
+}
+
+void do_init() {
+  Runtime &r = rt();
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n < 1) {
+    r.status = (e != hipSuccess) ? (int)e : (int)hipErrorNoDevice;
+    return;
+  }
+  if ((e = hipSetDevice(0)) != hipSuccess) { r.status = (int)e; return; }
+  if ((e = hipGetDeviceProperties(&r.prop, 0)) != hipSuccess) { r.status = (int)e; return; }
+  r.cus = r.prop.multiProcessorCount;
+  // One in-order stream at the default priority plays the part of the Dawn queue.
+  if ((e = hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking)) != hipSuccess) {
+    r.status = (int)e;
+    return;
+  }
+  r.status = 0;
+}
+
+// ------------------------------------------------------------ allocator
+
+constexpr size_t kSmallGranule = 512;
+constexpr size_t kLargeGranule = size_t(2) << 20;
+constexpr size_t kLargeThreshold = size_t(1) << 20;
+
+size_t round_size(size_t n) {
+  if (n < kLargeThreshold) return (n + kSmallGranule - 1) / kSmallGranule * kSmallGranule;
+  return (n + kLargeGranule - 1) / kLargeGranule * kLargeGranule;
+}
+
+struct Pool {
+  std::mutex mu;
+  std::multimap<size_t, void *> free_blocks;     // rounded size -> block
+  std::unordered_map<void *, size_t> live;       // block -> rounded size
+  twg_mem_stats_t st{};
+};
+
+Pool &pool() {
+  static Pool *p = new Pool;  // leaked on purpose: tensors may outlive static destructors
+  return *p;
+}
+
+int release_cached_locked(Pool &p) {
+  int rc = 0;
+  for (auto &kv : p.free_blocks) {
+    hipError_t e = hipFree(kv.second);
+    if (e != hipSuccess) rc = (int)e;
+  }
+  p.free_blocks.clear();
+  p.st.bytes_cached = 0;
+  return rc;
+}
+
+// ------------------------------------------------------------ staging ring
+
+constexpr size_t kStageBytes = size_t(32) << 20;
+constexpr int kStageSlots = 2;
+
+struct Staging {
+  std::mutex mu;
+  bool ready = false;
+  void *buf[kStageSlots] = {nullptr, nullptr};
+  hipEvent_t ev[kStageSlots] = {nullptr, nullptr};
+  bool busy[kStageSlots] = {false, false};
+};
+
+Staging &staging() {
+  static Staging *s = new Staging;
+  return *s;
+}
+
+int staging_prepare_locked(Staging &s) {
+  if (s.ready) return 0;
+  for (int i = 0; i < kStageSlots; ++i) {
+    TWG_HIP_TRY(hipHostMalloc(&s.buf[i], kStageBytes, hipHostMallocDefault));
+    TWG_HIP_TRY(hipEventCreateWithFlags(&s.ev[i], hipEventDisableTiming));
+  }
+  s.ready = true;
+  return 0;
+}
+
+__global__ void fill_bytes_kernel(uint8_t *dst, uint8_t v, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) dst[i] = v;
+}
+
+__global__ void fill_words_kernel(uint4 *dst, uint32_t w, size_t nvec) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t step = (size_t)gridDim.x * blockDim.x;
+  uint4 v = make_uint4(w, w, w, w);
+  for (; i < nvec; i += step) dst[i] = v;
+}
+
+}  // namespace
+
+int ensure_init() {
+  Runtime &r = rt();
+  std::call_once(r.once, do_init);
+  return r.status.load();
+}
+
+hipStream_t resolve_stream(twg_stream_t s) {
+  return s ? reinterpret_cast<hipStream_t>(s) : rt().stream;
+}
+
+int compute_units() { return rt().cus; }
+
+int canonicalize(const twg_iter_t *it, int nops, Geom *g) {
+  if (!it || !g) return TWG_E_INVALID_ARG;
+  if (it->ndim < 0 || it->ndim > TWG_MAX_DIMS) return TWG_E_INVALID_ARG;
+  int64_t numel = 1;
+  for (int d = 0; d < it->ndim; ++d) {
+    if (it->shape[d] < 0) return TWG_E_INVALID_ARG;
+    if (it->shape[d] != 0 && numel > INT64_MAX / it->shape[d]) return TWG_E_INVALID_ARG;
+    numel *= it->shape[d];
+  }
+  if (numel != it->numel) return TWG_E_INVALID_ARG;
+  g->numel = numel;
+  g->ndim = 0;
+  for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+    g->shape[d] = 1;
+    for (int o = 0; o < 3; ++o) g->stride[o][d] = 0;
+  }
+  if (numel == 0) return 0;
+  for (int d = 0; d < it->ndim; ++d) {
+    if (it->shape[d] == 1) continue;  // contributes nothing to any offset
+    int k = g->ndim;
+    bool merged = false;
+    if (k > 0) {
+      bool linear = true;
+      for (int o = 0; o < nops; ++o)
+        linear = linear && (it->stride[o][d] == g->stride[o][k - 1] * g->shape[k - 1]);
+      if (linear) {
+        g->shape[k - 1] *= it->shape[d];
+        merged = true;
+      }
+    }
+    if (!merged) {
+      g->shape[k] = it->shape[d];
+      for (int o = 0; o < nops; ++o) g->stride[o][k] = it->stride[o][d];
+      g->ndim = k + 1;
+    }
+  }
+  return 0;
+}
+
+}  // namespace twg
+
+using namespace twg;
+
+extern "C" {
+
+int twg_init(void) { return ensure_init(); }
+
+int twg_is_initialized(void) { return rt().status.load() == 0 ? 1 : 0; }
+
+const char *twg_error_string(int code) {
+  switch (code) {
+    case 0: return "success";
+    case TWG_E_INVALID_ARG: return "twg: invalid argument";
+    case TWG_E_UNSUPPORTED: return "twg: unsupported request";
+    case TWG_E_SCRATCH_SMALL: return "twg: scratch buffer too small";
+    case TWG_E_OVERLAP: return "twg: overlapping ranges";
+    case -1000: return "twg: not initialised";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "twg: unknown error";
+}
+
+int twg_device_info(char *name, size_t name_cap, int32_t *compute_units, int64_t *total_mem_bytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  Runtime &r = rt();
+  if (name && name_cap) {
+    std::snprintf(name, name_cap, "%s (%s)", r.prop.name, r.prop.gcnArchName);
+  }
+  if (compute_units) *compute_units = r.cus;
+  if (total_mem_bytes) *total_mem_bytes = (int64_t)r.prop.totalGlobalMem;
+  return 0;
+}
+
+twg_stream_t twg_default_stream(void) {
+  if (ensure_init()) return nullptr;
+  return reinterpret_cast<twg_stream_t>(rt().stream);
+}
+
+int twg_stream_sync(twg_stream_t stream) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  TWG_HIP_TRY(hipStreamSynchronize(resolve_stream(stream)));
+  return 0;
+}
+
+int twg_device_sync(void) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  TWG_HIP_TRY(hipDeviceSynchronize());
+  return 0;
+}
+
+int twg_event_create(twg_event_t *ev) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (!ev) return TWG_E_INVALID_ARG;
+  hipEvent_t e;
+  TWG_HIP_TRY(hipEventCreate(&e));
+  *ev = reinterpret_cast<twg_event_t>(e);
+  return 0;
+}
+
+int twg_event_destroy(twg_event_t ev) {
+  if (!ev) return 0;
+  TWG_HIP_TRY(hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)));
+  return 0;
+}
+
+int twg_event_record(twg_event_t ev, twg_stream_t stream) {
+  if (!ev) return TWG_E_INVALID_ARG;
+  TWG_HIP_TRY(hipEventRecord(reinterpret_cast<hipEvent_t>(ev), resolve_stream(stream)));
+  return 0;
+}
+
+int twg_event_sync(twg_event_t ev) {
+  if (!ev) return TWG_E_INVALID_ARG;
+  TWG_HIP_TRY(hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev)));
+  return 0;
+}
+
+int twg_event_elapsed_ms(float *ms, twg_event_t start, twg_event_t stop) {
+  if (!ms || !start || !stop) return TWG_E_INVALID_ARG;
+  TWG_HIP_TRY(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start),
+                                  reinterpret_cast<hipEvent_t>(stop)));
+  return 0;
+}
+
+// ---------------------------------------------------------------- allocator
+
+int twg_malloc(void **p, size_t n) {
+  if (!p) return TWG_E_INVALID_ARG;
+  *p = nullptr;
+  if (n == 0) return 0;
+  int rc = ensure_init();
+  if (rc) return rc;
+  const size_t want = round_size(n);
+  Pool &pl = pool();
+  std::lock_guard<std::mutex> lk(pl.mu);
+  pl.st.n_allocs++;
+  // Best fit: the smallest cached block that is large enough, as long as it
+  // wastes at most a quarter of itself (small blocks must match exactly).
+  auto it = pl.free_blocks.lower_bound(want);
+  if (it != pl.free_blocks.end()) {
+    size_t have = it->first;
+    bool ok = (have == want) || (want >= kLargeThreshold && have - want <= have / 4);
+    if (ok) {
+      *p = it->second;
+      pl.free_blocks.erase(it);
+      pl.live.emplace(*p, have);
+      pl.st.bytes_cached -= (int64_t)have;
+      pl.st.bytes_in_use += (int64_t)have;
+      pl.st.n_cache_hits++;
+      return 0;
+    }
+  }
+  void *d = nullptr;
+  hipError_t e = hipMalloc(&d, want);
+  if (e == hipErrorOutOfMemory) {
+    (void)hipGetLastError();
+    // Everything cached was freed by the caller; make sure queued work that
+    // still uses those blocks has drained before handing them to the driver.
+    (void)hipStreamSynchronize(rt().stream);
+    release_cached_locked(pl);
+    e = hipMalloc(&d, want);
+  }
+  if (e != hipSuccess) return (int)e;
+  pl.st.n_device_mallocs++;
+  pl.live.emplace(d, want);
+  pl.st.bytes_in_use += (int64_t)want;
+  *p = d;
+  return 0;
+}
+
+int twg_free(void *p) {
+  if (!p) return 0;
+  Pool &pl = pool();
+  std::lock_guard<std::mutex> lk(pl.mu);
+  auto it = pl.live.find(p);
+  if (it == pl.live.end()) return TWG_E_INVALID_ARG;
+  size_t sz = it->second;
+  pl.live.erase(it);
+  pl.free_blocks.emplace(sz, p);
+  pl.st.bytes_in_use -= (int64_t)sz;
+  pl.st.bytes_cached += (int64_t)sz;
+  return 0;
+}
+
+int twg_empty_cache(void) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  // Work queued before the matching twg_free calls may still touch the blocks.
+  TWG_HIP_TRY(hipStreamSynchronize(rt().stream));
+  Pool &pl = pool();
+  std::lock_guard<std::mutex> lk(pl.mu);
+  return release_cached_locked(pl);
+}
+
+int twg_mem_stats(twg_mem_stats_t *out) {
+  if (!out) return TWG_E_INVALID_ARG;
+  Pool &pl = pool();
+  std::lock_guard<std::mutex> lk(pl.mu);
+  *out = pl.st;
+  return 0;
+}
+
+// ------------------------------------------------------------------ copies
+
+int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_stream_t stream) {
+  if (nbytes == 0) return 0;
+  if (!dst_dev || !src_host) return TWG_E_INVALID_ARG;
+  int rc = ensure_init();
+  if (rc) return rc;
+  hipStream_t s = resolve_stream(stream);
+  Staging &st = staging();
+  std::lock_guard<std::mutex> lk(st.mu);
+  if ((rc = staging_prepare_locked(st))) return rc;
+  const char *src = static_cast<const char *>(src_host);
+  char *dst = static_cast<char *>(dst_dev);
+  size_t done = 0;
+  int slot = 0;
+  while (done < nbytes) {
+    size_t chunk = nbytes - done < kStageBytes ? nbytes - done : kStageBytes;
+    if (st.busy[slot]) {  // the DMA that last read this slot must have finished
+      TWG_HIP_TRY(hipEventSynchronize(st.ev[slot]));
+      st.busy[slot] = false;
+    }
+    std::memcpy(st.buf[slot], src + done, chunk);
+    TWG_HIP_TRY(hipMemcpyAsync(dst + done, st.buf[slot], chunk, hipMemcpyHostToDevice, s));
+    TWG_HIP_TRY(hipEventRecord(st.ev[slot], s));
+    st.busy[slot] = true;
+    done += chunk;
+    slot = (slot + 1) % kStageSlots;
+  }
+  return 0;  // the caller's host range is free again; the device side is stream ordered
+}
+
+int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_stream_t stream) {
+  if (nbytes == 0) return 0;
+  if (!dst_host || !src_dev) return TWG_E_INVALID_ARG;
+  int rc = ensure_init();
+  if (rc) return rc;
+  hipStream_t s = resolve_stream(stream);
+  Staging &st = staging();
+  std::lock_guard<std::mutex> lk(st.mu);
+  if ((rc = staging_prepare_locked(st))) return rc;
+  for (int i = 0; i < kStageSlots; ++i) {
+    if (st.busy[i]) {
+      TWG_HIP_TRY(hipEventSynchronize(st.ev[i]));
+      st.busy[i] = false;
+    }
+  }
+  char *dst = static_cast<char *>(dst_host);
+  const char *src = static_cast<const char *>(src_dev);
+  const size_t nchunks = (nbytes + kStageBytes - 1) / kStageBytes;
+  auto chunk_len = [&](size_t c) {
+    size_t off = c * kStageBytes;
+    return nbytes - off < kStageBytes ? nbytes - off : kStageBytes;
+  };
+  // Keep one DMA in flight while the CPU drains the previous chunk.
+  TWG_HIP_TRY(hipMemcpyAsync(st.buf[0], src, chunk_len(0), hipMemcpyDeviceToHost, s));
+  TWG_HIP_TRY(hipEventRecord(st.ev[0], s));
+  for (size_t c = 0; c < nchunks; ++c) {
+    int slot = (int)(c % kStageSlots);
+    if (c + 1 < nchunks) {
+      int nslot = (int)((c + 1) % kStageSlots);
+      TWG_HIP_TRY(hipMemcpyAsync(st.buf[nslot], src + (c + 1) * kStageBytes, chunk_len(c + 1),
+                                 hipMemcpyDeviceToHost, s));
+      TWG_HIP_TRY(hipEventRecord(st.ev[nslot], s));
+    }
+    TWG_HIP_TRY(hipEventSynchronize(st.ev[slot]));
+    std::memcpy(dst + c * kStageBytes, st.buf[slot], chunk_len(c));
+  }
+  return 0;
+}
+
+int twg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes, twg_stream_t stream) {
+  if (nbytes == 0) return 0;
+  if (!dst_dev || !src_dev) return TWG_E_INVALID_ARG;
+  int rc = ensure_init();
+  if (rc) return rc;
+  TWG_HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, nbytes, hipMemcpyDeviceToDevice,
+                             resolve_stream(stream)));
+  return 0;
+}
+
+int twg_fill_bytes(void *dst_dev, int value, size_t nbytes, twg_stream_t stream) {
+  if (nbytes == 0) return 0;
+  if (!dst_dev) return TWG_E_INVALID_ARG;
+  int rc = ensure_init();
+  if (rc) return rc;
+  hipStream_t s = resolve_stream(stream);
+  uint8_t v = (uint8_t)value;
+  uint8_t *p = static_cast<uint8_t *>(dst_dev);
+  // unaligned head, 16-byte body, tail
+  size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15;
+  if (head > nbytes) head = nbytes;
+  size_t body = (nbytes - head) / 16;
+  size_t tail = nbytes - head - body * 16;
+  if (head) fill_bytes_kernel<<<1, 64, 0, s>>>(p, v, head);
+  if (body) {
+    uint32_t w = 0x01010101u * v;
+    size_t blocks = (body + 255) / 256;
+    size_t cap = (size_t)compute_units() * 16;
+    if (blocks > cap) blocks = cap;
+    fill_words_kernel<<<(unsigned)blocks, 256, 0, s>>>(reinterpret_cast<uint4 *>(p + head), w, body);
+  }
+  if (tail) fill_bytes_kernel<<<1, 64, 0, s>>>(p + head + body * 16, v, tail);
+  TWG_HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"
