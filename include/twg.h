@@ -67,7 +67,8 @@ enum twg_unary_op {
   TWG_UNARY_RELU = 1,      /* csrc/ops/unary.cpp:90-92 */
   TWG_UNARY_GELU_ERF = 2,  /* aten gelu(approximate='none') */
   TWG_UNARY_GELU_TANH = 3, /* csrc/ops/unary.cpp:93-95 */
-  TWG_UNARY_SILU = 4       /* csrc/ops/unary.cpp:96-98 */
+  TWG_UNARY_SILU = 4,      /* csrc/ops/unary.cpp:96-98 */
+  TWG_UNARY_ABS = 5        /* |x|; a boxed CPU fallback in the reference, csrc/bindings.cpp:35 */
 };
 
 /* ---------------------------------------------------------------- runtime */

@@ -19,7 +19,7 @@ _LIB_PATH = os.path.join(_HERE, "libtwg_oracle.so")
 MAX_DIMS = 8
 
 ADD, MUL, ADD_RELU = 0, 1, 2
-COPY, RELU, GELU_ERF, GELU_TANH, SILU = 0, 1, 2, 3, 4
+COPY, RELU, GELU_ERF, GELU_TANH, SILU, ABS = 0, 1, 2, 3, 4, 5
 
 
 class Params(ctypes.Structure):

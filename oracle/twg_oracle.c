@@ -23,7 +23,7 @@
  *                                     on non-cancelling inputs
  *   oracle_binary_f32 (Mul, AddRelu)  pinned: tests/ops/test_mul.py:6-63 vectors,
  *                                     tests/test_dev.py:8-18 vector, ATen CPU
- *   oracle_unary_f32 (Copy, ReLU)     pinned: ATen CPU bit-exact incl. -0.0, NaN
+ *   oracle_unary_f32 (Copy, ReLU, Abs) pinned: ATen CPU bit-exact incl. -0.0, NaN
  *   oracle_unary_f32 (GeluErf, Silu,  pinned: 50-digit closed forms in
  *                     GeluTanh)       tests/golden/activations_mp.json; the
  *                                     reference's tests/ops/test_gelu.py and
@@ -58,7 +58,7 @@ typedef struct oracle_params {
 
 enum { ORACLE_ADD = 0, ORACLE_MUL = 1, ORACLE_ADD_RELU = 2 };                /* binary.h:18-23 */
 enum { ORACLE_COPY = 0, ORACLE_RELU = 1, ORACLE_GELU_ERF = 2, ORACLE_GELU_TANH = 3,
-       ORACLE_SILU = 4 };                                                     /* unary.h:20-26  */
+       ORACLE_SILU = 4, ORACLE_ABS = 5 };                                     /* unary.h:20-26  */
 
 /* csrc/ops/binary.cpp:58-79 (identical in unary.cpp:52-71): the linear id is
  * decomposed with dimension ndim-1 varying fastest, then dotted with each
@@ -121,6 +121,8 @@ static float oracle_unary_op(int op, float xf) {
       double u = 0.79788456080286535588 * (x + 0.044715 * x * x * x);
       return (float)(x / (1.0 + exp(-2.0 * u)));
     }
+    case ORACLE_ABS: /* aten::abs, a CPU fallback in the reference (csrc/bindings.cpp:35) */
+      return fabsf(xf);
     default: /* ORACLE_SILU */
       return (float)(x / (1.0 + exp(-x)));
   }

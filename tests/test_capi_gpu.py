@@ -207,6 +207,7 @@ def test_relu_and_copy_bits(twg):
     assert bit_equal(_unary(C.UNARY_RELU, x), oracle.relu(x))
     assert bit_equal(_unary(C.UNARY_RELU, x), torch.relu(x))
     assert bit_equal(_unary(C.UNARY_COPY, x), x)
+    assert bit_equal(_unary(C.UNARY_ABS, x), oracle.unary(oracle.ABS, x))
     s = torch.tensor([-0.0, 0.0, -1.0, 1.0, float("nan"), float("inf"), -float("inf"), -1e-45,
                       1e-45, 1e-30, -1e-30])
     got = _unary(C.UNARY_RELU, s)

@@ -108,6 +108,8 @@ def test_relu_matches_aten_bits():
     r = torch.randn(5000, generator=g)
     assert bit_equal(oracle.relu(r), torch.relu(r))
     assert bit_equal(oracle.unary(oracle.COPY, r), r)
+    assert bit_equal(oracle.unary(oracle.ABS, r), r.abs())
+    assert bit_equal(oracle.unary(oracle.ABS, x), x.abs())
 
 
 def test_activations_against_50_digit_closed_forms():

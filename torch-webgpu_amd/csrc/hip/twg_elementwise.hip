@@ -106,6 +106,9 @@ struct GeluTanhOp {  // csrc/ops/unary.cpp:94
 struct SiluOp {  // csrc/ops/unary.cpp:97
   __device__ __forceinline__ float operator()(float a) const { return silu_f32(a); }
 };
+struct AbsOp {
+  __device__ __forceinline__ float operator()(float a) const { return fabsf(a); }
+};
 struct EqOp {
   __device__ __forceinline__ uint8_t operator()(float a, float b) const { return a == b ? 1 : 0; }
 };
@@ -596,6 +599,8 @@ int twg_unary_f32(int op, float *out, const float *in, const twg_iter_t *it, twg
       return launch_ew<1, GeluTanhOp, float, float, float>(out, in, nb, it, GeluTanhOp{}, stream);
     case TWG_UNARY_SILU:
       return launch_ew<1, SiluOp, float, float, float>(out, in, nb, it, SiluOp{}, stream);
+    case TWG_UNARY_ABS:
+      return launch_ew<1, AbsOp, float, float, float>(out, in, nb, it, AbsOp{}, stream);
     default:
       return TWG_E_INVALID_ARG;
   }

@@ -1,0 +1,369 @@
+// Operator registrations for the "webgpu" device: TensorIterator -> twg_iter_t ->
+// the HIP kernels of libtwg_hip.so.
+//
+// Registration sites mirrored from the reference:
+//   csrc/ops/arithmetic.cpp:393-399        add.out (mul.out is commented out there)
+//   csrc/ops/activation_functions.cpp:116-126   relu / gelu / silu and their out forms
+//   csrc/bindings.cpp:32-43                abs, ne.Scalar, eq.Tensor, bitwise_and.Tensor,
+//                                          masked_select: boxed CPU fallbacks there,
+//                                          device kernels here
+//   csrc/ops/webgpu_ops.cpp:47-66          webgpu:: custom ops and the autograd fallthrough
+#include <ATen/ExpandUtils.h>
+#include <ATen/native/TensorIterator.h>
+#include <torch/library.h>
+
+#include "twg_torch.h"
+
+namespace torch_webgpu {
+namespace ops {
+namespace {
+
+void require_float(const at::TensorIteratorBase &iter, const char *op) {
+  // csrc/ops/binary.h:33, csrc/ops/unary.h:34
+  TORCH_CHECK(iter.common_dtype() == at::kFloat, "webgpu ", op,
+              ": only float32 tensors are supported, got ", iter.common_dtype());
+}
+
+void require_on_device(const at::Tensor &t, const char *op) {
+  TORCH_CHECK(is_webgpu(t), "webgpu ", op, ": expected a webgpu tensor, got ", t.device());
+}
+
+float *fptr(at::TensorIteratorBase &iter, int k) { return static_cast<float *>(iter.data_ptr(k)); }
+
+enum class Bin { Add, Mul, AddRelu };
+
+// csrc/ops/arithmetic.cpp:24-43 and csrc/ops/binary.h:29-215
+void binary_f32(Bin op, const at::Tensor &self, const at::Tensor &other, float alpha,
+                at::Tensor &out, const char *name) {
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(out);
+  config.add_const_input(self);
+  config.add_const_input(other);
+  config.promote_inputs_to_common_dtype(true);
+  config.cast_common_dtype_to_outputs(true);
+  config.allow_cpu_scalars(true);
+  auto iter = config.build();
+  require_float(iter, name);
+  // A 0-dim CPU operand (a Python number) is read on the host and passed by
+  // value.  The reference lets it into the iterator and then reinterprets its
+  // storage as a device buffer (csrc/ops/arithmetic.cpp:37, csrc/ops/binary.h:95).
+  const bool s1 = iter.is_cpu_scalar(1), s2 = iter.is_cpu_scalar(2);
+  // Off the CPU the iterator leaves operand dtypes alone; a host scalar of another
+  // dtype (torch.mul(t, 2)) is converted when it is read, device operands must be fp32.
+  TORCH_CHECK(iter.dtype(0) == at::kFloat && (s1 || iter.dtype(1) == at::kFloat) &&
+                  (s2 || iter.dtype(2) == at::kFloat),
+              "webgpu ", name, ": mixed dtypes are not supported");
+  if (iter.numel() == 0) return;
+  TORCH_CHECK(!(s1 && s2), "webgpu ", name, ": at least one operand must live on the device");
+  if (s2 || (s1 && (op == Bin::Mul || (op == Bin::Add && alpha == 1.0f)))) {
+    const int which = s2 ? 2 : 1;  // commutative cases let the scalar sit on either side
+    const float s = iter.scalar_value<float>(which);
+    iter.remove_operand(which);
+    twg_iter_t it;
+    fill_iter(iter, &it);
+    if (op == Bin::Add)
+      TWG_CHECK(twg_add_scalar_f32(fptr(iter, 0), fptr(iter, 1), s, alpha, &it, nullptr));
+    else if (op == Bin::Mul)
+      TWG_CHECK(twg_mul_scalar_f32(fptr(iter, 0), fptr(iter, 1), s, &it, nullptr));
+    else
+      TORCH_CHECK(false, "webgpu ", name, ": scalar operand not supported");
+    return;
+  }
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  at::Tensor staged;  // scalar on the left of a non-commutative form: one element, stride 0
+  const float *a = fptr(iter, 1);
+  if (s1) {
+    staged = at::empty({1}, out.options().dtype(at::kFloat));
+    const float v = iter.scalar_value<float>(1);
+    TWG_CHECK(twg_memcpy_h2d(staged.data_ptr(), &v, sizeof(float), nullptr));
+    a = staged.const_data_ptr<float>();
+    for (int d = 0; d < it.ndim; ++d) it.stride[TWG_A][d] = 0;
+  }
+  switch (op) {
+    case Bin::Add:
+      TWG_CHECK(twg_add_f32(fptr(iter, 0), a, fptr(iter, 2), alpha, &it, nullptr));
+      break;
+    case Bin::Mul:
+      TWG_CHECK(twg_mul_f32(fptr(iter, 0), a, fptr(iter, 2), &it, nullptr));
+      break;
+    case Bin::AddRelu:
+      TWG_CHECK(twg_add_relu_f32(fptr(iter, 0), a, fptr(iter, 2), &it, nullptr));
+      break;
+  }
+}
+
+// csrc/ops/activation_functions.cpp:27-114 and csrc/ops/unary.h:30-181
+void unary_f32(int op, const at::Tensor &self, at::Tensor &out, const char *name) {
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(out);
+  config.add_const_input(self);
+  config.check_all_same_dtype(true);
+  auto iter = config.build();
+  require_float(iter, name);
+  if (iter.numel() == 0) return;
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  TWG_CHECK(twg_unary_f32(op, fptr(iter, 0), fptr(iter, 1), &it, nullptr));
+}
+
+int gelu_op(c10::string_view approximate, const char *name) {
+  if (approximate == "none") return TWG_UNARY_GELU_ERF;
+  if (approximate == "tanh") return TWG_UNARY_GELU_TANH;  // the reference's only formula
+  TORCH_CHECK(false, "webgpu ", name, ": approximate must be 'none' or 'tanh', got '",
+              std::string(approximate), "'");
+}
+
+at::Tensor new_like(const at::Tensor &self) {
+  return at::empty_like(self, self.options(), c10::MemoryFormat::Preserve);
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ add / mul
+
+at::Tensor &add_out(const at::Tensor &self, const at::Tensor &other, const at::Scalar &alpha,
+                    at::Tensor &out) {
+  binary_f32(Bin::Add, self, other, alpha.to<float>(), out, "add");
+  return out;
+}
+
+at::Tensor &mul_out(const at::Tensor &self, const at::Tensor &other, at::Tensor &out) {
+  binary_f32(Bin::Mul, self, other, 1.0f, out, "mul");
+  return out;
+}
+
+// ---------------------------------------------------------------- activations
+
+at::Tensor relu(const at::Tensor &self) {
+  at::Tensor out = new_like(self);
+  unary_f32(TWG_UNARY_RELU, self, out, "relu");
+  return out;
+}
+at::Tensor &relu_(at::Tensor &self) {
+  unary_f32(TWG_UNARY_RELU, self, self, "relu_");
+  return self;
+}
+at::Tensor &relu_out(const at::Tensor &self, at::Tensor &out) {
+  unary_f32(TWG_UNARY_RELU, self, out, "relu");
+  return out;
+}
+at::Tensor gelu(const at::Tensor &self, c10::string_view approximate) {
+  const int op = gelu_op(approximate, "gelu");
+  at::Tensor out = new_like(self);
+  unary_f32(op, self, out, "gelu");
+  return out;
+}
+at::Tensor &gelu_out(const at::Tensor &self, c10::string_view approximate, at::Tensor &out) {
+  unary_f32(gelu_op(approximate, "gelu"), self, out, "gelu");
+  return out;
+}
+at::Tensor silu(const at::Tensor &self) {
+  at::Tensor out = new_like(self);
+  unary_f32(TWG_UNARY_SILU, self, out, "silu");
+  return out;
+}
+at::Tensor &silu_out(const at::Tensor &self, at::Tensor &out) {
+  unary_f32(TWG_UNARY_SILU, self, out, "silu");
+  return out;
+}
+at::Tensor &abs_out(const at::Tensor &self, at::Tensor &out) {
+  unary_f32(TWG_UNARY_ABS, self, out, "abs");
+  return out;
+}
+
+// ----------------------------------------------------------------- bool masks
+
+at::Tensor &eq_tensor_out(const at::Tensor &self, const at::Tensor &other, at::Tensor &out) {
+  require_on_device(self, "eq");
+  require_on_device(other, "eq");
+  TORCH_CHECK(self.scalar_type() == at::kFloat && other.scalar_type() == at::kFloat,
+              "webgpu eq: only float32 operands are supported, got ", self.scalar_type(), " and ",
+              other.scalar_type());
+  TORCH_CHECK(out.scalar_type() == at::kBool, "webgpu eq: the output must be a bool tensor");
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(out);
+  config.add_const_input(self);
+  config.add_const_input(other);
+  config.check_all_same_dtype(false);
+  auto iter = config.build();
+  if (iter.numel() == 0) return out;
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  TWG_CHECK(twg_eq_f32(static_cast<uint8_t *>(iter.data_ptr(0)), fptr(iter, 1), fptr(iter, 2), &it,
+                       nullptr));
+  return out;
+}
+
+at::Tensor eq_tensor(const at::Tensor &self, const at::Tensor &other) {
+  require_on_device(self, "eq");
+  at::Tensor out = at::empty({0}, self.options().dtype(at::kBool));
+  return eq_tensor_out(self, other, out);
+}
+
+at::Tensor &ne_scalar_out(const at::Tensor &self, const at::Scalar &other, at::Tensor &out) {
+  require_on_device(self, "ne");
+  TORCH_CHECK(self.scalar_type() == at::kFloat, "webgpu ne: only float32 is supported, got ",
+              self.scalar_type());
+  TORCH_CHECK(out.scalar_type() == at::kBool, "webgpu ne: the output must be a bool tensor");
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(out);
+  config.add_const_input(self);
+  config.check_all_same_dtype(false);
+  auto iter = config.build();
+  if (iter.numel() == 0) return out;
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  // ATen compares in the tensor's dtype: the scalar is rounded to float32 first
+  TWG_CHECK(twg_ne_scalar_f32(static_cast<uint8_t *>(iter.data_ptr(0)), fptr(iter, 1),
+                              other.to<float>(), &it, nullptr));
+  return out;
+}
+
+at::Tensor ne_scalar(const at::Tensor &self, const at::Scalar &other) {
+  at::Tensor out = at::empty({0}, self.options().dtype(at::kBool));
+  return ne_scalar_out(self, other, out);
+}
+
+at::Tensor &bitwise_and_out(const at::Tensor &self, const at::Tensor &other, at::Tensor &out) {
+  require_on_device(self, "bitwise_and");
+  require_on_device(other, "bitwise_and");
+  const auto dt = self.scalar_type();
+  TORCH_CHECK(dt == other.scalar_type() && dt == out.scalar_type() &&
+                  (dt == at::kBool || dt == at::kByte || dt == at::kChar),
+              "webgpu bitwise_and: operands and output must share a 1-byte dtype (bool, uint8, int8), got ",
+              self.scalar_type(), ", ", other.scalar_type(), " -> ", out.scalar_type());
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(out);
+  config.add_const_input(self);
+  config.add_const_input(other);
+  auto iter = config.build();
+  if (iter.numel() == 0) return out;
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  TWG_CHECK(twg_and_u8(static_cast<uint8_t *>(iter.data_ptr(0)),
+                       static_cast<const uint8_t *>(iter.data_ptr(1)),
+                       static_cast<const uint8_t *>(iter.data_ptr(2)), &it, nullptr));
+  return out;
+}
+
+at::Tensor bitwise_and(const at::Tensor &self, const at::Tensor &other) {
+  at::Tensor out = at::empty({0}, self.options());
+  return bitwise_and_out(self, other, out);
+}
+
+// -------------------------------------------------------------- masked_select
+
+at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
+  // Error text and semantics of ATen's CPU kernel, which is what the reference runs
+  // (csrc/bindings.cpp:42).
+  TORCH_CHECK(mask.scalar_type() == at::kBool, "masked_select: expected BoolTensor for mask");
+  require_on_device(self, "masked_select");
+  TORCH_CHECK(self.scalar_type() == at::kFloat, "webgpu masked_select: only float32 sources are supported, got ",
+              self.scalar_type());
+  at::Tensor m = is_webgpu(mask) ? mask : mask.to(self.device());
+  auto expanded = at::expand_outplace(m, self);
+  const at::Tensor &me = *std::get<0>(expanded);
+  const at::Tensor &se = *std::get<1>(expanded);
+  const int64_t n = se.numel();
+  if (n == 0) return at::empty({0}, self.options());
+
+  twg_iter_t it;
+  fill_iter_logical(se, me, &it);
+  const size_t scratch_bytes = twg_masked_select_scratch_bytes(n);
+  // one allocation: [count (8 B, padded to 256) | scratch]
+  at::Tensor work = at::empty({(int64_t)(scratch_bytes + 256)}, self.options().dtype(at::kByte));
+  auto *count_dev = static_cast<int64_t *>(work.data_ptr());
+  void *scratch = static_cast<char *>(work.data_ptr()) + 256;
+  at::Tensor out = at::empty({n}, self.options());
+  TWG_CHECK(twg_masked_select_f32(out.data_ptr<float>(), count_dev, se.const_data_ptr<float>(),
+                                  static_cast<const uint8_t *>(me.const_data_ptr()), &it, scratch,
+                                  scratch_bytes, nullptr));
+  int64_t k = 0;  // the output shape depends on the data: this read is the op's one sync point
+  TWG_CHECK(twg_memcpy_d2h(&k, count_dev, sizeof(k), nullptr));
+  TORCH_CHECK(k >= 0 && k <= n, "webgpu masked_select: implausible count ", k);
+  if (k * 4 <= n) {  // do not pin a source-sized block under a small result
+    at::Tensor exact = at::empty({k}, self.options());
+    if (k > 0)
+      TWG_CHECK(twg_memcpy_d2d(exact.data_ptr(), out.const_data_ptr(), (size_t)k * sizeof(float), nullptr));
+    return exact;
+  }
+  out.unsafeGetTensorImpl()->set_sizes_contiguous({k});
+  return out;
+}
+
+at::Tensor &masked_select_out(const at::Tensor &self, const at::Tensor &mask, at::Tensor &out) {
+  at::Tensor r = ops::masked_select(self, mask);
+  out.resize_(r.sizes());
+  out.copy_(r);
+  return out;
+}
+
+// ------------------------------------------------- webgpu:: ops (webgpu_ops.cpp)
+
+at::Tensor create_buffer(c10::IntArrayRef size, c10::IntArrayRef stride,
+                         std::optional<at::ScalarType> dtype_opt) {
+  return at::empty_strided(size, stride,
+                           at::TensorOptions().dtype(dtype_opt).device(c10::Device(c10::kPrivateUse1, 0)));
+}
+
+at::Tensor write_buffer(at::Tensor &self, const at::Tensor &src) {
+  self.copy_(src);
+  return self;
+}
+
+at::Tensor fused_add_relu(const at::Tensor &self, const at::Tensor &other) {
+  require_on_device(self, "fused_add_relu");
+  at::Tensor out = at::empty(at::infer_size(self.sizes(), other.sizes()), self.options());
+  binary_f32(Bin::AddRelu, self, other, 1.0f, out, "fused_add_relu");
+  return out;
+}
+
+}  // namespace ops
+
+TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
+  m.impl("add.out", TORCH_FN(ops::add_out));
+  m.impl("mul.out", TORCH_FN(ops::mul_out));
+  m.impl("relu", TORCH_FN(ops::relu));
+  m.impl("relu_", TORCH_FN(ops::relu_));
+  m.impl("relu.out", TORCH_FN(ops::relu_out));
+  m.impl("gelu", TORCH_FN(ops::gelu));
+  m.impl("gelu.out", TORCH_FN(ops::gelu_out));
+  m.impl("silu", TORCH_FN(ops::silu));
+  m.impl("silu.out", TORCH_FN(ops::silu_out));
+  m.impl("abs.out", TORCH_FN(ops::abs_out));
+  m.impl("eq.Tensor", TORCH_FN(ops::eq_tensor));
+  m.impl("eq.Tensor_out", TORCH_FN(ops::eq_tensor_out));
+  m.impl("ne.Scalar", TORCH_FN(ops::ne_scalar));
+  m.impl("ne.Scalar_out", TORCH_FN(ops::ne_scalar_out));
+  m.impl("bitwise_and.Tensor", TORCH_FN(ops::bitwise_and));
+  m.impl("bitwise_and.Tensor_out", TORCH_FN(ops::bitwise_and_out));
+  m.impl("masked_select", TORCH_FN(ops::masked_select));
+  m.impl("masked_select.out", TORCH_FN(ops::masked_select_out));
+}
+
+// csrc/ops/webgpu_ops.cpp:47-62
+TORCH_LIBRARY(webgpu, m) {
+  m.def("create_buffer(int[] size, int[] stride, ScalarType? dtype=None) -> Tensor");
+  m.def("write_buffer(Tensor(a!) self, Tensor src) -> Tensor(a!)");
+  m.def("fused_add_relu(Tensor self, Tensor src) -> Tensor");
+}
+TORCH_LIBRARY_IMPL(webgpu, PrivateUse1, m) {
+  m.impl("write_buffer", TORCH_FN(ops::write_buffer));
+  m.impl("fused_add_relu", TORCH_FN(ops::fused_add_relu));
+}
+TORCH_LIBRARY_IMPL(webgpu, CatchAll, m) {
+  m.impl("create_buffer", TORCH_FN(ops::create_buffer));
+}
+
+// csrc/ops/webgpu_ops.cpp:63-66: no autograd formulas; let every op skip the key
+TORCH_LIBRARY_IMPL(_, AutogradPrivateUse1, m) {
+  m.fallback(torch::CppFunction::makeFallthrough());
+}
+
+}  // namespace torch_webgpu

@@ -1,0 +1,35 @@
+"""torch_webgpu: the "webgpu" PrivateUse1 backend of PyTorch, with the eager op
+path implemented as hand-written gfx950 (MI355X) HIP kernels.
+
+`import torch_webgpu` registers the device exactly as the reference package does
+(python/torch_webgpu/__init__.py:1-13): after it, `device="webgpu"`,
+`.to("webgpu")` and `tensor.webgpu()` work.  The compiled extension `_C` (allocator,
+device guard, operator registrations) and the kernel library `libtwg_hip.so` are
+built in-tree by torch-webgpu_amd/build.py; there is no fallback if they are
+missing.
+"""
+import os as _os
+
+import torch
+
+try:
+    from . import _C
+except ImportError as exc:  # pragma: no cover - only without a build
+    _here = _os.path.dirname(_os.path.abspath(__file__))
+    raise ImportError(
+        "torch_webgpu._C could not be loaded (" + str(exc) + "). Build it with "
+        "`python " + _os.path.join(_os.path.dirname(_here), "build.py") + "`; "
+        "torch_webgpu has no CPU or PyTorch-ROCm fallback path.") from exc
+
+from . import webgpu  # noqa: E402
+
+torch.utils.rename_privateuse1_backend("webgpu")
+torch._register_device_module("webgpu", webgpu)
+torch.utils.generate_methods_for_privateuse1_backend(
+    for_tensor=True,
+    for_module=True,
+    for_storage=True,
+    for_packed_sequence=True,
+)
+
+__all__ = ["webgpu"]

@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "torch_webgpu", "libtwg_hip.so")
 MAX_DIMS = 8
 OUT, A, B = 0, 1, 2
 
-UNARY_COPY, UNARY_RELU, UNARY_GELU_ERF, UNARY_GELU_TANH, UNARY_SILU = 0, 1, 2, 3, 4
+UNARY_COPY, UNARY_RELU, UNARY_GELU_ERF, UNARY_GELU_TANH, UNARY_SILU, UNARY_ABS = 0, 1, 2, 3, 4, 5
 
 E_INVALID_ARG, E_UNSUPPORTED, E_SCRATCH_SMALL = -1, -2, -3
 
