@@ -336,6 +336,26 @@ def test_masked_select_bernoulli(twg, n, p):
     assert bit_equal(vals, torch.masked_select(x, m))
 
 
+@pytest.mark.parametrize("n,p", [(1 << 24, 0.5), ((1 << 24) + 3 * 65536 + 12345, 0.5),
+                                 ((1 << 24) + 5, 0.99), ((1 << 25) + 8191, 0.01),
+                                 ((1 << 24) + 70000, 1.0), ((1 << 24) + 70000, 0.0),
+                                 ((1 << 24) + 40000, -1.0)])
+def test_masked_select_large_tiles(twg, n, p):
+    # >= 2^24 elements take the 65536-element-tile kernel; a remainder below one big
+    # tile goes to a second launch that continues from the first one's count
+    _say(f"masked_select large n={n} p={p}")
+    x = W.select_source(n, seed=4)
+    if p < 0:
+        m = W.clustered_mask(n, mean_run=4096, seed=6)
+    elif 0.0 < p < 1.0:
+        m = W.bernoulli_mask(n, p, seed=11)
+    else:
+        m = torch.full((n,), p == 1.0)
+    vals, k = H.masked_select(x, m)
+    assert k == int(m.sum())
+    assert bit_equal(vals, torch.masked_select(x, m))
+
+
 def test_masked_select_clustered_and_empty(twg):
     n = (1 << 22) + 1234
     x = W.select_source(n, seed=4)

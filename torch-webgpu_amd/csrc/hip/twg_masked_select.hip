@@ -4,21 +4,32 @@
 // aten::masked_select (csrc/bindings.cpp:42): two blocking device->host copies,
 // ATen's CPU kernel, one host->device copy.
 //
-// Shape of the algorithm (one kernel, every element read once):
-//   * a tile is 4 wavefronts x 8 steps x 64 lanes x ITEMS elements;
-//   * tiles are handed out in launch order through an atomic ticket, so a tile
-//     only ever waits on tiles whose workgroups are already resident;
-//   * per step each lane turns its mask bytes into a count, three 64-wide
-//     ballots of the count's bits plus mbcnt give the lane's exclusive offset
-//     and the wavefront total; wavefront totals meet in LDS;
+// Shape of the algorithm (one kernel, mask and source each read once):
+//   * a tile is a contiguous run of elements owned by one workgroup; tiles are
+//     handed out in start order through one atomic ticket, so a tile only ever
+//     waits on tiles whose workgroups are already running (no deadlock whatever
+//     order the hardware starts workgroups in);
+//   * every lane turns 4 mask bytes into 4 selection bits; per-lane popcounts are
+//     reduced to wavefront totals, which meet in LDS;
 //   * the tile total is published at once as an AGGREGATE status word; wave 0
-//     then looks back 64 predecessors at a time (decoupled look-back) until it
-//     meets an INCLUSIVE word, and publishes its own inclusive prefix;
-//   * source values are fetched only where the lane's mask word is non-zero and
-//     while the look-back is in flight, then scattered to out[base + offset].
+//     then looks back over 256 predecessors per round (decoupled look-back) until
+//     it meets an INCLUSIVE word, and publishes its own inclusive prefix;
+//   * source values are fetched only where the lane has a selection bit set; three
+//     64-wide ballots of the lane counts plus mbcnt give each lane its offset, the
+//     values are compacted in LDS at the 16-byte phase they will have in memory
+//     and written as aligned float4s.
 // A status word packs {flag:2, value:62} so one relaxed agent-scope 64-bit
 // load/store carries everything; no fences are needed because no other memory
 // is communicated between tiles.
+//
+// Two facts about MI355X shape the large-input variant.  Same-address agent-scope
+// atomics retire at about one per 7 ns, so the ticket must not be paid 32768
+// times for 2^28 elements; and with one 1024-lane workgroup per CU the latency of
+// ticket -> mask -> look-back is only amortised by giving each workgroup a lot of
+// data.  Its tiles are therefore 65536 elements, walked as 2 sub-tiles in a rolled
+// loop; between sub-tiles only the packed selection bits (one register per 8
+// steps) stay live, and the next sub-tile's values are already in flight while the
+// current one is written out.
 #include <hip/hip_runtime.h>
 
 #include "twg_internal.h"
@@ -26,11 +37,12 @@
 namespace twg {
 namespace {
 
-constexpr int kMsThreads = 256;
-constexpr int kMsWaves = kMsThreads / 64;
-constexpr int kMsSteps = 8;
-constexpr int kMsMinTile = kMsThreads * kMsSteps;  // tile size of the 1-item variants
-constexpr size_t kMsHeaderBytes = 256;             // ticket counter, padded
+constexpr int kSteps = 8;           // steps of 256 elements per wavefront and sub-tile
+constexpr int kWaveElems = 256 * kSteps;
+constexpr int kScalarWaves = 4;     // fallback variants: one element per lane
+constexpr int kMsMinTile = 64 * kScalarWaves * kSteps;  // smallest tile of any variant
+constexpr size_t kMsHeaderBytes = 256;                  // tickets and carry, padded
+constexpr int kLookPerLane = 4;                         // look-back window = 64 * 4 tiles
 
 constexpr uint64_t kFlagShift = 62;
 constexpr uint64_t kFlagAggregate = 1ull << kFlagShift;
@@ -43,6 +55,8 @@ struct MsGeom {
   int64_t sstride[TWG_MAX_DIMS];  // source
   int64_t mstride[TWG_MAX_DIMS];  // mask
 };
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t lanes_below(uint64_t ballot) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(ballot >> 32),
@@ -62,25 +76,266 @@ __device__ __forceinline__ int64_t wave_sum_i64(int64_t v) {
   return v;
 }
 
-// High bit of each byte set where the byte is non-zero.
-__device__ __forceinline__ uint32_t nonzero_bytes(uint32_t w) {
-  return (((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u;
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
 }
 
-template <int ITEMS, bool STRIDED>
-__global__ __launch_bounds__(kMsThreads) void ms_compact(float *out, int64_t *d_count,
-                                                         const float *src, const uint8_t *mask,
-                                                         int64_t n, uint32_t ntiles,
-                                                         uint32_t *ticket, uint64_t *status,
-                                                         MsGeom g) {
-  static_assert(ITEMS == 1 || ITEMS == 4, "lane handles one element or one float4");
-  static_assert(!STRIDED || ITEMS == 1, "strided operands go one element per lane");
-  constexpr int kStepElems = 64 * ITEMS;
-  constexpr int kWaveElems = kStepElems * kMsSteps;
-  constexpr int kTileElems = kWaveElems * kMsWaves;
+// Four mask bytes -> four selection bits (bit j set if byte j is non-zero).
+__device__ __forceinline__ uint32_t select_bits(uint32_t w) {
+  const uint32_t high = (((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u;  // per byte: != 0
+  return (((high >> 7) * 0x01020408u) >> 24) & 0xFu;  // gather bits 0, 8, 16, 24
+}
+
+// From each lane's count c in 0..4: the lane's exclusive offset within the
+// wavefront and the wavefront total, by three ballots of the bits of c.
+__device__ __forceinline__ void wave_offsets(uint32_t c, uint32_t &below, uint32_t &total) {
+  const uint64_t b0 = __ballot(c & 1u), b1 = __ballot(c & 2u), b2 = __ballot(c & 4u);
+  below = lanes_below(b0) + 2u * lanes_below(b1) + 4u * lanes_below(b2);
+  total = (uint32_t)__popcll(b0) + 2u * (uint32_t)__popcll(b1) + 4u * (uint32_t)__popcll(b2);
+}
+
+// Exclusive prefix of tile `tile`: sum of the totals of all earlier tiles.  Run by
+// one full wavefront.  Each round inspects the 256 nearest unseen predecessors
+// (4 status words per lane, nearest first), waits until all of them have published
+// at least an aggregate, and stops at the nearest one that carries an inclusive
+// prefix.
+__device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t tile, int lane) {
+  int64_t exclusive = 0;
+  int64_t look = (int64_t)tile - 1 - lane;  // lane's nearest candidate
+  while (true) {
+    uint64_t st[kLookPerLane];
+    while (true) {
+      bool pending = false;
+#pragma unroll
+      for (int q = 0; q < kLookPerLane; ++q) {
+        const int64_t idx = look - 64 * q;
+        // slots before tile 0 behave like an inclusive prefix of 0
+        st[q] = (idx >= 0) ? status_load(status + idx) : kFlagInclusive;
+        pending |= (st[q] >> kFlagShift) == 0;
+      }
+      if (__ballot(pending) == 0) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    int64_t part = 0;
+    bool done = false;
+#pragma unroll
+    for (int q = 0; q < kLookPerLane; ++q) {
+      if (!done) {
+        const uint64_t incl = __ballot((st[q] >> kFlagShift) == 2);
+        const int64_t val = (int64_t)(st[q] & kValueMask);
+        if (incl) {
+          const int first = __builtin_ctzll(incl);  // nearest predecessor with a full prefix
+          part += (lane <= first) ? val : 0;
+          done = true;
+        } else {
+          part += val;
+        }
+      }
+    }
+    exclusive += wave_sum_i64(part);
+    if (done) return exclusive;
+    look -= 64 * kLookPerLane;
+  }
+}
+
+// Aggregate, look-back, inclusive prefix: the part every variant shares.  Call
+// with all threads; returns the tile's exclusive prefix to all of them.  s_slot is
+// one int64 of LDS.  The last tile also writes the grand total, plus *carry_in if a
+// previous launch compacted the elements before this one's.
+__device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, uint32_t ntiles,
+                                               uint32_t tile_total, int64_t *d_count,
+                                               int64_t *s_slot, const int64_t *carry_in) {
+  const int lane = threadIdx.x & 63;
+  if (threadIdx.x < 64) {  // wave 0
+    if (lane == 0)
+      status_store(status + tile,
+                   (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
+    int64_t exclusive = 0;
+    if (tile != 0) {
+      exclusive = look_back(status, tile, lane);
+      if (lane == 0)
+        status_store(status + tile, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+    }
+    if (lane == 0) {
+      *s_slot = exclusive;
+      if (tile == ntiles - 1)
+        *d_count = exclusive + (int64_t)tile_total + (carry_in ? *carry_in : 0);
+    }
+  }
+  __syncthreads();
+  return *s_slot;
+}
+
+// ------------------------------------------------------------------ fast variant
+// Dense source and mask, 16-byte aligned source, 4-byte aligned mask.
+// A tile is SUB sub-tiles; in each, wavefront w owns 8 steps of 256 elements
+// (lane l, step k: elements 4l..4l+3 of that step).
+//
+// RAGGED = false: the host guarantees that every tile of the launch is full, so the
+// kernel carries no bounds-checked code (a checked instance would set the register
+// budget of the whole kernel although at most one tile ever runs it).
+
+template <int WAVES, int SUB>
+struct MsShared {
+  uint32_t tile;
+  uint32_t wave_total[SUB][WAVES];
+  int64_t base;
+  __attribute__((aligned(16))) float stage[WAVES][kWaveElems + 4];
+};
+
+template <int WAVES, int SUB, bool RAGGED>
+__global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t *d_count,
+                                                             const float *src,
+                                                             const uint8_t *mask, int64_t n,
+                                                             uint32_t ntiles, uint32_t *ticket,
+                                                             uint64_t *status,
+                                                             const int64_t *carry_in) {
+  constexpr uint32_t kSubElems = (uint32_t)kWaveElems * WAVES;
+  constexpr int64_t kTileElems = (int64_t)kSubElems * SUB;
+  __shared__ MsShared<WAVES, SUB> sh;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0)
+    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const uint32_t tile = sh.tile;
+  // tile bases are wavefront-uniform; everything per lane is a 32-bit offset
+  const int64_t start = (int64_t)tile * kTileElems;
+  const uint8_t *mask_tile = mask + start;
+  const float *src_tile = src + start;
+  const uint32_t lane_off = wave * kWaveElems + lane * 4;
+  const int64_t left = n - start;
+  const uint32_t remaining = left < kTileElems ? (uint32_t)left : (uint32_t)kTileElems;
+  if (carry_in) out += *carry_in;
+
+  // ---- 1. the whole tile's mask -> packed selection bits and wavefront totals
+  uint32_t bits[SUB];  // 4 bits per step: bit 4k+j <=> element j of step k is selected
+#pragma unroll
+  for (int s = 0; s < SUB; ++s) {
+    uint32_t w[kSteps];
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {  // all 8 loads in flight before any is used
+      const uint32_t e = lane_off + s * kSubElems + k * 256;
+      if (!RAGGED || e + 4 <= remaining) {
+        w[k] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(mask_tile + e));
+      } else {
+        w[k] = 0;
+        for (uint32_t j = 0; j < 4; ++j)
+          if (e + j < remaining && mask_tile[e + j]) w[k] |= 1u << (8 * j);
+      }
+    }
+    uint32_t b = 0;
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) b |= select_bits(w[k]) << (4 * k);
+    bits[s] = b;
+    const uint32_t wt = wave_sum_u32(__popc(b));
+    if (lane == 0) sh.wave_total[s][wave] = wt;
+  }
+  __syncthreads();
+  uint32_t wbase[SUB];  // offset of this wavefront's part of sub-tile s from the tile's start
+  uint32_t wtot[SUB];
+  uint32_t tile_total = 0;
+#pragma unroll
+  for (int s = 0; s < SUB; ++s) {
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const uint32_t t = sh.wave_total[s][w];
+      if ((uint32_t)w == wave) {
+        wbase[s] = tile_total;
+        wtot[s] = t;
+      }
+      tile_total += t;
+    }
+  }
+
+  // ---- 2. source values of sub-tile 0 go in flight, then aggregate / look-back
+  f32x4 vals[kSteps];
+  auto fetch = [&](uint32_t b, uint32_t sub_off) {
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {
+      if ((b >> (4 * k)) & 0xFu) {
+        const uint32_t e = lane_off + sub_off + k * 256;
+        if (!RAGGED || e + 4 <= remaining) {
+          vals[k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src_tile + e));
+        } else {
+          for (uint32_t j = 0; j < 4; ++j) vals[k][j] = (e + j < remaining) ? src_tile[e + j] : 0.0f;
+        }
+      }
+    }
+  };
+  fetch(bits[0], 0);
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, carry_in);
+
+  // ---- 3. per sub-tile (rolled loop): compact in LDS at the output's 16-byte phase,
+  //         start the next sub-tile's loads, write aligned float4s.  The ragged ends
+  //         go out element by element: their neighbours belong to other wavefronts.
+  float *stage = sh.stage[wave];
+#pragma unroll 1
+  for (int s = 0; s < SUB; ++s) {
+    uint32_t b = bits[0], wb = wbase[0], wt = wtot[0], b_next = 0;
+#pragma unroll
+    for (int q = 1; q < SUB; ++q) {  // register arrays indexed by a loop-carried s
+      if (s == q) {
+        b = bits[q];
+        wb = wbase[q];
+        wt = wtot[q];
+      }
+      if (s + 1 == q) b_next = bits[q];
+    }
+    float *wout = out + (base + wb);  // this wavefront's first output value
+    const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 3u);
+    uint32_t run = shift;
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) {
+      const uint32_t f = (b >> (4 * k)) & 0xFu;
+      uint32_t below, total;
+      wave_offsets(__popc(f), below, total);
+      if (f) {
+        uint32_t pos = run + below;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (f & (1u << j)) stage[pos++] = vals[k][j];
+        }
+      }
+      run += total;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (s + 1 < SUB) fetch(b_next, (s + 1) * kSubElems);
+    const uint32_t span_end = shift + wt;
+    float *obase = wout - shift;  // 16-byte aligned
+    if (wt != 0) {
+      for (uint32_t v = lane; 4 * v < span_end; v += 64) {
+        const f32x4 x = *reinterpret_cast<const f32x4 *>(stage + 4 * v);
+        if (4 * v >= shift && 4 * v + 4 <= span_end) {
+          __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * v));
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const uint32_t i = 4 * v + c;
+            if (i >= shift && i < span_end) obase[i] = x[c];
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// -------------------------------------------------------------- fallback variants
+// One element per lane: misaligned pointers (STRIDED = false) or broadcast /
+// strided source and mask addressed through div/mod index math (STRIDED = true).
+
+template <bool STRIDED>
+__global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
+    float *out, int64_t *d_count, const float *src, const uint8_t *mask, int64_t n,
+    uint32_t ntiles, uint32_t *ticket, uint64_t *status, MsGeom g) {
+  constexpr int kWaveSpan = 64 * kSteps;
+  constexpr int kTileElems = kWaveSpan * kScalarWaves;
 
   __shared__ uint32_t s_tile;
-  __shared__ uint32_t s_wave_total[kMsWaves];
+  __shared__ uint32_t s_wave_total[kScalarWaves];
   __shared__ int64_t s_base;
 
   const int lane = threadIdx.x & 63;
@@ -89,139 +344,65 @@ __global__ __launch_bounds__(kMsThreads) void ms_compact(float *out, int64_t *d_
     s_tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t tile = s_tile;
-  const int64_t wstart = (int64_t)tile * kTileElems + (int64_t)wave * kWaveElems;
+  const int64_t wstart = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
 
-  // ---- 1. mask -> per-lane offsets inside the wavefront
-  uint32_t nz[kMsSteps];    // ITEMS == 4: bit 8j+7 set if element j selected; ITEMS == 1: 0/1
-  uint32_t loff[kMsSteps];  // exclusive offset of the lane's first element within the wave
-  int64_t soff[STRIDED ? kMsSteps : 1];
+  bool sel[kSteps];
+  uint32_t loff[kSteps];
+  int64_t soff[kSteps];
   uint32_t wtotal = 0;
 #pragma unroll
-  for (int k = 0; k < kMsSteps; ++k) {
-    const int64_t e = wstart + (int64_t)k * kStepElems + (int64_t)lane * ITEMS;
-    uint32_t f = 0;
-    if constexpr (ITEMS == 4) {
-      if (e + 4 <= n) {
-        f = nonzero_bytes(*reinterpret_cast<const uint32_t *>(mask + e));
-      } else {
-        for (int j = 0; j < 4; ++j)
-          if (e + j < n && mask[e + j]) f |= 0x80u << (8 * j);
-      }
-      const uint32_t c = __popc(f);
-      const uint64_t b0 = __ballot(c & 1u), b1 = __ballot(c & 2u), b2 = __ballot(c & 4u);
-      loff[k] = wtotal + lanes_below(b0) + 2u * lanes_below(b1) + 4u * lanes_below(b2);
-      wtotal += (uint32_t)__popcll(b0) + 2u * (uint32_t)__popcll(b1) + 4u * (uint32_t)__popcll(b2);
-    } else {
-      if (e < n) {
-        if constexpr (STRIDED) {
-          int64_t rem = e, om = 0, os = 0;
-          for (int d = 0; d < g.ndim; ++d) {
-            const int64_t q = rem / g.shape[d];
-            const int64_t c = rem - q * g.shape[d];
-            rem = q;
-            om += c * g.mstride[d];
-            os += c * g.sstride[d];
-          }
-          soff[k] = os;
-          f = mask[om] != 0;
-        } else {
-          f = mask[e] != 0;
+  for (int k = 0; k < kSteps; ++k) {
+    const int64_t e = wstart + k * 64 + lane;
+    bool f = false;
+    soff[k] = e;
+    if (e < n) {
+      if constexpr (STRIDED) {
+        int64_t rem = e, om = 0, os = 0;
+        for (int d = 0; d < g.ndim; ++d) {  // dimension 0 is the fastest-moving one
+          const int64_t q = rem / g.shape[d];
+          const int64_t c = rem - q * g.shape[d];
+          rem = q;
+          om += c * g.mstride[d];
+          os += c * g.sstride[d];
         }
+        soff[k] = os;
+        f = mask[om] != 0;
+      } else {
+        f = mask[e] != 0;
       }
-      const uint64_t b = __ballot(f);
-      loff[k] = wtotal + lanes_below(b);
-      wtotal += (uint32_t)__popcll(b);
     }
-    nz[k] = f;
+    const uint64_t b = __ballot(f);
+    loff[k] = wtotal + lanes_below(b);
+    wtotal += (uint32_t)__popcll(b);
+    sel[k] = f;
   }
   if (lane == 0) s_wave_total[wave] = wtotal;
   __syncthreads();
   uint32_t wave_base = 0, tile_total = 0;
 #pragma unroll
-  for (int w = 0; w < kMsWaves; ++w) {
+  for (int w = 0; w < kScalarWaves; ++w) {
     const uint32_t t = s_wave_total[w];
     if (w < wave) wave_base += t;
     tile_total += t;
   }
-
-  // ---- 2. publish the aggregate as early as possible
-  if (threadIdx.x == 0) {
-    status_store(status + tile, (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
-  }
-
-  // ---- 3. fetch the selected source values (in flight during the look-back)
-  float vals[kMsSteps][ITEMS];
+  float vals[kSteps];
 #pragma unroll
-  for (int k = 0; k < kMsSteps; ++k) {
-    const int64_t e = wstart + (int64_t)k * kStepElems + (int64_t)lane * ITEMS;
-    if constexpr (ITEMS == 4) {
-      if (nz[k]) {
-        if (e + 4 <= n) {
-          const float4 v = *reinterpret_cast<const float4 *>(src + e);
-          vals[k][0] = v.x; vals[k][1] = v.y; vals[k][2] = v.z; vals[k][3] = v.w;
-        } else {
-          for (int j = 0; j < 4; ++j) vals[k][j] = (e + j < n) ? src[e + j] : 0.0f;
-        }
-      }
-    } else {
-      if (nz[k]) vals[k][0] = STRIDED ? src[soff[k]] : src[e];
-    }
-  }
-
-  // ---- 4. decoupled look-back (wave 0)
-  if (wave == 0) {
-    int64_t exclusive = 0;
-    if (tile != 0) {
-      int64_t look = (int64_t)tile - 1 - lane;
-      while (true) {
-        uint64_t st;
-        while (true) {
-          // lanes that ran off the front behave like an inclusive prefix of 0
-          st = (look >= 0) ? status_load(status + look) : kFlagInclusive;
-          if (__ballot((st >> kFlagShift) == 0) == 0) break;
-          __builtin_amdgcn_s_sleep(1);
-        }
-        const uint64_t incl = __ballot((st >> kFlagShift) == 2);
-        const int64_t val = (int64_t)(st & kValueMask);
-        if (incl) {
-          const int first = __builtin_ctzll(incl);  // nearest predecessor with a full prefix
-          exclusive += wave_sum_i64(lane <= first ? val : 0);
-          break;
-        }
-        exclusive += wave_sum_i64(val);
-        look -= 64;
-      }
-      if (lane == 0) status_store(status + tile, kFlagInclusive | (uint64_t)(exclusive + tile_total));
-    }
-    if (lane == 0) {
-      s_base = exclusive;
-      if (tile == ntiles - 1) *d_count = exclusive + (int64_t)tile_total;
-    }
-  }
-  __syncthreads();
-
-  // ---- 5. ordered scatter
-  const int64_t base = s_base + wave_base;
+  for (int k = 0; k < kSteps; ++k)
+    if (sel[k]) vals[k] = src[soff[k]];
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &s_base, nullptr);
+  const int64_t wpos = base + wave_base;
 #pragma unroll
-  for (int k = 0; k < kMsSteps; ++k) {
-    if constexpr (ITEMS == 4) {
-      if (nz[k]) {
-        int64_t pos = base + loff[k];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (nz[k] & (0x80u << (8 * j))) out[pos++] = vals[k][j];
-        }
-      }
-    } else {
-      if (nz[k]) out[base + loff[k]] = vals[k][0];
-    }
-  }
+  for (int k = 0; k < kSteps; ++k)
+    if (sel[k]) out[wpos + loff[k]] = vals[k];
 }
 
-template <int ITEMS>
-constexpr int64_t tile_elems() {
-  return (int64_t)kMsThreads * kMsSteps * ITEMS;
-}
+// Tile shapes of the fast variant: 65536-element tiles (1024 lanes, 2 sub-tiles)
+// once there is one per CU, 8192-element tiles (256 lanes) below that.
+constexpr int kBigWaves = 16, kBigSub = 2;
+constexpr int kSmallWaves = 4, kSmallSub = 1;
+constexpr int64_t kBigTile = (int64_t)kWaveElems * kBigWaves * kBigSub;
+constexpr int64_t kSmallTile = (int64_t)kWaveElems * kSmallWaves * kSmallSub;
+constexpr int64_t kBigMinElems = kBigTile * 256;  // 2^24
 
 }  // namespace
 }  // namespace twg
@@ -258,33 +439,62 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
   const bool dense =
       g.ndim == 0 || (g.ndim == 1 && g.stride[TWG_A][0] == 1 && g.stride[TWG_B][0] == 1);
   const bool vec4 = dense && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
-                    reinterpret_cast<uintptr_t>(mask) % 4 == 0;
-  const int64_t tile = vec4 ? tile_elems<4>() : tile_elems<1>();
-  const int64_t ntiles64 = (g.numel + tile - 1) / tile;
+                    reinterpret_cast<uintptr_t>(mask) % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(out) % 4 == 0;
+  const bool big = vec4 && g.numel >= kBigMinElems;
+
+  // scratch: [0] ticket, [4] ticket of the remainder launch, [8] carry between the
+  // two launches, [256...] one status word per tile
+  uint32_t *ticket = static_cast<uint32_t *>(scratch);
+  int64_t *carry = reinterpret_cast<int64_t *>(static_cast<char *>(scratch) + 8);
+  uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+  auto tiles_of = [](int64_t n, int64_t tile) { return (n + tile - 1) / tile; };
+
+  if (big) {
+    // Full 65536-element tiles go through the check-free kernel; what is left (less
+    // than one big tile) is compacted by a second launch of the small variant that
+    // starts from the first launch's total.
+    const int64_t nbig = g.numel / kBigTile;
+    const int64_t rem = g.numel - nbig * kBigTile;
+    const int64_t nrem = tiles_of(rem, kSmallTile);
+    if (nbig > INT32_MAX) return TWG_E_UNSUPPORTED;
+    if ((rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (size_t)(nbig + nrem),
+                             stream)))
+      return rc;
+    ms_compact_vec<kBigWaves, kBigSub, false><<<(unsigned)nbig, kBigWaves * 64, 0, s>>>(
+        out, rem ? carry : d_count, src, mask, nbig * kBigTile, (uint32_t)nbig, ticket, status,
+        nullptr);
+    if (rem)
+      ms_compact_vec<kSmallWaves, kSmallSub, true><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
+          out, d_count, src + nbig * kBigTile, mask + nbig * kBigTile, rem, (uint32_t)nrem,
+          ticket + 1, status + nbig, carry);
+    return (int)hipGetLastError();
+  }
+
+  const int64_t tile = vec4 ? kSmallTile : (int64_t)kMsMinTile;
+  const int64_t ntiles64 = tiles_of(g.numel, tile);
   if (ntiles64 > INT32_MAX) return TWG_E_UNSUPPORTED;
   const uint32_t ntiles = (uint32_t)ntiles64;
-
-  uint32_t *ticket = static_cast<uint32_t *>(scratch);
-  uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
   if ((rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
     return rc;
 
-  MsGeom mg{};
-  mg.ndim = g.ndim;
-  for (int d = 0; d < TWG_MAX_DIMS; ++d) {
-    mg.shape[d] = g.shape[d];
-    mg.sstride[d] = g.stride[TWG_A][d];
-    mg.mstride[d] = g.stride[TWG_B][d];
-  }
   if (vec4) {
-    ms_compact<4, false><<<ntiles, kMsThreads, 0, s>>>(out, d_count, src, mask, g.numel, ntiles,
-                                                        ticket, status, mg);
-  } else if (dense) {
-    ms_compact<1, false><<<ntiles, kMsThreads, 0, s>>>(out, d_count, src, mask, g.numel, ntiles,
-                                                        ticket, status, mg);
+    ms_compact_vec<kSmallWaves, kSmallSub, true><<<ntiles, kSmallWaves * 64, 0, s>>>(
+        out, d_count, src, mask, g.numel, ntiles, ticket, status, nullptr);
   } else {
-    ms_compact<1, true><<<ntiles, kMsThreads, 0, s>>>(out, d_count, src, mask, g.numel, ntiles,
-                                                       ticket, status, mg);
+    MsGeom mg{};
+    mg.ndim = g.ndim;
+    for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+      mg.shape[d] = g.shape[d];
+      mg.sstride[d] = g.stride[TWG_A][d];
+      mg.mstride[d] = g.stride[TWG_B][d];
+    }
+    if (dense)
+      ms_compact_scalar<false><<<ntiles, kScalarWaves * 64, 0, s>>>(out, d_count, src, mask,
+                                                                    g.numel, ntiles, ticket, status, mg);
+    else
+      ms_compact_scalar<true><<<ntiles, kScalarWaves * 64, 0, s>>>(out, d_count, src, mask,
+                                                                   g.numel, ntiles, ticket, status, mg);
   }
   return (int)hipGetLastError();
 }
