@@ -134,7 +134,10 @@ def test_add_row_and_column_bias(twg, rows, cols):
     assert bit_equal(H.add(tall[::2], bias), tall[::2] + bias)
 
 
-@pytest.mark.parametrize("rows,cols", [(256, 512), (100, 70), (64, 64), (65, 33), (16, 1000)])
+@pytest.mark.parametrize("rows,cols", [(256, 512), (100, 70), (64, 64), (65, 33), (16, 1000),
+                                       # multiples of 4 take the 128-bit tile kernel: full and
+                                       # ragged 256x32 tiles, and the 64x64 shape below 256
+                                       (264, 300), (68, 132), (36, 1028), (1024, 40), (20, 16)])
 def test_add_transposed_operand(twg, rows, cols):
     # config 3b shape family: A[rows, cols] viewed as (cols, rows) with strides
     # (1, cols), plus a contiguous C[cols, rows].  TensorIterator gives the output
