@@ -182,11 +182,19 @@ def main():
         "algorithmic_bytes_per_launch": dominant["bytes"],
         "avg_launch_ms": dominant["avg_ms"],
     }
-    tr = os.path.join(ROOT, "profiles", "hbm_traffic_bytes.json")
-    if os.path.exists(tr):  # measured FETCH_SIZE + WRITE_SIZE per launch, scaled by a copy kernel
+    # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE + WRITE_SIZE, each scaled by
+    # the plain copy kernel); a recorded figure, not re-measured by this run
+    traffic = {}
+    tr = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if os.path.exists(tr):
         with open(tr) as f:
-            traffic = json.load(f)
-        roofline["traffic"] = traffic.get(dominant["op"] + f"@2^{args.log2n}")
+            for line in f:
+                if "=" in line and not line.startswith("#"):
+                    k, v = line.split("=")
+                    traffic[k.strip()] = int(v)
+    roofline["traffic"] = traffic.get(dominant["op"] + f"@2^{args.log2n}")
+    for d in head:
+        d["traffic"] = traffic.get(d["op"] + f"@2^{args.log2n}")
 
     # ------------------------------------------------------------ sweep of the other configs
     del a_h, b_h
