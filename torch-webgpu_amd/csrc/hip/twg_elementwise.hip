@@ -168,18 +168,21 @@ __device__ __forceinline__ TO apply(const Op &op, TA a, TB b) {
 }
 
 // ------------------------------------------------------------- ew_contig
-// One pack per lane, one block per 256 packs, no loop: on MI355X a grid of a few
-// hundred thousand short-lived blocks streams faster (add: 6.4 TB/s) than a
-// persistent grid-stride loop sized to the 256 CUs (5.4 TB/s).
+// One pack per lane, no loop: on MI355X a grid of very many short-lived blocks
+// streams faster (add: 6.4-6.7 TB/s) than a persistent grid-stride loop sized to
+// the 256 CUs (5.4 TB/s).  Block size matters too: single-wavefront blocks give add
+// 83% of peak against 80% for 256 lanes, while kernels whose output is narrower
+// than their input (compares: one dword of bools per lane) do best at 256.
 
-template <int NIN, int VEC, bool STREAM, typename Op, typename TO, typename TA, typename TB>
-__global__ __launch_bounds__(kThreads) void ew_contig(TO *out, const TA *a, const TB *b,
-                                                      int64_t numel, Op op) {
+template <int THREADS, int NIN, int VEC, bool STREAM, typename Op, typename TO, typename TA,
+          typename TB>
+__global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const TB *b,
+                                                     int64_t numel, Op op) {
   using PO = Pack<TO, VEC>;
   using PA = Pack<TA, VEC>;
   using PB = Pack<TB, VEC>;
   const int64_t nvec = numel / VEC;
-  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t i = (int64_t)blockIdx.x * THREADS + threadIdx.x;
   if (i < nvec) {
     const PA va = load_pack<STREAM>(reinterpret_cast<const PA *>(a) + i);
     PB vb;
@@ -208,9 +211,9 @@ struct RowGeom {
   int64_t ostride[3][TWG_MAX_DIMS - 1];
 };
 
-template <int NIN, int VEC, int UNROLL, bool STREAM, bool A_BC, bool B_BC, typename Op, typename TO,
-          typename TA, typename TB>
-__global__ __launch_bounds__(kThreads) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
+template <int THREADS, int NIN, int VEC, int UNROLL, bool STREAM, bool A_BC, bool B_BC, typename Op,
+          typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
                                                     Op op) {
   using PO = Pack<TO, VEC>;
   using PA = Pack<TA, VEC>;
@@ -237,12 +240,12 @@ __global__ __launch_bounds__(kThreads) void ew_rows(TO *out, const TA *a, const 
   if constexpr (A_BC) abc = arow[0];
   if constexpr (NIN == 2 && B_BC) bbc = brow[0];
 
-  const int64_t e0 = (int64_t)chunk * (kThreads * VEC * UNROLL) + (int64_t)threadIdx.x * VEC;
+  const int64_t e0 = (int64_t)chunk * (THREADS * VEC * UNROLL) + (int64_t)threadIdx.x * VEC;
   PA va[UNROLL];
   PB vb[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const int64_t e = e0 + (int64_t)u * kThreads * VEC;
+    const int64_t e = e0 + (int64_t)u * THREADS * VEC;
     if (e < g.len) {
       if constexpr (!A_BC) va[u] = load_pack<STREAM>(reinterpret_cast<const PA *>(arow + e));
       if constexpr (NIN == 2 && !B_BC) vb[u] = load_pack<STREAM>(reinterpret_cast<const PB *>(brow + e));
@@ -250,7 +253,7 @@ __global__ __launch_bounds__(kThreads) void ew_rows(TO *out, const TA *a, const 
   }
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const int64_t e = e0 + (int64_t)u * kThreads * VEC;
+    const int64_t e = e0 + (int64_t)u * THREADS * VEC;
     if (e < g.len) {
       PO r;
 #pragma unroll
@@ -541,7 +544,8 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
   constexpr int U = TWG_ROWS_UNROLL;
   RowGeom rg{};
   rg.len = g.shape[0];
-  const int64_t per_block = (int64_t)kThreads * VEC * U;
+  constexpr int kBlock = 64;  // single-wavefront blocks stream best (see ew_contig)
+  const int64_t per_block = (int64_t)kBlock * VEC * U;
   const int64_t cpr = (rg.len + per_block - 1) / per_block;
   const int64_t rows = g.numel / rg.len;
   if (cpr * rows > INT32_MAX || cpr > UINT32_MAX) return TWG_E_UNSUPPORTED;
@@ -553,11 +557,11 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
   }
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
   if (stream)
-    ew_rows<NIN, VEC, U, true, A_BC, B_BC, Op, TO, TA, TB>
-        <<<(unsigned)(cpr * rows), kThreads, 0, s>>>(out, a, b, rg, op);
+    ew_rows<kBlock, NIN, VEC, U, true, A_BC, B_BC, Op, TO, TA, TB>
+        <<<(unsigned)(cpr * rows), kBlock, 0, s>>>(out, a, b, rg, op);
   else
-    ew_rows<NIN, VEC, U, false, A_BC, B_BC, Op, TO, TA, TB>
-        <<<(unsigned)(cpr * rows), kThreads, 0, s>>>(out, a, b, rg, op);
+    ew_rows<kBlock, NIN, VEC, U, false, A_BC, B_BC, Op, TO, TA, TB>
+        <<<(unsigned)(cpr * rows), kBlock, 0, s>>>(out, a, b, rg, op);
   return (int)hipGetLastError();
 }
 
@@ -673,18 +677,19 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
                         (NIN == 1 || aligned_to(b, sizeof(TB) * VEC));
     const bool stream =
         g.numel * (int64_t)(sizeof(TO) + sizeof(TA) + (NIN == 2 ? sizeof(TB) : 0)) > kStreamBytes;
+    constexpr int kBlock = sizeof(TO) < sizeof(TA) ? 256 : 64;
     const int64_t packs = vec_ok ? (g.numel + VEC - 1) / VEC : g.numel;
-    const int64_t blocks = (packs + kThreads - 1) / kThreads;
+    const int64_t blocks = (packs + kBlock - 1) / kBlock;
     if (blocks > INT32_MAX) return TWG_E_UNSUPPORTED;
     const unsigned grid = (unsigned)blocks;
     if (vec_ok && stream)
-      ew_contig<NIN, VEC, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, VEC, true, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     else if (vec_ok)
-      ew_contig<NIN, VEC, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, VEC, false, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     else if (stream)
-      ew_contig<NIN, 1, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, 1, true, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     else
-      ew_contig<NIN, 1, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, 1, false, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     return (int)hipGetLastError();
   }
 
