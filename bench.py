@@ -169,7 +169,7 @@ def main():
     head = [
         summarize("add", "ew_contig<AddOp>", bytes_add, add_ms, n),
         summarize("gelu", "ew_contig<GeluErfOp>", bytes_gelu, gelu_ms, n),
-        summarize("masked_select_p0.50", "ms_compact<4>", bytes_ms, msk_ms, n,
+        summarize("masked_select_p0.50", "ms_compact_vec<16,2>", bytes_ms, msk_ms, n,
                   {"selected": k50, "op_ms_with_count_readback": round(sum(mso_ms) / K, 5)}),
     ]
     ops += head
@@ -273,7 +273,7 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
                 it_t.stride[slot][0], it_t.stride[slot][1] = st
             ms = time_launches(lambda: capi.check(L.twg_add_f32(d_out.ptr, d_a3.ptr, d_c3.ptr, f32(1.0),
                                                                 ctypes.byref(it_t), None)), Wm, K)
-            res.append(summarize("add_transposed", "ew_tile<AddOp>", by["add_transposed"] * n, ms, n,
+            res.append(summarize("add_transposed", "ew_tile_vec<AddOp,256,32>", by["add_transposed"] * n, ms, n,
                                  {"logical_shape": [c3, r3], "out_strides": [1, c3]}))
         del d_a3, d_bias, d_c3
 
@@ -314,7 +314,7 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         ms_full = time_launches(full, 1, K)
         if int(cnt_host[0]) != k:
             raise RuntimeError(f"{name}: count {int(cnt_host[0])} != {k}")
-        res.append(summarize(name, "ms_compact<4>", W.masked_select_bytes(n, k), ms_kernel, n,
+        res.append(summarize(name, "ms_compact_vec<16,2>", W.masked_select_bytes(n, k), ms_kernel, n,
                              {"selected": k,
                               "op_ms_with_count_readback": round(sum(ms_full) / len(ms_full), 5)}))
         del d_mask
@@ -328,9 +328,10 @@ def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu
     import torch.nn.functional as F
 
     OL = oracle.lib()
-    ns_add = min(n, 1 << 26)
-    ns_gelu = min(n, 1 << 24)
-    ns_ms = min(n, 1 << 26)
+    # about 10 s of single-thread work in total (gelu through libm erfc dominates)
+    ns_add = min(n, 1 << 27)
+    ns_gelu = min(n, 1 << 27)
+    ns_ms = min(n, 1 << 27)
     a = torch.rand(ns_add) * 8 - 4
     b = torch.rand(ns_add) * 8 - 4
     o = torch.empty(ns_add)
@@ -360,7 +361,7 @@ def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu
     threads = os.cpu_count() or 1
     torch.set_num_threads(threads)
     log(f"CPU baseline: PyTorch CPU kernels, {threads} threads ...")
-    nt = min(n, 1 << 27)
+    nt = n  # the full configuration
     a = torch.rand(nt) * 8 - 4
     b = torch.rand(nt) * 8 - 4
     o = torch.empty(nt)

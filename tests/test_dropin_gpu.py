@@ -192,6 +192,19 @@ def test_empty_strided_resize_as_strided():
     assert oracle.as_strided_fits((3,), (-1,), 2, 24)  # negative strides are admitted when they fit
 
 
+def test_scalar_readback_and_printing():
+    t = dev(torch.tensor([0.0, 1.5, -2.0, 0.0]))
+    assert t[1].item() == 1.5 and float(t[2]) == -2.0
+    assert t.tolist() == [0.0, 1.5, -2.0, 0.0]
+    assert (t + t)[1].item() == 3.0
+    with pytest.raises((RuntimeError, ValueError)):
+        t.item()
+    text = repr(t)
+    assert "1.5" in text and "device='webgpu:0'" in text
+    assert "True" in repr(t.ne(0.0))
+    assert str(torch.empty(0, device="webgpu")).startswith("tensor([]")
+
+
 def test_allocator_reuses_blocks():
     a = dev(torch.randn(1 << 18))
     torch.webgpu.synchronize()
@@ -214,7 +227,7 @@ def test_add_forms_match_oracle():
     a, b = dev(a_h), dev(b_h)
     assert bit_equal((a + b).to("cpu"), oracle.add(a_h, b_h))
     assert bit_equal(torch.add(a, b, alpha=2.5).to("cpu"), oracle.add(a_h, b_h, alpha=2.5))
-    out = torch.empty(1, device="webgpu")
+    out = torch.empty(0, device="webgpu")
     torch.add(a, b, out=out)  # resized by the iterator
     assert bit_equal(out.to("cpu"), a_h + b_h)
     c = a.clone()

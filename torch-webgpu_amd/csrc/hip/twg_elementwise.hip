@@ -2,13 +2,14 @@
 // activations, strided copy, eq / ne / and.  All HBM-bound: no MFMA.
 //
 // One templated family of four kernels serves every op:
-//   ew_contig  - every operand dense and equally ordered: 128-bit loads/stores,
-//                grid-stride over block-sized chunks.
+//   ew_contig  - every operand dense and equally ordered: one 128-bit pack per
+//                lane, one short-lived block per 64 (or 256) packs, no loop.
 //   ew_rows    - inner dimension unit-stride (or broadcast) for every operand,
 //                outer dimensions arbitrary (row bias, column bias, slices).
-//   ew_tile    - an input whose unit stride lies along another dimension than
-//                the output's: 64x64 tiles staged through LDS so both sides of
-//                the transpose stay coalesced.
+//   ew_tile(_vec) - an input whose unit stride lies along another dimension than
+//                the output's: tiles staged through LDS so both sides of the
+//                transpose stay coalesced (256x32 with 128-bit accesses when
+//                everything is a multiple of 4 elements, 64x64 dwords otherwise).
 //   ew_generic - anything else, one element per lane, div/mod index math with
 //                dimension 0 fastest.
 //

@@ -126,12 +126,24 @@ at::Tensor _copy_from_and_resize(const at::Tensor &self, const at::Tensor &dst) 
   return dst;
 }
 
+// t.item(), float(t), t.tolist(): one element travels to the host (a blocking
+// device->host copy of its bytes).  The reference has no registration for it, so
+// reading a scalar back from a webgpu tensor fails there.
+at::Scalar _local_scalar_dense(const at::Tensor &self) {
+  TORCH_CHECK(self.numel() == 1, "a Tensor with ", self.numel(),
+              " elements cannot be converted to Scalar");
+  at::Tensor host = at::empty({}, self.options().device(at::kCPU));
+  device_to_host(host, self.reshape({}));
+  return host.item();
+}
+
 }  // namespace ops
 
 TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
   m.impl("copy_", TORCH_FN(ops::copy_));
   m.impl("_copy_from", TORCH_FN(ops::_copy_from));
   m.impl("_copy_from_and_resize", TORCH_FN(ops::_copy_from_and_resize));
+  m.impl("_local_scalar_dense", TORCH_FN(ops::_local_scalar_dense));
 }
 
 }  // namespace torch_webgpu

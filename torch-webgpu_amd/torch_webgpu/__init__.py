@@ -32,4 +32,27 @@ torch.utils.generate_methods_for_privateuse1_backend(
     for_packed_sequence=True,
 )
 
+
+
+def _install_repr():
+    """Printing a tensor makes torch run a dozen ops on the tensor's own device
+    (isfinite, min, max, ceil, casts ...) unless it knows the backend; it moves
+    xla / lazy / ipu / mtia tensors to the host first (torch/_tensor_str.py) and a
+    renamed PrivateUse1 backend is not on that list.  Do the same for "webgpu": format
+    the host copy and name the real device in the result."""
+    original = torch.Tensor.__repr__
+
+    def __repr__(self, *, tensor_contents=None):
+        if tensor_contents is None and type(self) is torch.Tensor and self.device.type == "webgpu":
+            text = original(self.detach().to("cpu"))
+            if text.endswith(")"):
+                text = text[:-1] + ", device='" + str(self.device) + "')"
+            return text
+        return original(self, tensor_contents=tensor_contents)
+
+    torch.Tensor.__repr__ = __repr__
+
+
+_install_repr()
+
 __all__ = ["webgpu"]
