@@ -53,13 +53,25 @@ def test_allocator_caches_and_handles_zero(twg):
 
 def test_copy_round_trip_fp32_and_bool(twg):
     g = torch.Generator().manual_seed(1)
-    # 80 MiB crosses two 32 MiB staging chunks with a ragged tail
+    # 80 MiB wraps the ring of pinned staging slots several times, with a ragged tail
     for t in (torch.randn((80 << 20) // 4 + 3, generator=g),
               torch.rand(1000003, generator=g) < 0.5,
               torch.randn(5, generator=g)):
         buf = twg.to_device(t)
         back = buf.download(t.shape, t.dtype)
         assert bit_equal(back, t)
+    # large copies into and out of host ranges that start at odd addresses
+    raw = torch.randint(0, 256, ((40 << 20) + 77,), dtype=torch.uint8, generator=g)
+    L = twg.load()
+    for off in (1, 15, 16, 33):
+        nb = raw.numel() - off - 5
+        dev = twg.DeviceBuffer(nb)
+        twg.check(L.twg_memcpy_h2d(dev.ptr, raw.data_ptr() + off, nb, None))
+        back = torch.full((raw.numel(),), 0xEE, dtype=torch.uint8)
+        twg.check(L.twg_memcpy_d2h(back.data_ptr() + off, dev.ptr, nb, None))
+        assert torch.equal(back[off:off + nb], raw[off:off + nb])
+        assert bool((back[:off] == 0xEE).all()) and bool((back[off + nb:] == 0xEE).all())
+        dev.free()
     # device -> device and fill
     t = torch.randn(4097, generator=g)
     src = twg.to_device(t)

@@ -210,9 +210,19 @@ struct RowGeom {
   int64_t len;               // extent of dimension 0
   uint32_t chunks_per_row;   // blocks along one row
   int32_t nouter;            // remaining dimensions
+  uint32_t reused;           // bit k: operand k is the same row for every block (a bias)
   int64_t oshape[TWG_MAX_DIMS - 1];
   int64_t ostride[3][TWG_MAX_DIMS - 1];
 };
+
+// A row every block re-reads should stay in L2: streaming hints only for the rest.
+template <bool STREAM, typename P>
+__device__ __forceinline__ P load_row_pack(const P *p, bool reused) {
+  if constexpr (STREAM) {
+    if (!reused) return load_pack<true>(p);
+  }
+  return load_pack<false>(p);
+}
 
 template <int THREADS, int NIN, int VEC, int UNROLL, bool STREAM, bool A_BC, bool B_BC, typename Op,
           typename TO, typename TA, typename TB>
@@ -250,8 +260,10 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
   for (int u = 0; u < UNROLL; ++u) {
     const int64_t e = e0 + (int64_t)u * THREADS * VEC;
     if (e < g.len) {
-      if constexpr (!A_BC) va[u] = load_pack<STREAM>(reinterpret_cast<const PA *>(arow + e));
-      if constexpr (NIN == 2 && !B_BC) vb[u] = load_pack<STREAM>(reinterpret_cast<const PB *>(brow + e));
+      if constexpr (!A_BC)
+        va[u] = load_row_pack<STREAM>(reinterpret_cast<const PA *>(arow + e), g.reused & 2u);
+      if constexpr (NIN == 2 && !B_BC)
+        vb[u] = load_row_pack<STREAM>(reinterpret_cast<const PB *>(brow + e), g.reused & 4u);
     }
   }
 #pragma unroll
@@ -557,6 +569,11 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
   for (int d = 1; d < g.ndim; ++d) {
     rg.oshape[d - 1] = g.shape[d];
     for (int o = 0; o < 3; ++o) rg.ostride[o][d - 1] = g.stride[o][d];
+  }
+  for (int o = 1; o <= NIN; ++o) {
+    bool same_row = true;
+    for (int d = 1; d < g.ndim; ++d) same_row = same_row && g.stride[o][d] == 0;
+    if (same_row) rg.reused |= 1u << o;
   }
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
   if (stream)

@@ -6,6 +6,7 @@
 //   csrc/core/webgpu_allocator.cpp:10-55  one wgpu::Buffer per tensor storage
 //   csrc/ops/copy.cpp:12-62,74-122        WriteBuffer / CopyBufferToBuffer / MapAsync
 #include <hip/hip_runtime.h>
+#include <emmintrin.h>
 
 #include <atomic>
 #include <cstdio>
@@ -88,16 +89,49 @@ int release_cached_locked(Pool &p) {
 
 // ------------------------------------------------------------ staging ring
 
-constexpr size_t kStageBytes = size_t(32) << 20;
-constexpr int kStageSlots = 2;
+constexpr int kStageSlots = 8;
+constexpr size_t kStreamingDrainBytes = size_t(32) << 20;  // beyond what a last-level cache keeps
 
 struct Staging {
   std::mutex mu;
   bool ready = false;
-  void *buf[kStageSlots] = {nullptr, nullptr};
-  hipEvent_t ev[kStageSlots] = {nullptr, nullptr};
-  bool busy[kStageSlots] = {false, false};
+  // 2 MiB slots keep the ring in the CPU's last-level cache and let a 4 MiB copy
+  // already overlap its second half with the DMA of the first.
+  size_t chunk = size_t(2) << 20;
+  int slots = kStageSlots;
+  char *base = nullptr;            // one pinned allocation, slots * chunk bytes
+  hipEvent_t ev[kStageSlots] = {};
+  bool busy[kStageSlots] = {};
+  char *buf(int i) const { return base + (size_t)i * chunk; }
 };
+
+// Copy out of a staging slot into pageable memory.  Large destinations do not fit in
+// the CPU caches, and an ordinary store would first read each destination line from
+// DRAM; streaming stores skip that read.
+void drain_slot(char *dst, const char *src, size_t n, bool streaming) {
+  if (!streaming || n < 64) {
+    std::memcpy(dst, src, n);
+    return;
+  }
+  const size_t head = (16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15;
+  std::memcpy(dst, src, head);
+  dst += head;
+  src += head;
+  n -= head;
+  const size_t body = n & ~size_t(63);
+  for (size_t i = 0; i < body; i += 64) {
+    const __m128i v0 = _mm_loadu_si128(reinterpret_cast<const __m128i *>(src + i));
+    const __m128i v1 = _mm_loadu_si128(reinterpret_cast<const __m128i *>(src + i + 16));
+    const __m128i v2 = _mm_loadu_si128(reinterpret_cast<const __m128i *>(src + i + 32));
+    const __m128i v3 = _mm_loadu_si128(reinterpret_cast<const __m128i *>(src + i + 48));
+    _mm_stream_si128(reinterpret_cast<__m128i *>(dst + i), v0);
+    _mm_stream_si128(reinterpret_cast<__m128i *>(dst + i + 16), v1);
+    _mm_stream_si128(reinterpret_cast<__m128i *>(dst + i + 32), v2);
+    _mm_stream_si128(reinterpret_cast<__m128i *>(dst + i + 48), v3);
+  }
+  _mm_sfence();
+  std::memcpy(dst + body, src + body, n - body);
+}
 
 Staging &staging() {
   static Staging *s = new Staging;
@@ -106,10 +140,9 @@ Staging &staging() {
 
 int staging_prepare_locked(Staging &s) {
   if (s.ready) return 0;
-  for (int i = 0; i < kStageSlots; ++i) {
-    TWG_HIP_TRY(hipHostMalloc(&s.buf[i], kStageBytes, hipHostMallocDefault));
+  TWG_HIP_TRY(hipHostMalloc((void **)&s.base, s.chunk * s.slots, hipHostMallocDefault));
+  for (int i = 0; i < s.slots; ++i)
     TWG_HIP_TRY(hipEventCreateWithFlags(&s.ev[i], hipEventDisableTiming));
-  }
   s.ready = true;
   return 0;
 }
@@ -364,17 +397,17 @@ int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_strea
   size_t done = 0;
   int slot = 0;
   while (done < nbytes) {
-    size_t chunk = nbytes - done < kStageBytes ? nbytes - done : kStageBytes;
+    size_t chunk = nbytes - done < st.chunk ? nbytes - done : st.chunk;
     if (st.busy[slot]) {  // the DMA that last read this slot must have finished
       TWG_HIP_TRY(hipEventSynchronize(st.ev[slot]));
       st.busy[slot] = false;
     }
-    std::memcpy(st.buf[slot], src + done, chunk);
-    TWG_HIP_TRY(hipMemcpyAsync(dst + done, st.buf[slot], chunk, hipMemcpyHostToDevice, s));
+    std::memcpy(st.buf(slot), src + done, chunk);
+    TWG_HIP_TRY(hipMemcpyAsync(dst + done, st.buf(slot), chunk, hipMemcpyHostToDevice, s));
     TWG_HIP_TRY(hipEventRecord(st.ev[slot], s));
     st.busy[slot] = true;
     done += chunk;
-    slot = (slot + 1) % kStageSlots;
+    slot = (slot + 1) % st.slots;
   }
   return 0;  // the caller's host range is free again; the device side is stream ordered
 }
@@ -388,7 +421,7 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   Staging &st = staging();
   std::lock_guard<std::mutex> lk(st.mu);
   if ((rc = staging_prepare_locked(st))) return rc;
-  for (int i = 0; i < kStageSlots; ++i) {
+  for (int i = 0; i < st.slots; ++i) {
     if (st.busy[i]) {
       TWG_HIP_TRY(hipEventSynchronize(st.ev[i]));
       st.busy[i] = false;
@@ -396,24 +429,31 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   }
   char *dst = static_cast<char *>(dst_host);
   const char *src = static_cast<const char *>(src_dev);
-  const size_t nchunks = (nbytes + kStageBytes - 1) / kStageBytes;
+  const size_t nchunks = (nbytes + st.chunk - 1) / st.chunk;
   auto chunk_len = [&](size_t c) {
-    size_t off = c * kStageBytes;
-    return nbytes - off < kStageBytes ? nbytes - off : kStageBytes;
+    size_t off = c * st.chunk;
+    return nbytes - off < st.chunk ? nbytes - off : st.chunk;
   };
-  // Keep one DMA in flight while the CPU drains the previous chunk.
-  TWG_HIP_TRY(hipMemcpyAsync(st.buf[0], src, chunk_len(0), hipMemcpyDeviceToHost, s));
-  TWG_HIP_TRY(hipEventRecord(st.ev[0], s));
+  auto issue = [&](size_t c) -> int {
+    int slot = (int)(c % st.slots);
+    TWG_HIP_TRY(hipMemcpyAsync(st.buf(slot), src + c * st.chunk, chunk_len(c),
+                               hipMemcpyDeviceToHost, s));
+    TWG_HIP_TRY(hipEventRecord(st.ev[slot], s));
+    return 0;
+  };
+  const bool streaming = nbytes >= kStreamingDrainBytes;
+  // The DMA engine runs up to a ring ahead of the CPU draining the slots.
+  size_t issued = 0;
+  for (; issued < nchunks && issued < (size_t)st.slots; ++issued)
+    if ((rc = issue(issued))) return rc;
   for (size_t c = 0; c < nchunks; ++c) {
-    int slot = (int)(c % kStageSlots);
-    if (c + 1 < nchunks) {
-      int nslot = (int)((c + 1) % kStageSlots);
-      TWG_HIP_TRY(hipMemcpyAsync(st.buf[nslot], src + (c + 1) * kStageBytes, chunk_len(c + 1),
-                                 hipMemcpyDeviceToHost, s));
-      TWG_HIP_TRY(hipEventRecord(st.ev[nslot], s));
-    }
+    int slot = (int)(c % st.slots);
     TWG_HIP_TRY(hipEventSynchronize(st.ev[slot]));
-    std::memcpy(dst + c * kStageBytes, st.buf[slot], chunk_len(c));
+    drain_slot(dst + c * st.chunk, st.buf(slot), chunk_len(c), streaming);
+    if (issued < nchunks) {
+      if ((rc = issue(issued))) return rc;
+      ++issued;
+    }
   }
   return 0;
 }
