@@ -86,8 +86,9 @@ def add(a, b, alpha=1.0, out=None):
     return binary("twg_add_f32", a, b, out=out, extra=(ctypes.c_float(alpha),))
 
 
-def masked_select(x, mask, scratch_bytes=None):
-    """Returns (values, count) from twg_masked_select_f32."""
+def masked_select(x, mask, scratch_bytes=None, out_offset=0):
+    """Returns (values, count) from twg_masked_select_f32.  out_offset (in floats)
+    shifts the output pointer off its 128-byte alignment."""
     L = capi.load()
     shape = torch.broadcast_shapes(x.shape, mask.shape)
     xe, me = _expanded(shape, x, mask)
@@ -95,15 +96,16 @@ def masked_select(x, mask, scratch_bytes=None):
     for s in shape:
         n *= s
     ux, um = Uploaded(x), Uploaded(mask)
-    out = capi.DeviceBuffer(max(4 * n, 4))
+    out = capi.DeviceBuffer(max(4 * n, 4) + 4 * out_offset)
     cnt = capi.DeviceBuffer(8)
     need = L.twg_masked_select_scratch_bytes(n)
     scratch = capi.DeviceBuffer(need if scratch_bytes is None else max(scratch_bytes, 8))
     it = _iter_for(shape, None, (xe, me), sort_by_out=False)
-    rc = L.twg_masked_select_f32(out.ptr, cnt.ptr, ux.ptr, um.ptr, ctypes.byref(it),
+    rc = L.twg_masked_select_f32(out.ptr + 4 * out_offset, cnt.ptr, ux.ptr, um.ptr, ctypes.byref(it),
                                  scratch.ptr, scratch.nbytes if scratch_bytes is None else scratch_bytes,
                                  None)
     capi.check(rc)
     k = int(cnt.download((1,), torch.int64)[0])
-    vals = out.download((k,), torch.float32) if k else torch.empty(0, dtype=torch.float32)
+    vals = (out.download((k,), torch.float32, byte_offset=4 * out_offset) if k
+            else torch.empty(0, dtype=torch.float32))
     return vals, k

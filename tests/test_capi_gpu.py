@@ -351,14 +351,15 @@ def test_masked_select_bernoulli(twg, n, p):
     assert bit_equal(vals, torch.masked_select(x, m))
 
 
-@pytest.mark.parametrize("n,p", [(1 << 24, 0.5), ((1 << 24) + 3 * 65536 + 12345, 0.5),
-                                 ((1 << 24) + 5, 0.99), ((1 << 25) + 8191, 0.01),
-                                 ((1 << 24) + 70000, 1.0), ((1 << 24) + 70000, 0.0),
-                                 ((1 << 24) + 40000, -1.0)])
-def test_masked_select_large_tiles(twg, n, p):
-    # >= 2^24 elements take the 65536-element-tile kernel; a remainder below one big
-    # tile goes to a second launch that continues from the first one's count
-    _say(f"masked_select large n={n} p={p}")
+@pytest.mark.parametrize("n,p,out_offset", [
+    (1 << 25, 0.5, 0), ((1 << 25) + 3 * 131072 + 12345, 0.5, 1), ((1 << 25) + 5, 0.99, 31),
+    ((1 << 25) + 8191, 0.01, 0), ((1 << 25) + 8191, 0.001, 7), ((1 << 25) + 140000, 1.0, 3),
+    ((1 << 25) + 140000, 0.0, 0), ((1 << 25) + 40000, -1.0, 17), ((1 << 24) + 70000, 0.5, 0)])
+def test_masked_select_large_tiles(twg, n, p, out_offset):
+    # >= 2^25 elements take the streaming kernel with 131072-element tiles; a remainder
+    # below one big tile goes to a second launch that continues from the first one's
+    # count.  A shifted output pointer moves every wavefront's first and last line.
+    _say(f"masked_select large n={n} p={p} out_offset={out_offset}")
     x = W.select_source(n, seed=4)
     if p < 0:
         m = W.clustered_mask(n, mean_run=4096, seed=6)
@@ -366,7 +367,7 @@ def test_masked_select_large_tiles(twg, n, p):
         m = W.bernoulli_mask(n, p, seed=11)
     else:
         m = torch.full((n,), p == 1.0)
-    vals, k = H.masked_select(x, m)
+    vals, k = H.masked_select(x, m, out_offset=out_offset)
     assert k == int(m.sum())
     assert bit_equal(vals, torch.masked_select(x, m))
 

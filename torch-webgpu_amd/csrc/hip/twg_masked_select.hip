@@ -22,14 +22,15 @@
 // load/store carries everything; no fences are needed because no other memory
 // is communicated between tiles.
 //
-// Two facts about MI355X shape the large-input variant.  Same-address agent-scope
+// Three facts about MI355X shape the large-input variant.  Same-address agent-scope
 // atomics retire at about one per 7 ns, so the ticket must not be paid 32768
-// times for 2^28 elements; and with one 1024-lane workgroup per CU the latency of
-// ticket -> mask -> look-back is only amortised by giving each workgroup a lot of
-// data.  Its tiles are therefore 65536 elements, walked as 2 sub-tiles in a rolled
-// loop; between sub-tiles only the packed selection bits (one register per 8
-// steps) stay live, and the next sub-tile's values are already in flight while the
-// current one is written out.
+// times for 2^28 elements: its tiles are 131072 elements.  A wavefront that mixes
+// loads and stores in a loop only keeps its loads in flight if the compiler can
+// count them, so its loads are unconditional (a lane with nothing selected reads
+// one shared dummy address).  And stores that leave partial 128-byte lines behind
+// cost HBM write efficiency, so each wavefront compacts through a small LDS ring
+// and writes whole aligned lines as soon as they are complete; only the first and
+// last line of a wavefront's run go out element by element.
 #include <hip/hip_runtime.h>
 
 #include "twg_internal.h"
@@ -168,33 +169,152 @@ __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, 
   return *s_slot;
 }
 
-// ------------------------------------------------------------------ fast variant
-// Dense source and mask, 16-byte aligned source, 4-byte aligned mask.
-// A tile is SUB sub-tiles; in each, wavefront w owns 8 steps of 256 elements
-// (lane l, step k: elements 4l..4l+3 of that step).
-//
-// RAGGED = false: the host guarantees that every tile of the launch is full, so the
-// kernel carries no bounds-checked code (a checked instance would set the register
-// budget of the whole kernel although at most one tile ever runs it).
+// ------------------------------------------------------------------ fast variants
+// Dense source and mask, 16-byte aligned source, 4-byte aligned mask.  Lane l of a
+// wavefront owns elements 4l..4l+3 of each 256-element step.
 
-template <int WAVES, int SUB>
+// ---- streaming variant: full tiles only (the host launches it on a multiple of the
+// tile size, so it carries no bounds checks).  Wavefront w owns GROUPS * 8
+// consecutive steps of the tile.
+constexpr int kRingElems = 512;  // per wavefront; at most 31 + 256 values wait in it
+
+template <int WAVES, int GROUPS>
+struct MsStreamShared {
+  uint32_t tile;
+  uint32_t wave_total[WAVES];
+  int64_t base;
+  uint32_t bits[GROUPS][WAVES * 64];  // 4 selection bits per step, 8 steps per word
+  __attribute__((aligned(16))) float ring[WAVES][kRingElems];
+};
+
+template <int WAVES, int GROUPS>
+__global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int64_t *d_count,
+                                                                const float *src,
+                                                                const uint8_t *mask,
+                                                                uint32_t ntiles, uint32_t *ticket,
+                                                                uint64_t *status) {
+  constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
+  constexpr int64_t kTileElems = (int64_t)kWaveSpan * WAVES;
+  __shared__ MsStreamShared<WAVES, GROUPS> sh;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0)
+    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const uint32_t tile = sh.tile;
+  const int64_t start = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
+  const uint8_t *mask_w = mask + start + lane * 4;
+  const float *src_w = src + start + lane * 4;
+
+  // ---- 1. masks -> packed selection bits in LDS, wavefront totals
+  uint32_t cnt = 0;
+#pragma unroll 2
+  for (int g = 0; g < GROUPS; ++g) {
+    uint32_t w[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      w[k] = __builtin_nontemporal_load(
+          reinterpret_cast<const uint32_t *>(mask_w + (g * 8 + k) * 256));
+    uint32_t b = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) b |= select_bits(w[k]) << (4 * k);
+    sh.bits[g][threadIdx.x] = b;
+    cnt += __popc(b);
+  }
+  const uint32_t wt = wave_sum_u32(cnt);
+  if (lane == 0) sh.wave_total[wave] = wt;
+  __syncthreads();
+  uint32_t wbase = 0, tile_total = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const uint32_t t = sh.wave_total[w];
+    if ((uint32_t)w < wave) wbase += t;
+    tile_total += t;
+  }
+
+  // ---- 2. the first 8 steps' values go in flight, then aggregate / look-back
+  const f32x4 *dummy = reinterpret_cast<const f32x4 *>(src + (int64_t)tile * kTileElems);
+  auto fetch = [&](uint32_t b, int g, int k) {
+    const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + (g * 8 + k) * 256);
+    return __builtin_nontemporal_load(((b >> (4 * k)) & 0xFu) ? p : dummy);
+  };
+  uint32_t b_cur = sh.bits[0][threadIdx.x];
+  f32x4 vals[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) vals[k] = fetch(b_cur, 0, k);
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
+
+  // ---- 3. stream: compact a step into the ring, refill its register for 8 steps
+  //         later, write out the lines the step completed.  Position p of this
+  //         wavefront's run is obase[p] in memory and ring[p % kRingElems] in LDS.
+  float *ring = sh.ring[wave];
+  float *wout = out + (base + wbase);
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 31u);
+  float *obase = wout - shift;         // 128-byte aligned
+  uint32_t run = shift;                // next free position
+  uint32_t flushed = shift ? 8u : 0u;  // float4 slots written; a shifted first line is not ours alone
+#pragma unroll 1
+  for (int g = 0; g < GROUPS; ++g) {
+    const int gn = (g + 1 < GROUPS) ? g + 1 : g;  // past the end: all lanes read the dummy
+    const uint32_t b_next = (g + 1 < GROUPS) ? sh.bits[gn][threadIdx.x] : 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t f = (b_cur >> (4 * k)) & 0xFu;
+      uint32_t below, total;
+      wave_offsets(__popc(f), below, total);
+      const f32x4 x4 = vals[k];
+      vals[k] = fetch(b_next, gn, k);
+      if (f) {
+        uint32_t pos = run + below;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (f & (1u << j)) {
+            const float x = x4[j];
+            ring[pos & (kRingElems - 1)] = x;
+            if (pos < 32u && shift) obase[pos] = x;  // shared first line: element by element
+            ++pos;
+          }
+        }
+      }
+      run += total;
+      const uint32_t end4 = (run >> 5) << 3;  // whole 128-byte lines only
+      if (end4 > flushed) {                   // wavefront-uniform
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t idx = flushed + lane; idx < end4; idx += 64) {
+          const f32x4 x =
+              *reinterpret_cast<const f32x4 *>(ring + ((4 * idx) & (kRingElems - 1)));
+          __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * (size_t)idx));
+        }
+        flushed = end4;
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+    b_cur = b_next;
+  }
+  // the last, incomplete line (its other elements belong to the next wavefront)
+  const uint32_t p = 4 * flushed + lane;
+  if (lane < 32 && p < run) obase[p] = ring[p & (kRingElems - 1)];
+}
+
+// ---- tile variant: any length.  One pass of 8 steps per wavefront, compacted in LDS at
+// the 16-byte phase the values will have in memory and written as aligned float4s.
+template <int WAVES>
 struct MsShared {
   uint32_t tile;
-  uint32_t wave_total[SUB][WAVES];
+  uint32_t wave_total[WAVES];
   int64_t base;
   __attribute__((aligned(16))) float stage[WAVES][kWaveElems + 4];
 };
 
-template <int WAVES, int SUB, bool RAGGED>
+template <int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t *d_count,
                                                              const float *src,
                                                              const uint8_t *mask, int64_t n,
                                                              uint32_t ntiles, uint32_t *ticket,
                                                              uint64_t *status,
                                                              const int64_t *carry_in) {
-  constexpr uint32_t kSubElems = (uint32_t)kWaveElems * WAVES;
-  constexpr int64_t kTileElems = (int64_t)kSubElems * SUB;
-  __shared__ MsShared<WAVES, SUB> sh;
+  constexpr int64_t kTileElems = (int64_t)kWaveElems * WAVES;
+  __shared__ MsShared<WAVES> sh;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
   if (threadIdx.x == 0)
@@ -210,116 +330,84 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t
   const uint32_t remaining = left < kTileElems ? (uint32_t)left : (uint32_t)kTileElems;
   if (carry_in) out += *carry_in;
 
-  // ---- 1. the whole tile's mask -> packed selection bits and wavefront totals
-  uint32_t bits[SUB];  // 4 bits per step: bit 4k+j <=> element j of step k is selected
+  // ---- 1. mask -> packed selection bits (bit 4k+j <=> element j of step k) and totals
+  uint32_t w[kSteps];
 #pragma unroll
-  for (int s = 0; s < SUB; ++s) {
-    uint32_t w[kSteps];
-#pragma unroll
-    for (int k = 0; k < kSteps; ++k) {  // all 8 loads in flight before any is used
-      const uint32_t e = lane_off + s * kSubElems + k * 256;
-      if (!RAGGED || e + 4 <= remaining) {
-        w[k] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(mask_tile + e));
-      } else {
-        w[k] = 0;
-        for (uint32_t j = 0; j < 4; ++j)
-          if (e + j < remaining && mask_tile[e + j]) w[k] |= 1u << (8 * j);
-      }
+  for (int k = 0; k < kSteps; ++k) {  // all 8 loads in flight before any is used
+    const uint32_t e = lane_off + k * 256;
+    if (e + 4 <= remaining) {
+      w[k] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(mask_tile + e));
+    } else {
+      w[k] = 0;
+      for (uint32_t j = 0; j < 4; ++j)
+        if (e + j < remaining && mask_tile[e + j]) w[k] |= 1u << (8 * j);
     }
-    uint32_t b = 0;
-#pragma unroll
-    for (int k = 0; k < kSteps; ++k) b |= select_bits(w[k]) << (4 * k);
-    bits[s] = b;
-    const uint32_t wt = wave_sum_u32(__popc(b));
-    if (lane == 0) sh.wave_total[s][wave] = wt;
   }
+  uint32_t bits = 0;
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) bits |= select_bits(w[k]) << (4 * k);
+  const uint32_t wt = wave_sum_u32(__popc(bits));
+  if (lane == 0) sh.wave_total[wave] = wt;
   __syncthreads();
-  uint32_t wbase[SUB];  // offset of this wavefront's part of sub-tile s from the tile's start
-  uint32_t wtot[SUB];
-  uint32_t tile_total = 0;
+  uint32_t wbase = 0, tile_total = 0;
 #pragma unroll
-  for (int s = 0; s < SUB; ++s) {
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      const uint32_t t = sh.wave_total[s][w];
-      if ((uint32_t)w == wave) {
-        wbase[s] = tile_total;
-        wtot[s] = t;
-      }
-      tile_total += t;
-    }
+  for (int v = 0; v < WAVES; ++v) {
+    const uint32_t t = sh.wave_total[v];
+    if ((uint32_t)v < wave) wbase += t;
+    tile_total += t;
   }
 
-  // ---- 2. source values of sub-tile 0 go in flight, then aggregate / look-back
+  // ---- 2. source values go in flight, then aggregate / look-back
   f32x4 vals[kSteps];
-  auto fetch = [&](uint32_t b, uint32_t sub_off) {
 #pragma unroll
-    for (int k = 0; k < kSteps; ++k) {
-      if ((b >> (4 * k)) & 0xFu) {
-        const uint32_t e = lane_off + sub_off + k * 256;
-        if (!RAGGED || e + 4 <= remaining) {
-          vals[k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src_tile + e));
-        } else {
-          for (uint32_t j = 0; j < 4; ++j) vals[k][j] = (e + j < remaining) ? src_tile[e + j] : 0.0f;
-        }
+  for (int k = 0; k < kSteps; ++k) {
+    if ((bits >> (4 * k)) & 0xFu) {
+      const uint32_t e = lane_off + k * 256;
+      if (e + 4 <= remaining) {
+        vals[k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src_tile + e));
+      } else {
+        for (uint32_t j = 0; j < 4; ++j) vals[k][j] = (e + j < remaining) ? src_tile[e + j] : 0.0f;
       }
     }
-  };
-  fetch(bits[0], 0);
+  }
   const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, carry_in);
 
-  // ---- 3. per sub-tile (rolled loop): compact in LDS at the output's 16-byte phase,
-  //         start the next sub-tile's loads, write aligned float4s.  The ragged ends
-  //         go out element by element: their neighbours belong to other wavefronts.
+  // ---- 3. compact in LDS, write aligned float4s; the ragged ends go out element by
+  //         element: their neighbours belong to other wavefronts.
   float *stage = sh.stage[wave];
-#pragma unroll 1
-  for (int s = 0; s < SUB; ++s) {
-    uint32_t b = bits[0], wb = wbase[0], wt = wtot[0], b_next = 0;
+  float *wout = out + (base + wbase);  // this wavefront's first output value
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 3u);
+  uint32_t run = shift;
 #pragma unroll
-    for (int q = 1; q < SUB; ++q) {  // register arrays indexed by a loop-carried s
-      if (s == q) {
-        b = bits[q];
-        wb = wbase[q];
-        wt = wtot[q];
+  for (int k = 0; k < kSteps; ++k) {
+    const uint32_t f = (bits >> (4 * k)) & 0xFu;
+    uint32_t below, total;
+    wave_offsets(__popc(f), below, total);
+    if (f) {
+      uint32_t pos = run + below;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (f & (1u << j)) stage[pos++] = vals[k][j];
       }
-      if (s + 1 == q) b_next = bits[q];
     }
-    float *wout = out + (base + wb);  // this wavefront's first output value
-    const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 3u);
-    uint32_t run = shift;
+    run += total;
+  }
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t span_end = shift + wt;
+  float *obase = wout - shift;  // 16-byte aligned
+  if (wt != 0) {
+    for (uint32_t v = lane; 4 * v < span_end; v += 64) {
+      const f32x4 x = *reinterpret_cast<const f32x4 *>(stage + 4 * v);
+      if (4 * v >= shift && 4 * v + 4 <= span_end) {
+        __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * v));
+      } else {
 #pragma unroll
-    for (int k = 0; k < kSteps; ++k) {
-      const uint32_t f = (b >> (4 * k)) & 0xFu;
-      uint32_t below, total;
-      wave_offsets(__popc(f), below, total);
-      if (f) {
-        uint32_t pos = run + below;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (f & (1u << j)) stage[pos++] = vals[k][j];
-        }
-      }
-      run += total;
-    }
-    __builtin_amdgcn_wave_barrier();
-    if (s + 1 < SUB) fetch(b_next, (s + 1) * kSubElems);
-    const uint32_t span_end = shift + wt;
-    float *obase = wout - shift;  // 16-byte aligned
-    if (wt != 0) {
-      for (uint32_t v = lane; 4 * v < span_end; v += 64) {
-        const f32x4 x = *reinterpret_cast<const f32x4 *>(stage + 4 * v);
-        if (4 * v >= shift && 4 * v + 4 <= span_end) {
-          __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * v));
-        } else {
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const uint32_t i = 4 * v + c;
-            if (i >= shift && i < span_end) obase[i] = x[c];
-          }
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t i = 4 * v + c;
+          if (i >= shift && i < span_end) obase[i] = x[c];
         }
       }
     }
-    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -396,13 +484,14 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     if (sel[k]) out[wpos + loff[k]] = vals[k];
 }
 
-// Tile shapes of the fast variant: 65536-element tiles (1024 lanes, 2 sub-tiles)
-// once there is one per CU, 8192-element tiles (256 lanes) below that.
-constexpr int kBigWaves = 16, kBigSub = 2;
-constexpr int kSmallWaves = 4, kSmallSub = 1;
-constexpr int64_t kBigTile = (int64_t)kWaveElems * kBigWaves * kBigSub;
-constexpr int64_t kSmallTile = (int64_t)kWaveElems * kSmallWaves * kSmallSub;
-constexpr int64_t kBigMinElems = kBigTile * 256;  // 2^24
+// Tile shapes of the fast variants: 131072-element tiles (1024 lanes, 32 steps per
+// wavefront) once there is one per CU, 8192-element tiles (256 lanes) below that and
+// for what the big tiles leave over.
+constexpr int kBigWaves = 16, kBigGroups = 4;
+constexpr int kSmallWaves = 4;
+constexpr int64_t kBigTile = (int64_t)256 * 8 * kBigGroups * kBigWaves;
+constexpr int64_t kSmallTile = (int64_t)kWaveElems * kSmallWaves;
+constexpr int64_t kBigMinElems = kBigTile * 256;  // 2^25
 
 }  // namespace
 }  // namespace twg
@@ -451,8 +540,8 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
   auto tiles_of = [](int64_t n, int64_t tile) { return (n + tile - 1) / tile; };
 
   if (big) {
-    // Full 65536-element tiles go through the check-free kernel; what is left (less
-    // than one big tile) is compacted by a second launch of the small variant that
+    // Full 131072-element tiles go through the streaming kernel; what is left (less
+    // than one big tile) is compacted by a second launch of the tile variant that
     // starts from the first launch's total.
     const int64_t nbig = g.numel / kBigTile;
     const int64_t rem = g.numel - nbig * kBigTile;
@@ -461,11 +550,10 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
     if ((rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (size_t)(nbig + nrem),
                              stream)))
       return rc;
-    ms_compact_vec<kBigWaves, kBigSub, false><<<(unsigned)nbig, kBigWaves * 64, 0, s>>>(
-        out, rem ? carry : d_count, src, mask, nbig * kBigTile, (uint32_t)nbig, ticket, status,
-        nullptr);
+    ms_compact_stream<kBigWaves, kBigGroups><<<(unsigned)nbig, kBigWaves * 64, 0, s>>>(
+        out, rem ? carry : d_count, src, mask, (uint32_t)nbig, ticket, status);
     if (rem)
-      ms_compact_vec<kSmallWaves, kSmallSub, true><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
+      ms_compact_vec<kSmallWaves><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
           out, d_count, src + nbig * kBigTile, mask + nbig * kBigTile, rem, (uint32_t)nrem,
           ticket + 1, status + nbig, carry);
     return (int)hipGetLastError();
@@ -479,7 +567,7 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
     return rc;
 
   if (vec4) {
-    ms_compact_vec<kSmallWaves, kSmallSub, true><<<ntiles, kSmallWaves * 64, 0, s>>>(
+    ms_compact_vec<kSmallWaves><<<ntiles, kSmallWaves * 64, 0, s>>>(
         out, d_count, src, mask, g.numel, ntiles, ticket, status, nullptr);
   } else {
     MsGeom mg{};
