@@ -177,6 +177,10 @@ __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, 
 // tile size, so it carries no bounds checks).  Wavefront w owns GROUPS * 8
 // consecutive steps of the tile.
 constexpr int kRingElems = 512;  // per wavefront; at most 31 + 256 values wait in it
+// Source steps in flight per wavefront.  4 measured best: 8 keeps more in flight than
+// the memory system rewards (dense masks lose 2-3%), and below ~64 VGPRs a second
+// 1024-lane workgroup becomes resident per CU, which costs dense masks 5-10%.
+constexpr int kDepth = 4;
 
 template <int WAVES, int GROUPS>
 struct MsStreamShared {
@@ -232,19 +236,19 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
     tile_total += t;
   }
 
-  // ---- 2. the first 8 steps' values go in flight, then aggregate / look-back
+  // ---- 2. the first kDepth steps' values go in flight, then aggregate / look-back
   const f32x4 *dummy = reinterpret_cast<const f32x4 *>(src + (int64_t)tile * kTileElems);
-  auto fetch = [&](uint32_t b, int g, int k) {
-    const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + (g * 8 + k) * 256);
-    return __builtin_nontemporal_load(((b >> (4 * k)) & 0xFu) ? p : dummy);
+  auto fetch = [&](uint32_t four_bits, int step) {
+    const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + step * 256);
+    return __builtin_nontemporal_load(four_bits ? p : dummy);
   };
   uint32_t b_cur = sh.bits[0][threadIdx.x];
-  f32x4 vals[8];
+  f32x4 vals[kDepth];
 #pragma unroll
-  for (int k = 0; k < 8; ++k) vals[k] = fetch(b_cur, 0, k);
+  for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
   const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
 
-  // ---- 3. stream: compact a step into the ring, refill its register for 8 steps
+  // ---- 3. stream: compact a step into the ring, refill its register for kDepth steps
   //         later, write out the lines the step completed.  Position p of this
   //         wavefront's run is obase[p] in memory and ring[p % kRingElems] in LDS.
   float *ring = sh.ring[wave];
@@ -262,8 +266,12 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
       const uint32_t f = (b_cur >> (4 * k)) & 0xFu;
       uint32_t below, total;
       wave_offsets(__popc(f), below, total);
-      const f32x4 x4 = vals[k];
-      vals[k] = fetch(b_next, gn, k);
+      const f32x4 x4 = vals[k % kDepth];
+      {
+        const int ahead = k + kDepth;  // the step to prefetch, counted from this group's first
+        vals[k % kDepth] = ahead < 8 ? fetch((b_cur >> (4 * ahead)) & 0xFu, g * 8 + ahead)
+                                     : fetch((b_next >> (4 * (ahead - 8))) & 0xFu, gn * 8 + ahead - 8);
+      }
       if (f) {
         uint32_t pos = run + below;
 #pragma unroll
