@@ -169,7 +169,7 @@ def main():
     head = [
         summarize("add", "ew_contig<AddOp>", bytes_add, add_ms, n),
         summarize("gelu", "ew_contig<GeluErfOp>", bytes_gelu, gelu_ms, n),
-        summarize("masked_select_p0.50", "ms_compact_vec<16,2>", bytes_ms, msk_ms, n,
+        summarize("masked_select_p0.50", "ms_compact_stream<16,4>", bytes_ms, msk_ms, n,
                   {"selected": k50, "op_ms_with_count_readback": round(sum(mso_ms) / K, 5)}),
     ]
     ops += head
@@ -210,6 +210,11 @@ def main():
                              d_out, d_cnt, d_scratch, scratch_bytes, d_src, d_x, it, cnt_host, want)
     ops += result_sweep
 
+    # ------------------------------------------------------------ config 1: small add + transfers
+    small = None
+    if not args.no_sweep and want("config1"):
+        small = config1(capi, W, L, torch, time_launches, Wm, K)
+
     # ------------------------------------------------------------ CPU baselines
     cpu = None
     if not args.no_cpu:
@@ -228,6 +233,7 @@ def main():
         "pct_hbm_peak": round(value / HBM_PEAK_GBS * 100, 2),
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "config1_small_add_and_transfers": small,
         "ops": ops,
         "device": {"name": dev_name, "compute_units": cus},
     }
@@ -314,11 +320,43 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         ms_full = time_launches(full, 1, K)
         if int(cnt_host[0]) != k:
             raise RuntimeError(f"{name}: count {int(cnt_host[0])} != {k}")
-        res.append(summarize(name, "ms_compact_vec<16,2>", W.masked_select_bytes(n, k), ms_kernel, n,
+        res.append(summarize(name, "ms_compact_stream<16,4>", W.masked_select_bytes(n, k), ms_kernel, n,
                              {"selected": k,
                               "op_ms_with_count_readback": round(sum(ms_full) / len(ms_full), 5)}))
         del d_mask
     return res
+
+
+def config1(capi, W, L, torch, time_launches, Wm, K):
+    """The 2^20-element add with its copies up and down: too small for an HBM figure (it
+    fits the caches), so it is reported as launch latency and host-link rates."""
+    n1 = 1 << 20
+    a_h, b_h = W.add_contiguous(n1, seed=0)
+    d_a, d_b, d_o = capi.to_device(a_h), capi.to_device(b_h), capi.DeviceBuffer(4 * n1)
+    it1 = capi.dense_iter(n1)
+    ms = time_launches(lambda: capi.check(L.twg_add_f32(d_o.ptr, d_a.ptr, d_b.ptr, ctypes.c_float(1.0),
+                                                        ctypes.byref(it1), None)), Wm, K)
+    back = torch.empty(n1)
+    reps = 20
+
+    def wall(fn):
+        capi.sync()
+        t = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        capi.sync()
+        return (time.perf_counter() - t) / reps
+
+    t_up = wall(lambda: d_a.upload(a_h))
+    t_down = wall(lambda: capi.check(L.twg_memcpy_d2h(back.data_ptr(), d_o.ptr, 4 * n1, None)))
+    if not torch.equal(back, a_h + b_h):
+        raise RuntimeError("config 1: add result differs from the CPU sum")
+    d = {"elements": n1, "add_kernel_us": round(statistics.median(ms) * 1e3, 2),
+         "h2d_4MiB_us": round(t_up * 1e6, 1), "h2d_GBps": round(4 * n1 / t_up / 1e9, 2),
+         "d2h_4MiB_us": round(t_down * 1e6, 1), "d2h_GBps": round(4 * n1 / t_down / 1e9, 2),
+         "note": "pageable host memory through the pinned staging ring; result equals the CPU sum"}
+    log(f"  config 1 (2^20): add {d['add_kernel_us']} us, H2D {d['h2d_GBps']} GB/s, D2H {d['d2h_GBps']} GB/s")
+    return d
 
 
 def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu, bytes_ms):
@@ -371,6 +409,17 @@ def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu
     tm = best(lambda: torch.masked_select(st, mt), 5)
     kt = int(mt.sum())
     ga, gg, gm = 12 * nt / ta / 1e9, 8 * nt / tg / 1e9, (5 * nt + 4 * kt) / tm / 1e9
+    # the other ops of the sweep, same inputs as the GPU side, same bytes-per-element figures
+    others = {}
+    others["silu_GBps"] = round(8 * nt / best(lambda: F.silu(xt)) / 1e9, 2)
+    others["relu_GBps"] = round(8 * nt / best(lambda: torch.relu(xt)) / 1e9, 2)
+    del a, b, o
+    p_h, q_h, z_h = W.mask_inputs(nt, seed=3)
+    others["eq_GBps"] = round(9 * nt / best(lambda: torch.eq(p_h, q_h)) / 1e9, 2)
+    others["ne_scalar_GBps"] = round(5 * nt / best(lambda: z_h.ne(0.0)) / 1e9, 2)
+    m1, m2 = torch.eq(p_h, q_h), z_h.ne(0.0)
+    others["bitwise_and_GBps"] = round(3 * nt / best(lambda: torch.bitwise_and(m1, m2)) / 1e9, 2)
+    del p_h, q_h, z_h, m1, m2
     step_t = bytes_add / ga / 1e9 + bytes_gelu / gg / 1e9 + bytes_ms / gm / 1e9
     try:
         with open("/proc/cpuinfo") as f:
@@ -388,8 +437,8 @@ def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu
             "cpu_model": model,
             "sample": f"torch.add / F.gelu / torch.masked_select on 2^{nt.bit_length() - 1} elements, "
                       "median of 5 (ATen's CPU kernel is the reference's own masked_select)",
-            "per_op": {"add_GBps": round(ga, 2), "gelu_GBps": round(gg, 2),
-                       "masked_select_GBps": round(gm, 2)},
+            "per_op": dict({"add_GBps": round(ga, 2), "gelu_GBps": round(gg, 2),
+                            "masked_select_GBps": round(gm, 2)}, **others),
         },
     }
 
