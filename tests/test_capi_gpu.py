@@ -191,6 +191,51 @@ def test_add_generic_strides_bruteforce(twg):
     assert bit_equal(H.add(a8, b8), a8 + b8)
 
 
+def _random_view(g, shape, rng):
+    """A tensor of logical `shape` with random memory layout: permuted dimensions,
+    stepped slices, a storage offset of 0..3 elements."""
+    nd = len(shape)
+    perm = rng.sample(range(nd), nd)
+    steps = [rng.choice((1, 1, 1, 2, 3)) for _ in range(nd)]
+    phys = [shape[perm[i]] * steps[perm[i]] for i in range(nd)]
+    off = rng.randrange(4)
+    numel = 1
+    for e in phys:
+        numel *= e
+    base = torch.randint(-8, 8, (numel + off,), generator=g).float()[off:].view(*phys)
+    inv = [perm.index(d) for d in range(nd)]
+    t = base.permute(*inv)
+    return t[tuple(slice(None, None, steps[d]) for d in range(nd))]
+
+
+def test_random_geometries(twg):
+    # 120 seeded layouts: every dispatch path of the elementwise launcher (contiguous,
+    # rows with broadcast operands, LDS tiles, 128-bit tiles, div/mod) and the strided
+    # masked_select, against ATen's CPU kernels on the very same views
+    import random
+    rng = random.Random(1234)
+    g = torch.Generator().manual_seed(77)
+    extents = (1, 2, 3, 4, 5, 8, 16, 63, 64, 65, 128, 260)
+    for case in range(120):
+        nd = rng.randint(1, 5)
+        shape = [rng.choice(extents) for _ in range(nd)]
+        while torch.Size(shape).numel() > (1 << 18):
+            shape[rng.randrange(nd)] = rng.choice(extents[:6])
+        bshape = [1 if rng.random() < 0.3 else e for e in shape]
+        ashape = list(shape) if rng.random() < 0.8 else [1 if rng.random() < 0.3 else e for e in shape]
+        a, b = _random_view(g, ashape, rng), _random_view(g, bshape, rng)
+        _say(f"geometry {case}: a {tuple(a.shape)}/{a.stride()} b {tuple(b.shape)}/{b.stride()}")
+        assert bit_equal(H.add(a, b), a + b)
+        out = _random_view(g, list(torch.broadcast_shapes(a.shape, b.shape)), rng)
+        assert bit_equal(H.add(a, b, alpha=-2.0, out=out), a + b * -2.0)  # small integers: exact
+        eq = H.binary("twg_eq_f32", a, b, out_dtype=torch.bool)
+        assert torch.equal(eq, torch.eq(a, b))
+        if case % 3 == 0:
+            vals, k = H.masked_select(a, torch.eq(a, b))
+            ref = torch.masked_select(a, torch.eq(a, b))
+            assert k == ref.numel() and bit_equal(vals, ref)
+
+
 def test_mul_and_fused_add_relu(twg):
     g = torch.Generator().manual_seed(6)
     a = torch.randn(70001, generator=g)

@@ -357,3 +357,41 @@ def test_masked_select_semantics():
     assert torch.equal(torch.masked_select(t, t.ne(0)).to("cpu"), torch.tensor([1.5, -2.0]))
     assert torch.equal(torch.masked_select(t, torch.eq(t, t) & t.ne(0)).to("cpu"),
                        torch.tensor([1.5, -2.0]))
+
+
+def test_random_views_through_the_dispatcher():
+    # Seeded random layouts built ON the device with the same view calls as on the CPU
+    # (permute, stepped slices, expand): as_strided, at::TensorIterator's reordering and
+    # merging, and every kernel family behind add / eq / masked_select must agree with ATen.
+    import random
+    rng = random.Random(4321)
+    g = torch.Generator().manual_seed(99)
+    extents = (1, 2, 3, 4, 5, 8, 16, 63, 64, 65, 128, 260)
+
+    def make(shape):
+        nd = len(shape)
+        perm = rng.sample(range(nd), nd)
+        steps = [rng.choice((1, 1, 1, 2, 3)) for _ in range(nd)]
+        phys = [shape[perm[i]] * steps[perm[i]] for i in range(nd)]
+        base = torch.randint(-8, 8, phys, generator=g).float()
+        inv = [perm.index(d) for d in range(nd)]
+        index = tuple(slice(None, None, steps[d]) for d in range(nd))
+        return base.permute(*inv)[index], dev(base).permute(*inv)[index]
+
+    for case in range(60):
+        nd = rng.randint(1, 5)
+        shape = [rng.choice(extents) for _ in range(nd)]
+        while torch.Size(shape).numel() > (1 << 17):
+            shape[rng.randrange(nd)] = rng.choice(extents[:6])
+        bshape = [1 if rng.random() < 0.3 else e for e in shape]
+        (a, da), (b, db) = make(shape), make(bshape)
+        print(f"views {case}: a {tuple(a.shape)}/{a.stride()} b {tuple(b.shape)}/{b.stride()}", flush=True)
+        assert da.stride() == a.stride() and db.stride() == b.stride()
+        assert bit_equal((da + db).cpu(), a + b)
+        assert bit_equal(torch.add(da, db, alpha=-2.0).cpu(), torch.add(a, b, alpha=-2.0))
+        assert torch.equal(torch.eq(da, db).cpu(), torch.eq(a, b))
+        assert bit_equal(torch.relu(da).cpu(), torch.relu(a))
+        if case % 3 == 0:
+            m, dm = torch.eq(a, b), torch.eq(da, db)
+            assert bit_equal(torch.masked_select(da, dm).cpu(), torch.masked_select(a, m))
+            assert bit_equal(torch.masked_select(db, dm).cpu(), torch.masked_select(b, m))

@@ -45,8 +45,10 @@ def bit_equal(a, b):
         return False
     if a.numel() == 0:
         return True
-    av = a.contiguous().view(torch.uint8) if a.dtype != torch.bool else a.contiguous().view(torch.uint8)
-    bv = b.contiguous().view(torch.uint8) if b.dtype != torch.bool else b.contiguous().view(torch.uint8)
+    # copy into fresh 1-D tensors: a "contiguous" tensor may still carry odd strides on
+    # size-1 dimensions, which view(dtype) refuses
+    av = torch.empty(a.numel(), dtype=a.dtype).copy_(a.reshape(-1)).view(torch.uint8)
+    bv = torch.empty(b.numel(), dtype=b.dtype).copy_(b.reshape(-1)).view(torch.uint8)
     return bool(torch.equal(av, bv))
 
 
