@@ -178,6 +178,31 @@ int twg_unary_f32(int op, float *out, const float *in, const twg_iter_t *it,
 int twg_copy_strided(void *out, const void *in, int32_t elem_size,
                      const twg_iter_t *it, twg_stream_t stream);
 
+/* Element types twg_cast converts between (torch.bool is one byte holding 0 or 1). */
+enum twg_dtype {
+  TWG_DT_BOOL = 0,
+  TWG_DT_U8 = 1,
+  TWG_DT_I32 = 2,
+  TWG_DT_I64 = 3,
+  TWG_DT_F16 = 4,
+  TWG_DT_BF16 = 5,
+  TWG_DT_F32 = 6,
+  TWG_DT_F64 = 7,
+  TWG_DT_I8 = 8,
+  TWG_DT_I16 = 9
+};
+/* out[i] = (out_dtype) in[i] with ATen's CPU conversion rules (anything -> bool is
+ * x != 0, float -> integer truncates, narrowing floats round to nearest even), any
+ * strides.  No counterpart in the reference, whose copy_ moves bytes of one dtype
+ * (csrc/ops/copy.cpp:95-134) and whose strided copy is fp32 only (unary.h:34); it is
+ * what keeps `mask.float()`, `x.to(torch.int64)` and copies between host and device
+ * tensors of different dtypes off the CPU.  Direct pairs: everything <-> TWG_DT_F32,
+ * {BOOL, U8, I8, I16, I32, F64} <-> TWG_DT_I64, F64 -> BOOL; any other pair returns
+ * TWG_E_UNSUPPORTED and is composed exactly from two of these by the caller (through
+ * I64 between integer types and between F64 and integers, through F32 otherwise). */
+int twg_cast(void *out, int32_t out_dtype, const void *in, int32_t in_dtype,
+             const twg_iter_t *it, twg_stream_t stream);
+
 /* out[i] = (a[i] == b[i]) as a 0/1 byte, IEEE semantics (NaN != NaN, -0 == +0).
  * Replaces the boxed CPU fallback registered for eq.Tensor / eq.Tensor_out
  * (csrc/bindings.cpp:38-39). */

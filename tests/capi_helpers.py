@@ -82,6 +82,17 @@ def unary(fn_name, a, out=None, out_dtype=torch.float32, pre=(), extra=(), sort_
     return uo.fetch()
 
 
+def cast(a, out_dtype, out=None):
+    """out = a converted to out_dtype by twg_cast; returns (rc, tensor)."""
+    L = capi.load()
+    if out is None:
+        out = torch.zeros(tuple(a.shape), dtype=out_dtype)
+    ua, uo = Uploaded(a), Uploaded(out)
+    it = _iter_for(tuple(a.shape), out, (a,), True)
+    rc = L.twg_cast(uo.ptr, capi.DTYPES[out_dtype], ua.ptr, capi.DTYPES[a.dtype], ctypes.byref(it), None)
+    return rc, (uo.fetch() if rc == 0 else None)
+
+
 def add(a, b, alpha=1.0, out=None):
     return binary("twg_add_f32", a, b, out=out, extra=(ctypes.c_float(alpha),))
 

@@ -255,6 +255,83 @@ def test_mul_and_fused_add_relu(twg):
     assert bit_equal(m, a * 2.0)
 
 
+# ------------------------------------------------------------------- casts
+
+_INT_TYPES = (torch.bool, torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64)
+_FLOAT_TYPES = (torch.float16, torch.bfloat16, torch.float32, torch.float64)
+
+
+def _cast_source(dtype, n, g):
+    """Values every target type can hold (0..100 plus specials that stay defined)."""
+    if dtype == torch.bool:
+        return torch.rand(n, generator=g) < 0.5
+    if dtype in _INT_TYPES:
+        t = torch.randint(0, 101, (n,), generator=g).to(dtype)
+        if dtype == torch.int64:  # beyond 2^24 and 2^53: rounding on the way to float
+            t[:6] = torch.tensor([16777217, 33554435, (1 << 53) + 1, 123456789012345, 0, 1])
+        return t
+    t = (torch.rand(n, generator=g, dtype=torch.float64) * 100).to(dtype)
+    t[:8] = torch.tensor([0.0, -0.0, 0.5, 0.999, 1.5, 2.5, 99.99, 3.0]).to(dtype)
+    return t
+
+
+def test_cast_direct_pairs_match_aten(twg):
+    # every direct pair of twg_cast against ATen's CPU conversion of the same values
+    g = torch.Generator().manual_seed(21)
+    L = twg.load()
+    n = 70001
+    direct = 0
+    for src_t in _INT_TYPES + _FLOAT_TYPES:
+        for dst_t in _INT_TYPES + _FLOAT_TYPES:
+            if src_t == dst_t:
+                continue
+            a = _cast_source(src_t, n, g)
+            rc, got = H.cast(a, dst_t)
+            if rc == twg.E_UNSUPPORTED:
+                continue
+            twg.check(rc)
+            direct += 1
+            _say(f"cast {src_t} -> {dst_t}")
+            assert bit_equal(got, a.to(dst_t)), (src_t, dst_t)
+            # misaligned base pointers and a strided source / destination (div/mod kernel)
+            rc, got = H.cast(a[1:], dst_t)
+            assert rc == 0 and bit_equal(got, a[1:].to(dst_t))
+            a2 = a[:60000].view(200, 300).t()
+            rc, got = H.cast(a2, dst_t, out=torch.zeros(300, 400, dtype=dst_t)[:, ::2])
+            assert rc == 0 and bit_equal(got, a2.to(dst_t))
+    assert direct == 31
+    assert L.twg_cast(None, 99, None, 0, None, None) == twg.E_INVALID_ARG
+
+
+def test_cast_float_edge_cases(twg):
+    # rounding to half / bfloat16 (ties, overflow to inf, subnormals), NaN and inf,
+    # float -> bool on values that vanish in a narrower type, negative truncation
+    f = torch.tensor([1.0 + 2 ** -11, 1.0 + 3 * 2 ** -11, 65504.0, 65520.0, 65519.99, 1e-8, 6e-8,
+                      -6.1e-5, float("inf"), -float("inf"), float("nan"), 3.3895314e38,
+                      1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8, 1e-40, -1e-45, 0.0, -0.0])
+    for dst_t in (torch.float16, torch.bfloat16, torch.float64, torch.bool):
+        rc, got = H.cast(f, dst_t)
+        ref = f.to(dst_t)
+        assert rc == 0
+        assert bit_equal(got, ref) or (dst_t != torch.bool and torch.equal(got.isnan(), ref.isnan())
+                                       and bit_equal(got.nan_to_num(), ref.nan_to_num()))
+    d = torch.tensor([1e-300, -1e-310, 0.0, -0.0, float("nan"), 1e300, 16777217.0, 0.1],
+                     dtype=torch.float64)
+    rc, got = H.cast(d, torch.bool)
+    assert rc == 0 and torch.equal(got, d.to(torch.bool))
+    rc, got = H.cast(d, torch.float32)
+    assert rc == 0 and bit_equal(got.nan_to_num(), d.to(torch.float32).nan_to_num())
+    neg = torch.tensor([-0.9, -1.0, -1.5, -2.5, -100.7, 100.7, 2147483000.0, -2147483000.0])
+    for dst_t in (torch.int32, torch.int64, torch.int16, torch.int8):
+        src = neg if dst_t in (torch.int32, torch.int64) else neg[:6]
+        rc, got = H.cast(src, dst_t)
+        assert rc == 0 and torch.equal(got, src.to(dst_t)), dst_t
+    for src_t in (torch.float16, torch.bfloat16):
+        h = f.to(src_t)
+        rc, got = H.cast(h, torch.float32)
+        assert rc == 0 and bit_equal(got.nan_to_num(), h.to(torch.float32).nan_to_num())
+
+
 # ------------------------------------------------------------- activations
 
 def _unary(op, x, **kw):

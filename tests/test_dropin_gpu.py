@@ -395,3 +395,42 @@ def test_random_views_through_the_dispatcher():
             m, dm = torch.eq(a, b), torch.eq(da, db)
             assert bit_equal(torch.masked_select(da, dm).cpu(), torch.masked_select(a, m))
             assert bit_equal(torch.masked_select(db, dm).cpu(), torch.masked_select(b, m))
+
+
+def test_dtype_conversions_stay_on_the_device():
+    # t.to(dtype) / t.float() / mask.long() on webgpu tensors, and copy_ between host and
+    # device tensors of different dtypes: all ten dtypes both ways, against ATen's CPU result.
+    # Pairs without a direct kernel are composed of two (through int64 or float32).
+    g = torch.Generator().manual_seed(31)
+    dtypes = (torch.bool, torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64,
+              torch.float16, torch.bfloat16, torch.float32, torch.float64)
+    n = 5003
+    for src_t in dtypes:
+        if src_t == torch.bool:
+            a = torch.rand(n, generator=g) < 0.5
+        elif src_t.is_floating_point:
+            a = (torch.rand(n, generator=g, dtype=torch.float64) * 100).to(src_t)
+            a[:6] = torch.tensor([0.0, -0.0, 0.5, 0.999, 2.5, 99.5]).to(src_t)
+        else:
+            a = torch.randint(0, 101, (n,), generator=g).to(src_t)
+        da = dev(a)
+        assert da.dtype == src_t
+        for dst_t in dtypes:
+            ref = a.to(dst_t)
+            got = da.to(dst_t)
+            assert got.device.type == "webgpu" and got.dtype == dst_t
+            assert bit_equal(got.cpu(), ref), (src_t, dst_t)
+            # host -> device and device -> host with conversion on the way
+            up = torch.empty(n, dtype=dst_t, device="webgpu").copy_(a)
+            assert bit_equal(up.cpu(), ref), ("h2d", src_t, dst_t)
+            down = torch.empty(n, dtype=dst_t).copy_(da)
+            assert bit_equal(down, ref), ("d2h", src_t, dst_t)
+    # float64 -> bool keeps values that vanish in float32; strided views convert too
+    d = dev(torch.tensor([1e-300, 0.0, -0.0, 5e-324], dtype=torch.float64))
+    assert d.to(torch.bool).cpu().tolist() == [True, False, False, True]
+    m = torch.rand(64, 48, generator=g) < 0.3
+    assert bit_equal(dev(m).t().float().cpu(), m.t().float())
+    assert bit_equal(dev(m)[::2, 1::3].long().cpu(), m[::2, 1::3].long())
+    # the path's own ops accept the converted tensors
+    x = torch.randn(1000, generator=g, dtype=torch.float64)
+    assert bit_equal((dev(x).float() + dev(x).float()).cpu(), x.float() + x.float())

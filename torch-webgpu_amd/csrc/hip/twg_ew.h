@@ -1,0 +1,703 @@
+// Kernel templates and launch logic shared by the elementwise translation units of
+// libtwg_hip.so (arithmetic / activations / compares in twg_elementwise.hip, dtype
+// conversion in twg_cast.hip).  Everything is in an anonymous namespace: each unit
+// instantiates only what its entry points use.
+//
+// One templated family of kernels serves every op:
+//   ew_contig  - every operand dense and equally ordered: one 128-bit pack per
+//                lane, one short-lived block per 64 (or 256) packs, no loop.
+//   ew_rows    - inner dimension unit-stride (or broadcast) for every operand,
+//                outer dimensions arbitrary (row bias, column bias, slices).
+//   ew_tile(_vec) - an input whose unit stride lies along another dimension than
+//                the output's: tiles staged through LDS so both sides of the
+//                transpose stay coalesced (256x32 with 128-bit accesses when
+//                everything is a multiple of 4 elements, 64x64 dwords otherwise).
+//   ew_generic - anything else, one element per lane, div/mod index math with
+//                dimension 0 fastest.
+//
+// Replaces the two WGSL templates of the reference and their host drivers:
+//   csrc/ops/binary.cpp:23-104, csrc/ops/binary.h:29-215
+//   csrc/ops/unary.cpp:23-98,   csrc/ops/unary.h:30-181
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "twg_internal.h"
+
+namespace twg {
+namespace {
+
+constexpr int kThreads = 256;  // 4 wavefronts of 64
+
+#ifndef TWG_ROWS_UNROLL
+#define TWG_ROWS_UNROLL 1
+#endif
+#ifndef TWG_EW_BLOCKS_PER_CU
+#define TWG_EW_BLOCKS_PER_CU 8  // grid cap of the generic (grid-stride) kernel only
+#endif
+
+// Operands larger than this in total are treated as streaming (touched once, bigger
+// than the caches): loads and stores carry the nontemporal hint.  Smaller problems
+// keep default caching so a following op can hit in L2 / Infinity Cache.
+constexpr int64_t kStreamBytes = int64_t(64) << 20;
+
+// ------------------------------------------------------------------ packs
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Pack {
+  T v[N];
+};
+
+// Memory access goes through an integer vector of the pack's size so that one
+// instruction moves the whole pack (global_load/store_dwordx4 for 16 bytes) and so
+// that it can carry the nontemporal hint.  STREAM = true marks data that is touched
+// exactly once: on MI355X streaming kernels gain 5-10% from it.
+template <int BYTES>
+struct RawOf;
+template <>
+struct RawOf<1> { typedef uint8_t type; };
+template <>
+struct RawOf<2> { typedef uint16_t type; };
+template <>
+struct RawOf<4> { typedef uint32_t type; };
+template <>
+struct RawOf<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <>
+struct RawOf<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+
+template <bool STREAM, typename P>
+__device__ __forceinline__ P load_pack(const P *p) {
+  using R = typename RawOf<sizeof(P)>::type;
+  R r;
+  if constexpr (STREAM) {
+    r = __builtin_nontemporal_load(reinterpret_cast<const R *>(p));
+  } else {
+    r = *reinterpret_cast<const R *>(p);
+  }
+  P out;
+  __builtin_memcpy(&out, &r, sizeof(P));
+  return out;
+}
+template <bool STREAM, typename P>
+__device__ __forceinline__ void store_pack(P *p, const P &x) {
+  using R = typename RawOf<sizeof(P)>::type;
+  R r;
+  __builtin_memcpy(&r, &x, sizeof(P));
+  if constexpr (STREAM) {
+    __builtin_nontemporal_store(r, reinterpret_cast<R *>(p));
+  } else {
+    *reinterpret_cast<R *>(p) = r;
+  }
+}
+
+template <typename... Ts>
+struct MaxSize;
+template <typename T>
+struct MaxSize<T> {
+  static constexpr int value = (int)sizeof(T);
+};
+template <typename T, typename... Ts>
+struct MaxSize<T, Ts...> {
+  static constexpr int rest = MaxSize<Ts...>::value;
+  static constexpr int value = (int)sizeof(T) > rest ? (int)sizeof(T) : rest;
+};
+
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+__device__ __forceinline__ TO apply(const Op &op, TA a, TB b) {
+  if constexpr (NIN == 2) {
+    return op(a, b);
+  } else {
+    return op(a);
+  }
+}
+
+// ------------------------------------------------------------- ew_contig
+// One pack per lane, no loop: on MI355X a grid of very many short-lived blocks
+// streams faster (add: 6.4-6.7 TB/s) than a persistent grid-stride loop sized to
+// the 256 CUs (5.4 TB/s).  Block size matters too: single-wavefront blocks give add
+// 83% of peak against 80% for 256 lanes, while kernels whose output is narrower
+// than their input (compares: one dword of bools per lane) do best at 256.
+
+template <int THREADS, int NIN, int VEC, bool STREAM, typename Op, typename TO, typename TA,
+          typename TB>
+__global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const TB *b,
+                                                     int64_t numel, Op op) {
+  using PO = Pack<TO, VEC>;
+  using PA = Pack<TA, VEC>;
+  using PB = Pack<TB, VEC>;
+  const int64_t nvec = numel / VEC;
+  const int64_t i = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+  if (i < nvec) {
+    const PA va = load_pack<STREAM>(reinterpret_cast<const PA *>(a) + i);
+    PB vb;
+    if constexpr (NIN == 2) vb = load_pack<STREAM>(reinterpret_cast<const PB *>(b) + i);
+    PO r;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k)
+      r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
+    // the nontemporal hint pays for 16-byte stores only: one dword of bools per lane
+    // streams faster with a plain store (ne: 83% vs 79% of peak)
+    store_pack<STREAM && sizeof(PO) == 16>(reinterpret_cast<PO *>(out) + i, r);
+  }
+  if constexpr (VEC > 1) {  // the last numel % VEC elements
+    if (blockIdx.x == gridDim.x - 1) {
+      const int64_t e = nvec * VEC + threadIdx.x;
+      if (e < numel) out[e] = apply<NIN, Op, TO, TA, TB>(op, a[e], NIN == 2 ? b[e] : TB());
+    }
+  }
+}
+
+// --------------------------------------------------------------- ew_rows
+
+struct RowGeom {
+  int64_t len;               // extent of dimension 0
+  uint32_t chunks_per_row;   // blocks along one row
+  int32_t nouter;            // remaining dimensions
+  uint32_t reused;           // bit k: operand k is the same row for every block (a bias)
+  int64_t oshape[TWG_MAX_DIMS - 1];
+  int64_t ostride[3][TWG_MAX_DIMS - 1];
+};
+
+// A row every block re-reads should stay in L2: streaming hints only for the rest.
+template <bool STREAM, typename P>
+__device__ __forceinline__ P load_row_pack(const P *p, bool reused) {
+  if constexpr (STREAM) {
+    if (!reused) return load_pack<true>(p);
+  }
+  return load_pack<false>(p);
+}
+
+template <int THREADS, int NIN, int VEC, int UNROLL, bool STREAM, bool A_BC, bool B_BC, typename Op,
+          typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
+                                                    Op op) {
+  using PO = Pack<TO, VEC>;
+  using PA = Pack<TA, VEC>;
+  using PB = Pack<TB, VEC>;
+  uint32_t row = blockIdx.x / g.chunks_per_row;
+  const uint32_t chunk = blockIdx.x - row * g.chunks_per_row;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  {
+    int64_t r = row;
+    for (int d = 0; d < g.nouter; ++d) {
+      const int64_t q = r / g.oshape[d];
+      const int64_t c = r - q * g.oshape[d];
+      r = q;
+      off_o += c * g.ostride[0][d];
+      off_a += c * g.ostride[1][d];
+      if constexpr (NIN == 2) off_b += c * g.ostride[2][d];
+    }
+  }
+  TO *orow = out + off_o;
+  const TA *arow = a + off_a;
+  const TB *brow = (NIN == 2) ? b + off_b : nullptr;
+  TA abc = TA();
+  TB bbc = TB();
+  if constexpr (A_BC) abc = arow[0];
+  if constexpr (NIN == 2 && B_BC) bbc = brow[0];
+
+  const int64_t e0 = (int64_t)chunk * (THREADS * VEC * UNROLL) + (int64_t)threadIdx.x * VEC;
+  PA va[UNROLL];
+  PB vb[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t e = e0 + (int64_t)u * THREADS * VEC;
+    if (e < g.len) {
+      if constexpr (!A_BC)
+        va[u] = load_row_pack<STREAM>(reinterpret_cast<const PA *>(arow + e), g.reused & 2u);
+      if constexpr (NIN == 2 && !B_BC)
+        vb[u] = load_row_pack<STREAM>(reinterpret_cast<const PB *>(brow + e), g.reused & 4u);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t e = e0 + (int64_t)u * THREADS * VEC;
+    if (e < g.len) {
+      PO r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const TA x = A_BC ? abc : va[u].v[k];
+        const TB y = (NIN == 2) ? (B_BC ? bbc : vb[u].v[k]) : TB();
+        r.v[k] = apply<NIN, Op, TO, TA, TB>(op, x, y);
+      }
+      store_pack<STREAM && sizeof(PO) == 16>(reinterpret_cast<PO *>(orow + e), r);
+    }
+  }
+}
+
+// --------------------------------------------------------------- ew_tile
+
+constexpr int kTile = 64;
+
+struct TileGeom {
+  int64_t n0, nt;          // extents of dimension 0 and of the transposed dimension t
+  int64_t s0[3], st[3];    // strides along those two, per operand
+  uint32_t tiles0, tilest; // tile counts
+  int32_t nbatch;          // remaining dimensions
+  int64_t bshape[TWG_MAX_DIMS - 2];
+  int64_t bstride[3][TWG_MAX_DIMS - 2];
+};
+
+// Lane x (0..63) runs along dimension 0, the 4 wavefronts and 16 steps cover 64
+// positions along t.  An operand marked *_T has its unit stride along t: it is
+// read with lane x along t instead, parked in LDS and picked up transposed.
+template <int NIN, bool A_T, bool B_T, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_tile(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                    Op op) {
+  __shared__ TA sa[A_T ? kTile : 1][kTile + 1];
+  __shared__ TB sb[(NIN == 2 && B_T) ? kTile : 1][kTile + 1];
+
+  uint32_t bid = blockIdx.x;
+  const uint32_t t0i = bid % g.tiles0;
+  bid /= g.tiles0;
+  const uint32_t tti = bid % g.tilest;
+  int64_t r = bid / g.tilest;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const int64_t q = r / g.bshape[d];
+    const int64_t c = r - q * g.bshape[d];
+    r = q;
+    off_o += c * g.bstride[0][d];
+    off_a += c * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
+  }
+  const int x = threadIdx.x & 63;
+  const int y = threadIdx.x >> 6;  // 0..3
+  const int64_t base0 = (int64_t)t0i * kTile;
+  const int64_t baset = (int64_t)tti * kTile;
+
+  if constexpr (A_T) {
+    const int64_t tt = baset + x;
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) {
+      const int64_t d0 = base0 + y + 4 * k;
+      if (tt < g.nt && d0 < g.n0) sa[y + 4 * k][x] = a[off_a + d0 * g.s0[1] + tt * g.st[1]];
+    }
+  }
+  if constexpr (NIN == 2 && B_T) {
+    const int64_t tt = baset + x;
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) {
+      const int64_t d0 = base0 + y + 4 * k;
+      if (tt < g.nt && d0 < g.n0) sb[y + 4 * k][x] = b[off_b + d0 * g.s0[2] + tt * g.st[2]];
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+
+  const int64_t d0 = base0 + x;
+  if (d0 >= g.n0) return;
+#pragma unroll 4
+  for (int k = 0; k < kTile / 4; ++k) {
+    const int tl = y + 4 * k;
+    const int64_t tt = baset + tl;
+    if (tt >= g.nt) break;
+    TA va;
+    TB vb = TB();
+    if constexpr (A_T) {
+      va = sa[x][tl];
+    } else {
+      va = a[off_a + d0 * g.s0[1] + tt * g.st[1]];
+    }
+    if constexpr (NIN == 2) {
+      if constexpr (B_T) {
+        vb = sb[x][tl];
+      } else {
+        vb = b[off_b + d0 * g.s0[2] + tt * g.st[2]];
+      }
+    }
+    out[off_o + d0 * g.s0[0] + tt * g.st[0]] = apply<NIN, Op, TO, TA, TB>(op, va, vb);
+  }
+}
+
+// Same job with 128-bit accesses on both sides of the transpose, for 4-byte
+// elements when extents, strides and pointers are all multiples of 4 elements.
+// Tile = TD0 (dimension 0) x TT (dimension t).  The output and the operands with
+// unit stride along dimension 0 move as float4 runs of TD0 elements; an operand
+// marked *_T is read as float4 runs of TT elements along t, scattered into LDS as
+// st[t][d0] (row pitch TD0 + 4 keeps the float4 reads aligned) and read back along
+// dimension 0.  Wide tiles matter: 256 x 32 reaches 75% of HBM peak on the
+// [32768, 8192] transposed add, 64 x 64 only 66%, one dword per lane 52%.
+template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO, typename TA,
+          typename TB>
+__global__ __launch_bounds__(kThreads) void ew_tile_vec(TO *out, const TA *a, const TB *b,
+                                                        TileGeom g, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  constexpr int kPitch = TD0 + 4;
+  __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
+  __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
+
+  uint32_t bid = blockIdx.x;
+  const uint32_t t0i = bid % g.tiles0;
+  bid /= g.tiles0;
+  const uint32_t tti = bid % g.tilest;
+  int64_t r = bid / g.tilest;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const int64_t q = r / g.bshape[d];
+    const int64_t c = r - q * g.bshape[d];
+    r = q;
+    off_o += c * g.bstride[0][d];
+    off_a += c * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
+  }
+  const int64_t base0 = (int64_t)t0i * TD0;
+  const int64_t baset = (int64_t)tti * TT;
+
+  // transposed operands: float4 along t -> LDS[t][d0]
+  constexpr int kLanesT = TT / 4, kRowsT = kThreads / kLanesT, kPassT = TD0 / kRowsT;
+  static_assert(TT % 4 == 0 && kThreads % kLanesT == 0 && TD0 % kRowsT == 0, "tile shape");
+  {
+    const int tx = threadIdx.x % kLanesT, ty = threadIdx.x / kLanesT;
+    const int64_t tt = baset + 4 * tx;
+    if constexpr (A_T) {
+      PA v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t d0 = base0 + ty + kRowsT * p;
+        if (d0 < g.n0 && tt < g.nt)
+          v[p] = load_pack<true>(reinterpret_cast<const PA *>(a + off_a + d0 * g.s0[1] + tt));
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (base0 + rr < g.n0 && tt < g.nt) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sa[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+    if constexpr (NIN == 2 && B_T) {
+      PB v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t d0 = base0 + ty + kRowsT * p;
+        if (d0 < g.n0 && tt < g.nt)
+          v[p] = load_pack<true>(reinterpret_cast<const PB *>(b + off_b + d0 * g.s0[2] + tt));
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (base0 + rr < g.n0 && tt < g.nt) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sb[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+  }
+
+  // everything else: float4 along dimension 0
+  constexpr int kLanes0 = TD0 / 4, kRows0 = kThreads / kLanes0, kPass0 = TT / kRows0;
+  static_assert(TD0 % 4 == 0 && kThreads % kLanes0 == 0 && TT % kRows0 == 0, "tile shape");
+  const int tx = threadIdx.x % kLanes0, ty = threadIdx.x / kLanes0;
+  const int64_t d0 = base0 + 4 * tx;
+  PA va[kPass0];
+  PB vb[kPass0];
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int64_t tt = baset + ty + kRows0 * p;
+    if (d0 < g.n0 && tt < g.nt) {
+      if constexpr (!A_T) va[p] = load_pack<true>(reinterpret_cast<const PA *>(a + off_a + d0 + tt * g.st[1]));
+      if constexpr (NIN == 2 && !B_T)
+        vb[p] = load_pack<true>(reinterpret_cast<const PB *>(b + off_b + d0 + tt * g.st[2]));
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int rr = ty + kRows0 * p;
+    const int64_t tt = baset + rr;
+    if (d0 < g.n0 && tt < g.nt) {
+      if constexpr (A_T) va[p] = *reinterpret_cast<const PA *>(&sa[rr][4 * tx]);
+      if constexpr (NIN == 2 && B_T) vb[p] = *reinterpret_cast<const PB *>(&sb[rr][4 * tx]);
+      PO o;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        o.v[c] = apply<NIN, Op, TO, TA, TB>(op, va[p].v[c], NIN == 2 ? vb[p].v[c] : TB());
+      store_pack<true>(reinterpret_cast<PO *>(out + off_o + d0 + tt * g.st[0]), o);
+    }
+  }
+}
+
+// ------------------------------------------------------------ ew_generic
+
+template <typename UIdx, typename SIdx>
+struct GenGeom {
+  int32_t ndim;
+  UIdx numel;
+  UIdx shape[TWG_MAX_DIMS];
+  SIdx stride[3][TWG_MAX_DIMS];
+};
+
+template <int NIN, typename UIdx, typename SIdx, typename Op, typename TO, typename TA,
+          typename TB>
+__global__ __launch_bounds__(kThreads) void ew_generic(TO *out, const TA *a, const TB *b,
+                                                       GenGeom<UIdx, SIdx> g, Op op) {
+  const UIdx step = (UIdx)gridDim.x * kThreads;
+  for (UIdx i = (UIdx)blockIdx.x * kThreads + threadIdx.x; i < g.numel; i += step) {
+    UIdx rem = i;
+    SIdx oo = 0, oa = 0, ob = 0;
+    for (int d = 0; d < g.ndim; ++d) {  // dimension 0 is the fastest-moving one
+      const UIdx q = rem / g.shape[d];
+      const SIdx c = (SIdx)(rem - q * g.shape[d]);
+      rem = q;
+      oo += c * g.stride[0][d];
+      oa += c * g.stride[1][d];
+      if constexpr (NIN == 2) ob += c * g.stride[2][d];
+    }
+    out[oo] = apply<NIN, Op, TO, TA, TB>(op, a[oa], NIN == 2 ? b[ob] : TB());
+  }
+}
+
+// -------------------------------------------------------------- dispatch
+
+inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+
+inline unsigned capped_grid(int64_t blocks_wanted) {
+  int64_t cap = (int64_t)compute_units() * TWG_EW_BLOCKS_PER_CU;
+  if (cap < 1) cap = 1;
+  if (blocks_wanted < 1) blocks_wanted = 1;
+  return (unsigned)(blocks_wanted < cap ? blocks_wanted : cap);
+}
+
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_generic(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  bool fits32 = g.numel <= INT32_MAX;
+  for (int o = 0; o <= NIN && fits32; ++o) {
+    int64_t span = 0;
+    for (int d = 0; d < g.ndim; ++d) {
+      int64_t st = g.stride[o][d] < 0 ? -g.stride[o][d] : g.stride[o][d];
+      span += st * (g.shape[d] - 1);
+      if (span > INT32_MAX) { fits32 = false; break; }
+    }
+  }
+  const unsigned grid = capped_grid((g.numel + kThreads - 1) / kThreads);
+  if (fits32) {
+    GenGeom<uint32_t, int32_t> gg{};
+    gg.ndim = g.ndim;
+    gg.numel = (uint32_t)g.numel;
+    for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+      gg.shape[d] = (uint32_t)g.shape[d];
+      for (int o = 0; o < 3; ++o) gg.stride[o][d] = (int32_t)g.stride[o][d];
+    }
+    ew_generic<NIN, uint32_t, int32_t, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, gg, op);
+  } else {
+    GenGeom<uint64_t, int64_t> gg{};
+    gg.ndim = g.ndim;
+    gg.numel = (uint64_t)g.numel;
+    for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+      gg.shape[d] = (uint64_t)g.shape[d];
+      for (int o = 0; o < 3; ++o) gg.stride[o][d] = g.stride[o][d];
+    }
+    ew_generic<NIN, uint64_t, int64_t, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, gg, op);
+  }
+  return (int)hipGetLastError();
+}
+
+template <int NIN, int VEC, bool A_BC, bool B_BC, typename Op, typename TO, typename TA,
+          typename TB>
+int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  constexpr int U = TWG_ROWS_UNROLL;
+  RowGeom rg{};
+  rg.len = g.shape[0];
+  constexpr int kBlock = 64;  // single-wavefront blocks stream best (see ew_contig)
+  const int64_t per_block = (int64_t)kBlock * VEC * U;
+  const int64_t cpr = (rg.len + per_block - 1) / per_block;
+  const int64_t rows = g.numel / rg.len;
+  if (cpr * rows > INT32_MAX || cpr > UINT32_MAX) return TWG_E_UNSUPPORTED;
+  rg.chunks_per_row = (uint32_t)cpr;
+  rg.nouter = g.ndim - 1;
+  for (int d = 1; d < g.ndim; ++d) {
+    rg.oshape[d - 1] = g.shape[d];
+    for (int o = 0; o < 3; ++o) rg.ostride[o][d - 1] = g.stride[o][d];
+  }
+  for (int o = 1; o <= NIN; ++o) {
+    bool same_row = true;
+    for (int d = 1; d < g.ndim; ++d) same_row = same_row && g.stride[o][d] == 0;
+    if (same_row) rg.reused |= 1u << o;
+  }
+  const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
+  if (stream)
+    ew_rows<kBlock, NIN, VEC, U, true, A_BC, B_BC, Op, TO, TA, TB>
+        <<<(unsigned)(cpr * rows), kBlock, 0, s>>>(out, a, b, rg, op);
+  else
+    ew_rows<kBlock, NIN, VEC, U, false, A_BC, B_BC, Op, TO, TA, TB>
+        <<<(unsigned)(cpr * rows), kBlock, 0, s>>>(out, a, b, rg, op);
+  return (int)hipGetLastError();
+}
+
+template <int NIN, bool A_BC, bool B_BC, typename Op, typename TO, typename TA, typename TB>
+int launch_rows(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  constexpr int VEC = 16 / MaxSize<TO, TA, TB>::value;
+  // Packs need every row start aligned for every non-broadcast operand.
+  bool vec_ok = (g.shape[0] % VEC == 0) && aligned_to(out, sizeof(TO) * VEC) &&
+                (A_BC || aligned_to(a, sizeof(TA) * VEC)) &&
+                (NIN == 1 || B_BC || aligned_to(b, sizeof(TB) * VEC));
+  for (int d = 1; d < g.ndim && vec_ok; ++d) {
+    vec_ok = vec_ok && (g.stride[0][d] % VEC == 0) && (A_BC || g.stride[1][d] % VEC == 0) &&
+             (NIN == 1 || B_BC || g.stride[2][d] % VEC == 0);
+  }
+  if (vec_ok) return launch_rows_v<NIN, VEC, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
+  return launch_rows_v<NIN, 1, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
+}
+
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
+                hipStream_t s) {
+  TileGeom tg{};
+  tg.n0 = g.shape[0];
+  tg.nt = g.shape[t];
+  for (int o = 0; o < 3; ++o) {
+    tg.s0[o] = g.stride[o][0];
+    tg.st[o] = g.stride[o][t];
+  }
+  int64_t batch = 1;
+  tg.nbatch = 0;
+  for (int d = 1; d < g.ndim; ++d) {
+    if (d == t) continue;
+    tg.bshape[tg.nbatch] = g.shape[d];
+    for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+    tg.nbatch++;
+    batch *= g.shape[d];
+  }
+  auto set_tiles = [&](int td0, int tt, unsigned *grid) {
+    const int64_t tiles0 = (tg.n0 + td0 - 1) / td0;
+    const int64_t tilest = (tg.nt + tt - 1) / tt;
+    if (tiles0 > UINT32_MAX || tilest > UINT32_MAX) return false;
+    if (tiles0 * tilest > INT32_MAX || tiles0 * tilest * batch > INT32_MAX) return false;
+    tg.tiles0 = (uint32_t)tiles0;
+    tg.tilest = (uint32_t)tilest;
+    *grid = (unsigned)(tiles0 * tilest * batch);
+    return true;
+  };
+  unsigned grid = 0;
+
+  // 128-bit path: 4-byte elements, everything a multiple of 4 elements, and every
+  // operand with its unit stride either along dimension 0 or (if marked) along t.
+  if constexpr (sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4) {
+    bool ok = tg.n0 % 4 == 0 && tg.nt % 4 == 0 && tg.s0[0] == 1 && tg.st[0] % 4 == 0 &&
+              aligned_to(out, 16) && aligned_to(a, 16) && (NIN == 1 || aligned_to(b, 16));
+    ok = ok && (a_t ? (tg.st[1] == 1 && tg.s0[1] % 4 == 0) : (tg.s0[1] == 1 && tg.st[1] % 4 == 0));
+    if (NIN == 2)
+      ok = ok && (b_t ? (tg.st[2] == 1 && tg.s0[2] % 4 == 0) : (tg.s0[2] == 1 && tg.st[2] % 4 == 0));
+    for (int d = 0; d < tg.nbatch && ok; ++d)
+      for (int o = 0; o <= NIN; ++o) ok = ok && tg.bstride[o][d] % 4 == 0;
+    if (ok) {
+      const bool wide = tg.n0 >= 256;
+      if (!set_tiles(wide ? 256 : 64, wide ? 32 : 64, &grid)) return TWG_E_UNSUPPORTED;
+#define TWG_LAUNCH_TILE_VEC(AT, BT)                                                              \
+  do {                                                                                           \
+    if (wide)                                                                                    \
+      ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op); \
+    else                                                                                         \
+      ew_tile_vec<NIN, AT, BT, 64, 64, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);  \
+  } while (0)
+      if (a_t && b_t) {
+        if constexpr (NIN == 2) TWG_LAUNCH_TILE_VEC(true, true);
+      } else if (a_t) {
+        TWG_LAUNCH_TILE_VEC(true, false);
+      } else {
+        if constexpr (NIN == 2) TWG_LAUNCH_TILE_VEC(false, true);
+      }
+#undef TWG_LAUNCH_TILE_VEC
+      return (int)hipGetLastError();
+    }
+  }
+
+  if (!set_tiles(kTile, kTile, &grid)) return TWG_E_UNSUPPORTED;
+  if (a_t && b_t) {
+    if constexpr (NIN == 2)
+      ew_tile<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  } else if (a_t) {
+    ew_tile<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  } else {
+    if constexpr (NIN == 2)
+      ew_tile<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  }
+  return (int)hipGetLastError();
+}
+
+// Pick the kernel for a canonical geometry.  ALL_SHAPES = false keeps only the dense
+// kernel and the div/mod one (for op families with many type combinations, where the
+// row and tile kernels would multiply the code size for layouts that hardly occur).
+template <int NIN, typename Op, typename TO, typename TA, typename TB, bool ALL_SHAPES = true>
+int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, twg_stream_t stream) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  Geom g;
+  if ((rc = canonicalize(it, NIN + 1, &g))) return rc;
+  if (g.numel == 0) return 0;
+  if (!out || !a || (NIN == 2 && !b)) return TWG_E_INVALID_ARG;
+  hipStream_t s = resolve_stream(stream);
+  constexpr int VEC = 16 / MaxSize<TO, TA, TB>::value;
+
+  // (i) every operand dense in the same order
+  bool dense = g.ndim <= 1;
+  if (dense && g.ndim == 1)
+    dense = g.stride[0][0] == 1 && g.stride[1][0] == 1 && (NIN == 1 || g.stride[2][0] == 1);
+  if (dense) {
+    const bool vec_ok = aligned_to(out, sizeof(TO) * VEC) && aligned_to(a, sizeof(TA) * VEC) &&
+                        (NIN == 1 || aligned_to(b, sizeof(TB) * VEC));
+    const bool stream =
+        g.numel * (int64_t)(sizeof(TO) + sizeof(TA) + (NIN == 2 ? sizeof(TB) : 0)) > kStreamBytes;
+    constexpr int kBlock = sizeof(TO) < sizeof(TA) ? 256 : 64;
+    const int64_t packs = vec_ok ? (g.numel + VEC - 1) / VEC : g.numel;
+    const int64_t blocks = (packs + kBlock - 1) / kBlock;
+    if (blocks > INT32_MAX) return TWG_E_UNSUPPORTED;
+    const unsigned grid = (unsigned)blocks;
+    if (vec_ok && stream)
+      ew_contig<kBlock, NIN, VEC, true, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+    else if (vec_ok)
+      ew_contig<kBlock, NIN, VEC, false, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+    else if (stream)
+      ew_contig<kBlock, NIN, 1, true, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+    else
+      ew_contig<kBlock, NIN, 1, false, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+    return (int)hipGetLastError();
+  }
+
+  if constexpr (ALL_SHAPES) {
+    if (g.ndim >= 1 && g.stride[0][0] == 1) {
+      const int64_t sa0 = g.stride[1][0];
+      const int64_t sb0 = (NIN == 2) ? g.stride[2][0] : 1;
+      // (ii) inner dimension unit-stride or broadcast for every input
+      if ((sa0 == 0 || sa0 == 1) && (sb0 == 0 || sb0 == 1) && !(sa0 == 0 && sb0 == 0) &&
+          g.shape[0] >= 64) {
+        int r;
+        if (sa0 == 0) {
+          r = launch_rows<NIN, true, false, Op, TO, TA, TB>(out, a, b, g, op, s);
+        } else if (NIN == 2 && sb0 == 0) {
+          r = launch_rows<NIN, false, true, Op, TO, TA, TB>(out, a, b, g, op, s);
+        } else {
+          r = launch_rows<NIN, false, false, Op, TO, TA, TB>(out, a, b, g, op, s);
+        }
+        if (r != TWG_E_UNSUPPORTED) return r;
+      }
+      // (iii) an input with its unit stride along another dimension
+      if (g.ndim >= 2 && g.shape[0] >= 16) {
+        int t = -1;
+        for (int d = 1; d < g.ndim && t < 0; ++d) {
+          if (g.shape[d] < 16) continue;
+          if ((sa0 != 0 && sa0 != 1 && g.stride[1][d] == 1) ||
+              (NIN == 2 && sb0 != 0 && sb0 != 1 && g.stride[2][d] == 1))
+            t = d;
+        }
+        if (t > 0) {
+          const bool a_t = sa0 != 0 && sa0 != 1 && g.stride[1][t] == 1;
+          const bool b_t = NIN == 2 && sb0 != 0 && sb0 != 1 && g.stride[2][t] == 1;
+          int r = launch_tile<NIN, Op, TO, TA, TB>(out, a, b, g, t, a_t, b_t, op, s);
+          if (r != TWG_E_UNSUPPORTED) return r;
+        }
+      }
+    }
+  }
+  // (iv) anything else
+  return launch_generic<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
+}
+
+}  // namespace
+}  // namespace twg

@@ -5,7 +5,8 @@
 // (csrc/ops/copy.cpp:12-62,191-194); here _copy_from and copy_ handle that
 // direction themselves, so ATen's CPU kernel is left alone.  Restrictions the
 // reference has and this does not: fp32 only on the way back (copy.cpp:22),
-// contiguous destination (copy.cpp:78), source offset ignored (copy.cpp:42).
+// contiguous destination (copy.cpp:78), source offset ignored (copy.cpp:42), equal
+// dtypes (a copy between dtypes is converted on the device, never on the host).
 #include <ATen/ops/_copy_from_and_resize_native.h>
 #include <ATen/ops/copy_native.h>
 #include <torch/library.h>
@@ -24,12 +25,63 @@ bool same_dense_layout(const at::Tensor &a, const at::Tensor &b) {
          a.is_non_overlapping_and_dense();
 }
 
-// dst <- src, both on the device, same dtype; any strides, src broadcast to dst.
+int twg_dtype_of(at::ScalarType t) {
+  switch (t) {
+    case at::kBool: return TWG_DT_BOOL;
+    case at::kByte: return TWG_DT_U8;
+    case at::kChar: return TWG_DT_I8;
+    case at::kShort: return TWG_DT_I16;
+    case at::kInt: return TWG_DT_I32;
+    case at::kLong: return TWG_DT_I64;
+    case at::kHalf: return TWG_DT_F16;
+    case at::kBFloat16: return TWG_DT_BF16;
+    case at::kFloat: return TWG_DT_F32;
+    case at::kDouble: return TWG_DT_F64;
+    default: return -1;
+  }
+}
+
+bool is_integral_dt(int dt) { return dt <= TWG_DT_I64 || dt == TWG_DT_I8 || dt == TWG_DT_I16; }
+
+void device_to_device(const at::Tensor &dst, const at::Tensor &src);
+
+// dst <- (dtype of dst) src on the device.  Pairs libtwg_hip has no direct kernel for
+// go through the intermediate that keeps ATen's result: int64 between integer types
+// and between float64 and integers, float32 otherwise.
+void device_cast(const at::Tensor &dst, const at::Tensor &src) {
+  const int od = twg_dtype_of(dst.scalar_type()), id = twg_dtype_of(src.scalar_type());
+  TORCH_CHECK(od >= 0 && id >= 0, "webgpu copy_: no conversion from ", src.scalar_type(), " to ",
+              dst.scalar_type(), " on the device");
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(dst);
+  config.add_const_input(src);
+  config.resize_outputs(false);
+  config.check_all_same_dtype(false);
+  auto iter = config.build();
+  if (iter.numel() == 0) return;
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  const int rc = twg_cast(iter.data_ptr(0), od, iter.data_ptr(1), id, &it, nullptr);
+  if (rc != TWG_E_UNSUPPORTED) {
+    TWG_CHECK(rc);
+    return;
+  }
+  const bool via_i64 = (is_integral_dt(od) && is_integral_dt(id)) ||
+                       (id == TWG_DT_F64 && is_integral_dt(od)) ||
+                       (od == TWG_DT_F64 && is_integral_dt(id));
+  at::Tensor mid = at::empty(src.sizes(), src.options().dtype(via_i64 ? at::kLong : at::kFloat));
+  device_cast(mid, src);
+  device_cast(dst, mid);
+}
+
+// dst <- src, both on the device; any strides, src broadcast to dst.
 void device_to_device(const at::Tensor &dst, const at::Tensor &src) {
-  TORCH_CHECK(dst.scalar_type() == src.scalar_type(),
-              "webgpu copy_: device-to-device copies need equal dtypes, got ", dst.scalar_type(),
-              " and ", src.scalar_type());
   if (dst.numel() == 0) return;
+  if (dst.scalar_type() != src.scalar_type()) {
+    device_cast(dst, src);
+    return;
+  }
   if (same_dense_layout(dst, src)) {  // csrc/ops/copy.cpp:95-122
     if (dst.data_ptr() != src.data_ptr())
       TWG_CHECK(twg_memcpy_d2d(dst.data_ptr(), src.data_ptr(), nbytes_of(dst), nullptr));
@@ -52,9 +104,14 @@ void device_to_device(const at::Tensor &dst, const at::Tensor &src) {
 
 void host_to_device(const at::Tensor &dst, const at::Tensor &src) {
   if (dst.numel() == 0) return;
-  // dtype conversion and broadcasting happen on the host, where ATen has kernels
+  if (src.scalar_type() != dst.scalar_type()) {
+    // the bytes go up as they are; the conversion runs on the device
+    at::Tensor staged = at::empty(src.sizes(), dst.options().dtype(src.scalar_type()));
+    host_to_device(staged, src);
+    device_cast(dst, staged);
+    return;
+  }
   at::Tensor s = src;
-  if (s.scalar_type() != dst.scalar_type()) s = s.to(dst.scalar_type());
   if (s.sizes() != dst.sizes()) s = s.expand(dst.sizes());
   if (dst.is_contiguous()) {  // csrc/ops/copy.cpp:74-92
     s = s.contiguous();
@@ -72,22 +129,26 @@ void host_to_device(const at::Tensor &dst, const at::Tensor &src) {
 void device_to_host(const at::Tensor &dst, const at::Tensor &src) {
   if (dst.numel() == 0) return;
   at::Tensor s = src;
+  if (s.scalar_type() != dst.scalar_type()) {  // convert on the device, then bring it down
+    at::Tensor converted = at::empty(s.sizes(), s.options().dtype(dst.scalar_type()));
+    device_cast(converted, s);
+    s = converted;
+  }
   if (s.sizes() != dst.sizes()) s = s.expand(dst.sizes());
   if (!(s.is_contiguous() || (s.is_non_overlapping_and_dense() && s.strides() == dst.strides()))) {
     at::Tensor dense = at::empty(s.sizes(), s.options());
     device_to_device(dense, s);
     s = dense;
   }
-  const bool direct = s.scalar_type() == dst.scalar_type() &&
-                      ((dst.is_contiguous() && s.is_contiguous()) ||
-                       (dst.is_non_overlapping_and_dense() && dst.strides() == s.strides()));
+  const bool direct = (dst.is_contiguous() && s.is_contiguous()) ||
+                      (dst.is_non_overlapping_and_dense() && dst.strides() == s.strides());
   if (direct) {
     TWG_CHECK(twg_memcpy_d2h(dst.data_ptr(), s.const_data_ptr(), nbytes_of(dst), nullptr));
   } else {
     at::Tensor host = at::empty_strided(s.sizes(), s.strides(),
                                         dst.options().dtype(s.scalar_type()));
     TWG_CHECK(twg_memcpy_d2h(host.data_ptr(), s.const_data_ptr(), nbytes_of(host), nullptr));
-    at::native::copy_(const_cast<at::Tensor &>(dst), host, false);  // host-side cast / restride
+    at::native::copy_(const_cast<at::Tensor &>(dst), host, false);  // host-side restride only
   }
 }
 

@@ -19,6 +19,9 @@ MAX_DIMS = 8
 OUT, A, B = 0, 1, 2
 
 UNARY_COPY, UNARY_RELU, UNARY_GELU_ERF, UNARY_GELU_TANH, UNARY_SILU, UNARY_ABS = 0, 1, 2, 3, 4, 5
+# enum twg_dtype, keyed by torch dtype
+DTYPES = {torch.bool: 0, torch.uint8: 1, torch.int32: 2, torch.int64: 3, torch.float16: 4,
+          torch.bfloat16: 5, torch.float32: 6, torch.float64: 7, torch.int8: 8, torch.int16: 9}
 
 E_INVALID_ARG, E_UNSUPPORTED, E_SCRATCH_SMALL = -1, -2, -3
 
@@ -54,7 +57,7 @@ SYMBOLS = [
     "twg_malloc", "twg_free", "twg_empty_cache", "twg_mem_stats",
     "twg_memcpy_h2d", "twg_memcpy_d2h", "twg_memcpy_d2d", "twg_fill_bytes",
     "twg_add_f32", "twg_add_scalar_f32", "twg_mul_f32", "twg_mul_scalar_f32",
-    "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided",
+    "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided", "twg_cast",
     "twg_eq_f32", "twg_ne_scalar_f32", "twg_and_u8",
     "twg_masked_select_scratch_bytes", "twg_masked_select_f32",
 ]
@@ -104,6 +107,7 @@ def load():
     L.twg_add_relu_f32.argtypes = [vp, vp, vp, ip, vp]
     L.twg_unary_f32.argtypes = [ctypes.c_int, vp, vp, ip, vp]
     L.twg_copy_strided.argtypes = [vp, vp, i32, ip, vp]
+    L.twg_cast.argtypes = [vp, i32, vp, i32, ip, vp]
     L.twg_eq_f32.argtypes = [vp, vp, vp, ip, vp]
     L.twg_ne_scalar_f32.argtypes = [vp, vp, f32, ip, vp]
     L.twg_and_u8.argtypes = [vp, vp, vp, ip, vp]
