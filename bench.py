@@ -284,7 +284,7 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         del d_a3, d_bias, d_c3
 
     # config 4: eq, ne.Scalar, bitwise_and
-    if want("eq") or want("ne_scalar") or want("bitwise_and"):
+    if any(want(k) for k in ("eq", "ne_scalar", "bitwise_and", "cast_bool_f32", "cast_f32_f16")):
         p_h, q_h, z_h = W.mask_inputs(n, seed=3)
         d_p, d_q, d_z = capi.to_device(p_h), capi.to_device(q_h), capi.to_device(z_h)
         del p_h, q_h, z_h
@@ -295,6 +295,15 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         res.append(summarize("ne_scalar", "ew_contig<NeScalarOp>", by["ne_scalar"] * n, ms, n))
         ms = time_launches(lambda: capi.check(L.twg_and_u8(d_m3.ptr, d_m1.ptr, d_m2.ptr, ctypes.byref(it), None)), Wm, K)
         res.append(summarize("bitwise_and", "ew_contig<AndOp>", by["bitwise_and"] * n, ms, n))
+        # dtype conversion of a mask (mask.float()) and of fp32 data (x.half()): 5 and 6 B/element
+        if want("cast_bool_f32"):
+            ms = time_launches(lambda: capi.check(L.twg_cast(d_out.ptr, capi.DTYPES[torch.float32], d_m1.ptr,
+                                                             capi.DTYPES[torch.bool], ctypes.byref(it), None)), Wm, K)
+            res.append(summarize("cast_bool_f32", "ew_contig<CastOp<float,bool>>", 5 * n, ms, n))
+        if want("cast_f32_f16"):
+            ms = time_launches(lambda: capi.check(L.twg_cast(d_out.ptr, capi.DTYPES[torch.float16], d_z.ptr,
+                                                             capi.DTYPES[torch.float32], ctypes.byref(it), None)), Wm, K)
+            res.append(summarize("cast_f32_f16", "ew_contig<CastOp<half,float>>", 6 * n, ms, n))
         del d_p, d_q, d_z, d_m1, d_m2, d_m3
 
     # config 5: the other masks
