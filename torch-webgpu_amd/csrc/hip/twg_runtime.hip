@@ -91,6 +91,8 @@ int release_cached_locked(Pool &p) {
 
 constexpr int kStageSlots = 8;
 constexpr size_t kStreamingDrainBytes = size_t(32) << 20;  // beyond what a last-level cache keeps
+constexpr size_t kMailboxBytes = 256;                      // largest read served by the mailbox
+constexpr int kMailboxSpins = 200000;                      // then fall back to a stream sync
 
 struct Staging {
   std::mutex mu;
@@ -103,6 +105,12 @@ struct Staging {
   hipEvent_t ev[kStageSlots] = {};
   bool busy[kStageSlots] = {};
   char *buf(int i) const { return base + (size_t)i * chunk; }
+  // Mailbox for reads of a few bytes (a count, a scalar): coherent pinned memory a small
+  // kernel writes and the host polls, which returns in ~3 us where waiting on the stream
+  // or on an event takes ~12 us.  [0, kMailboxBytes) payload, then the sequence word.
+  char *mailbox = nullptr;      // host address
+  void *mailbox_dev = nullptr;  // the same memory as the device addresses it
+  uint32_t mailbox_seq = 0;
 };
 
 // Copy out of a staging slot into pageable memory.  Large destinations do not fit in
@@ -143,8 +151,23 @@ int staging_prepare_locked(Staging &s) {
   TWG_HIP_TRY(hipHostMalloc((void **)&s.base, s.chunk * s.slots, hipHostMallocDefault));
   for (int i = 0; i < s.slots; ++i)
     TWG_HIP_TRY(hipEventCreateWithFlags(&s.ev[i], hipEventDisableTiming));
+  TWG_HIP_TRY(hipHostMalloc((void **)&s.mailbox, kMailboxBytes + 64,
+                            hipHostMallocCoherent | hipHostMallocMapped));
+  TWG_HIP_TRY(hipHostGetDevicePointer(&s.mailbox_dev, s.mailbox, 0));
+  std::memset(s.mailbox, 0, kMailboxBytes + 64);
   s.ready = true;
   return 0;
+}
+
+// Copy n <= kMailboxBytes bytes into the mailbox, then publish the sequence number.
+// One wavefront, so the release below orders every lane's payload stores.
+__global__ __launch_bounds__(64) void mailbox_kernel(uint8_t *box, const uint8_t *src, uint32_t n,
+                                                     uint32_t seq) {
+  for (uint32_t i = threadIdx.x; i < n; i += 64) box[i] = src[i];
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(box + kMailboxBytes), seq, __ATOMIC_RELEASE,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+  }
 }
 
 __global__ void fill_bytes_kernel(uint8_t *dst, uint8_t v, size_t n) {
@@ -429,6 +452,24 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   }
   char *dst = static_cast<char *>(dst_host);
   const char *src = static_cast<const char *>(src_dev);
+  if (nbytes <= kMailboxBytes) {
+    const uint32_t seq = ++st.mailbox_seq;
+    mailbox_kernel<<<1, 64, 0, s>>>(reinterpret_cast<uint8_t *>(st.mailbox_dev),
+                                    reinterpret_cast<const uint8_t *>(src), (uint32_t)nbytes, seq);
+    TWG_HIP_TRY(hipGetLastError());
+    const uint32_t *flag = reinterpret_cast<const uint32_t *>(st.mailbox + kMailboxBytes);
+    bool seen = false;
+    for (int i = 0; i < kMailboxSpins && !seen; ++i) {
+      seen = __atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq;
+      if (!seen) _mm_pause();
+    }
+    if (!seen) {  // a long queue ahead of the kernel, or a failed launch: wait properly
+      TWG_HIP_TRY(hipStreamSynchronize(s));
+      if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) return (int)hipErrorUnknown;
+    }
+    std::memcpy(dst, st.mailbox, nbytes);
+    return 0;
+  }
   const size_t nchunks = (nbytes + st.chunk - 1) / st.chunk;
   auto chunk_len = [&](size_t c) {
     size_t off = c * st.chunk;
