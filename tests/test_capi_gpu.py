@@ -484,11 +484,14 @@ def test_masked_select_bernoulli(twg, n, p):
 @pytest.mark.parametrize("n,p,out_offset", [
     (1 << 25, 0.5, 0), ((1 << 25) + 3 * 131072 + 12345, 0.5, 1), ((1 << 25) + 5, 0.99, 31),
     ((1 << 25) + 8191, 0.01, 0), ((1 << 25) + 8191, 0.001, 7), ((1 << 25) + 140000, 1.0, 3),
-    ((1 << 25) + 140000, 0.0, 0), ((1 << 25) + 40000, -1.0, 17), ((1 << 24) + 70000, 0.5, 0)])
+    ((1 << 25) + 140000, 0.0, 0), ((1 << 25) + 40000, -1.0, 17), ((1 << 24) + 70000, 0.5, 0),
+    ((1 << 23) + 65536 + 5, 0.5, 9), ((1 << 23) - 1, 0.99, 2), ((1 << 22) + 3, -1.0, 30),
+    (1 << 21, 0.5, 1)])
 def test_masked_select_large_tiles(twg, n, p, out_offset):
-    # >= 2^25 elements take the streaming kernel with 131072-element tiles; a remainder
-    # below one big tile goes to a second launch that continues from the first one's
-    # count.  A shifted output pointer moves every wavefront's first and last line.
+    # From 2^21 elements the streaming kernel runs (16384-, 65536- and, from 2^25,
+    # 131072-element tiles); a remainder below one of its tiles goes to a second launch
+    # that continues from the first one's count.  A shifted output pointer moves every
+    # wavefront's first and last line.
     _say(f"masked_select large n={n} p={p} out_offset={out_offset}")
     x = W.select_source(n, seed=4)
     if p < 0:

@@ -492,14 +492,50 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     if (sel[k]) out[wpos + loff[k]] = vals[k];
 }
 
-// Tile shapes of the fast variants: 131072-element tiles (1024 lanes, 32 steps per
-// wavefront) once there is one per CU, 8192-element tiles (256 lanes) below that and
+// Tile shapes of the fast variants.  The streaming kernel wants about one tile per CU
+// or more and as few tickets as that allows: 131072-element tiles from 2^25 elements,
+// 65536 from 2^23, 16384 from 2^21 (measured: each is 1.2-1.8x faster in its range than
+// its neighbours); 8192-element tiles of the stage-then-write variant below that and
 // for what the big tiles leave over.
-constexpr int kBigWaves = 16, kBigGroups = 4;
 constexpr int kSmallWaves = 4;
-constexpr int64_t kBigTile = (int64_t)256 * 8 * kBigGroups * kBigWaves;
 constexpr int64_t kSmallTile = (int64_t)kWaveElems * kSmallWaves;
-constexpr int64_t kBigMinElems = kBigTile * 256;  // 2^25
+constexpr int64_t kStreamMinElems = int64_t(1) << 21;
+
+struct MsLaunch {
+  float *out;
+  int64_t *d_count;
+  const float *src;
+  const uint8_t *mask;
+  int64_t numel;
+  uint32_t *ticket;  // [0] streaming launch, [1] remainder launch
+  int64_t *carry;    // count handed from the first launch to the second
+  uint64_t *status;
+  void *scratch;
+  twg_stream_t stream;
+};
+
+// Full tiles go through the streaming kernel; what is left (less than one of its tiles)
+// is compacted by a second launch of the tile variant that starts from the first
+// launch's total.
+template <int WAVES, int GROUPS>
+int launch_stream(const MsLaunch &m) {
+  constexpr int64_t kTile = (int64_t)256 * 8 * GROUPS * WAVES;
+  const int64_t nbig = m.numel / kTile;
+  const int64_t rem = m.numel - nbig * kTile;
+  const int64_t nrem = (rem + kSmallTile - 1) / kSmallTile;
+  if (nbig > INT32_MAX) return TWG_E_UNSUPPORTED;
+  int rc = twg_fill_bytes(m.scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (size_t)(nbig + nrem),
+                          m.stream);
+  if (rc) return rc;
+  hipStream_t s = resolve_stream(m.stream);
+  ms_compact_stream<WAVES, GROUPS><<<(unsigned)nbig, WAVES * 64, 0, s>>>(
+      m.out, rem ? m.carry : m.d_count, m.src, m.mask, (uint32_t)nbig, m.ticket, m.status);
+  if (rem)
+    ms_compact_vec<kSmallWaves><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
+        m.out, m.d_count, m.src + nbig * kTile, m.mask + nbig * kTile, rem, (uint32_t)nrem,
+        m.ticket + 1, m.status + nbig, m.carry);
+  return (int)hipGetLastError();
+}
 
 }  // namespace
 }  // namespace twg
@@ -538,7 +574,6 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
   const bool vec4 = dense && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(mask) % 4 == 0 &&
                     reinterpret_cast<uintptr_t>(out) % 4 == 0;
-  const bool big = vec4 && g.numel >= kBigMinElems;
 
   // scratch: [0] ticket, [4] ticket of the remainder launch, [8] carry between the
   // two launches, [256...] one status word per tile
@@ -547,24 +582,11 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
   uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
   auto tiles_of = [](int64_t n, int64_t tile) { return (n + tile - 1) / tile; };
 
-  if (big) {
-    // Full 131072-element tiles go through the streaming kernel; what is left (less
-    // than one big tile) is compacted by a second launch of the tile variant that
-    // starts from the first launch's total.
-    const int64_t nbig = g.numel / kBigTile;
-    const int64_t rem = g.numel - nbig * kBigTile;
-    const int64_t nrem = tiles_of(rem, kSmallTile);
-    if (nbig > INT32_MAX) return TWG_E_UNSUPPORTED;
-    if ((rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (size_t)(nbig + nrem),
-                             stream)))
-      return rc;
-    ms_compact_stream<kBigWaves, kBigGroups><<<(unsigned)nbig, kBigWaves * 64, 0, s>>>(
-        out, rem ? carry : d_count, src, mask, (uint32_t)nbig, ticket, status);
-    if (rem)
-      ms_compact_vec<kSmallWaves><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
-          out, d_count, src + nbig * kBigTile, mask + nbig * kBigTile, rem, (uint32_t)nrem,
-          ticket + 1, status + nbig, carry);
-    return (int)hipGetLastError();
+  if (vec4 && g.numel >= kStreamMinElems) {
+    const MsLaunch m{out, d_count, src, mask, g.numel, ticket, carry, status, scratch, stream};
+    if (g.numel >= (int64_t(1) << 25)) return launch_stream<16, 4>(m);
+    if (g.numel >= (int64_t(1) << 23)) return launch_stream<16, 2>(m);
+    return launch_stream<8, 1>(m);
   }
 
   const int64_t tile = vec4 ? kSmallTile : (int64_t)kMsMinTile;
