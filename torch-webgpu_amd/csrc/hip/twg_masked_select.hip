@@ -14,17 +14,18 @@
 //   * the tile total is published at once as an AGGREGATE status word; wave 0
 //     then looks back over 256 predecessors per round (decoupled look-back) until
 //     it meets an INCLUSIVE word, and publishes its own inclusive prefix;
-//   * source values are fetched only where the lane has a selection bit set; three
-//     64-wide ballots of the lane counts plus mbcnt give each lane its offset, the
-//     values are compacted in LDS at the 16-byte phase they will have in memory
-//     and written as aligned float4s.
+//   * a source float4 is fetched from HBM only where the lane has a selection bit set;
+//     three 64-wide ballots of the lane counts plus mbcnt give each lane its offset, the
+//     values are compacted in LDS at the phase they will have in memory and written
+//     as aligned float4s.
 // A status word packs {flag:2, value:62} so one relaxed agent-scope 64-bit
 // load/store carries everything; no fences are needed because no other memory
 // is communicated between tiles.
 //
-// Three facts about MI355X shape the large-input variant.  Same-address agent-scope
-// atomics retire at about one per 7 ns, so the ticket must not be paid 32768
-// times for 2^28 elements: its tiles are 131072 elements.  A wavefront that mixes
+// Three facts about MI355X shape the streaming variant (inputs from 2^21 elements).
+// Same-address agent-scope atomics retire at about one per 7 ns, so the ticket must not
+// be paid 32768 times for 2^28 elements: its tiles are 131072 elements (smaller for
+// smaller inputs, about one tile per CU).  A wavefront that mixes
 // loads and stores in a loop only keeps its loads in flight if the compiler can
 // count them, so its loads are unconditional (a lane with nothing selected reads
 // one shared dummy address).  And stores that leave partial 128-byte lines behind
@@ -38,7 +39,7 @@
 namespace twg {
 namespace {
 
-constexpr int kSteps = 8;           // steps of 256 elements per wavefront and sub-tile
+constexpr int kSteps = 8;           // steps of 256 elements per wavefront (tile variants)
 constexpr int kWaveElems = 256 * kSteps;
 constexpr int kScalarWaves = 4;     // fallback variants: one element per lane
 constexpr int kMsMinTile = 64 * kScalarWaves * kSteps;  // smallest tile of any variant
