@@ -434,3 +434,13 @@ def test_dtype_conversions_stay_on_the_device():
     # the path's own ops accept the converted tensors
     x = torch.randn(1000, generator=g, dtype=torch.float64)
     assert bit_equal((dev(x).float() + dev(x).float()).cpu(), x.float() + x.float())
+
+
+def test_reshape_of_strided_int64_upload():  # tests/test_reshape.py:6-14
+    storage = torch.arange(200, device="cpu")
+    a_cpu = torch.as_strided(storage, size=(2, 3, 4), stride=(20, 6, 1))
+    a = a_cpu.to("webgpu")
+    with torch.no_grad():
+        b = a.reshape((4, 6))
+    assert b.shape == (4, 6) and b.dtype == torch.int64 and b.device.type == "webgpu"
+    assert torch.equal(b.to("cpu"), a_cpu.reshape((4, 6)))
