@@ -116,11 +116,21 @@ __device__ __forceinline__ TO apply(const Op &op, TA a, TB b) {
 // ------------------------------------------------------------- ew_contig
 // One pack per lane, no loop: on MI355X a grid of very many short-lived blocks
 // streams faster (add: 6.4-6.7 TB/s) than a persistent grid-stride loop sized to
-// the 256 CUs (5.4 TB/s).  Block size matters too: single-wavefront blocks give add
-// 83% of peak against 80% for 256 lanes, while kernels whose output is narrower
-// than their input (compares: one dword of bools per lane) or wider (bool -> float32)
-// do best with 1024 lanes (ne.Scalar: 78% at 256, 80% at 1024; bool -> float32: 66% at
-// 64, 71% at 256, 74.5% at 1024).
+// the 256 CUs (5.4 TB/s).  Block size matters too, and the best one was measured per
+// shape of traffic at 2^28 elements:
+//   same width in and out (add, activations, and): 64 lanes (add 83% of peak, 80% at 256);
+//   two float4 in, one dword of bools out (eq): 64 lanes (83%; 81% at 256, 80% at 1024);
+//   8 bytes out per lane (float32 -> half): 64 lanes (87%; 82% at 256);
+//   one pack in, at most a dword out (ne.Scalar, float32 -> bool): 1024 lanes (80%;
+//     78-79.5% at 128..512; a 64-lane block moves too little, 73%: the grid then
+//     launches no faster than ~4.5 blocks per ns);
+//   output wider than input (bool -> float32): 1024 lanes (74.5%; 71% at 256, 66% at 64).
+template <int NIN, int VEC, typename TO, typename TA>
+constexpr int contig_block_size() {
+  if (sizeof(TO) > sizeof(TA)) return 1024;
+  if (NIN == 1 && sizeof(TO) * VEC <= 4) return 1024;
+  return 64;
+}
 
 template <int THREADS, int NIN, int VEC, bool STREAM, typename Op, typename TO, typename TA,
           typename TB>
@@ -139,9 +149,10 @@ __global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const
 #pragma unroll
     for (int k = 0; k < VEC; ++k)
       r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
-    // the nontemporal hint pays for 16-byte stores only: one dword of bools per lane
-    // streams faster with a plain store (ne: 83% vs 79% of peak)
-    store_pack<STREAM && sizeof(PO) == 16>(reinterpret_cast<PO *>(out) + i, r);
+    // the nontemporal hint pays for stores of 8 and 16 bytes per lane (float32 -> half:
+    // 87% vs 84% of peak); one dword of bools per lane streams faster with a plain store
+    // (ne: 83% vs 79%)
+    store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
   }
   if constexpr (VEC > 1) {  // the last numel % VEC elements
     if (blockIdx.x == gridDim.x - 1) {
@@ -646,7 +657,7 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
                         (NIN == 1 || aligned_to(b, sizeof(TB) * VEC));
     const bool stream =
         g.numel * (int64_t)(sizeof(TO) + sizeof(TA) + (NIN == 2 ? sizeof(TB) : 0)) > kStreamBytes;
-    constexpr int kBlock = sizeof(TO) != sizeof(TA) ? 1024 : 64;
+    constexpr int kBlock = contig_block_size<NIN, VEC, TO, TA>();
     const int64_t packs = vec_ok ? (g.numel + VEC - 1) / VEC : g.numel;
     const int64_t blocks = (packs + kBlock - 1) / kBlock;
     if (blocks > INT32_MAX) return TWG_E_UNSUPPORTED;
