@@ -118,3 +118,27 @@ def test_full_masked_select(twg, kind):
     v2, k2 = H.masked_select(idx_src[:w], m[:w])
     assert k2 == int(m[:w].sum())
     assert bool((v2[1:] > v2[:-1]).all())
+
+
+def test_beyond_32bit_element_indices(twg):
+    # 2^31 + 4099 elements (8 GiB per fp32 operand): element indices and byte offsets no
+    # longer fit 32 bits anywhere; the reference stops at u32 offsets
+    # (csrc/ops/binary.h:108-124).  add, eq and masked_select against ATen bit for bit.
+    n = (1 << 31) + 4099
+    g = torch.Generator().manual_seed(3)
+    _say("beyond 2^31: generating")
+    a = torch.rand(n, generator=g)
+    b = torch.rand(n, generator=g)
+    _say("  add")
+    got = H.add(a, b)
+    assert torch.equal(got, a + b)
+    del got
+    _say("  eq")
+    b[::3] = a[::3]
+    m = torch.eq(a, b)
+    assert torch.equal(H.binary("twg_eq_f32", a, b, out_dtype=torch.bool), m)
+    del b
+    _say("  masked_select")
+    vals, k = H.masked_select(a, m)
+    ref = torch.masked_select(a, m)
+    assert k == ref.numel() and torch.equal(vals, ref)
