@@ -505,6 +505,31 @@ def test_masked_select_large_tiles(twg, n, p, out_offset):
     assert bit_equal(vals, torch.masked_select(x, m))
 
 
+def test_masked_select_streaming_edge_patterns(twg):
+    # masks that leave wavefronts, whole tiles or all but a few elements empty, and runs
+    # shorter than a 128-byte line, for each streaming tile size; every output phase
+    g = torch.Generator().manual_seed(12)
+    for n in ((1 << 21) + 12345, (1 << 23) + 777, (1 << 25) + 131072 + 9):
+        x = W.select_source(n, seed=4)
+        idx = torch.arange(n)
+        patterns = {
+            "one in 100000": idx % 100000 == 7,
+            "first only": idx == 0,
+            "last only": idx == n - 1,
+            "3 of 5003": idx % 5003 < 3,
+            "33 of 40000": idx % 40000 < 33,
+            "around tile edges": ((idx + 2) % 16384) < 4,
+            "second half": idx >= n // 2,
+            "one wavefront's span": (idx >= 70000) & (idx < 70000 + 2048),
+        }
+        for name, m in patterns.items():
+            ref = torch.masked_select(x, m)
+            for off in (0, 1, 31):
+                _say(f"masked_select pattern n={n} {name} out_offset={off}")
+                vals, k = H.masked_select(x, m, out_offset=off)
+                assert k == ref.numel() and bit_equal(vals, ref), (n, name, off)
+
+
 def test_masked_select_clustered_and_empty(twg):
     n = (1 << 22) + 1234
     x = W.select_source(n, seed=4)
