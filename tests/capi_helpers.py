@@ -48,11 +48,22 @@ class Uploaded:
         return ctypes.c_void_p(self.buf.ptr + self.off)
 
     def fetch(self):
-        """Download the storage and return a tensor with the original geometry."""
+        """Download the storage and return a tensor with the original geometry.  Storage
+        elements that do not belong to the view must come back exactly as uploaded."""
         st_bytes = self.t.untyped_storage().nbytes()
         raw = self.buf.download((st_bytes,), torch.uint8)
         out = torch.empty(0, dtype=self.t.dtype)
         out.set_(raw.untyped_storage(), self.t.storage_offset(), self.t.shape, self.t.stride())
+        isz = self.t.element_size()
+        n_store = st_bytes // isz
+        if self.t.numel() < n_store:
+            before = torch.empty(0, dtype=torch.uint8).set_(self.t.untyped_storage())[:n_store * isz]
+            inside = torch.zeros(n_store, dtype=torch.bool)
+            where = torch.arange(n_store).as_strided(self.t.shape, self.t.stride(), self.t.storage_offset())
+            inside[where.reshape(-1)] = True
+            outside = (~inside).repeat_interleave(isz)
+            assert torch.equal(raw[:n_store * isz][outside], before[outside]), \
+                "elements of the output's storage outside the view were written"
         return out
 
 
@@ -97,9 +108,10 @@ def add(a, b, alpha=1.0, out=None):
     return binary("twg_add_f32", a, b, out=out, extra=(ctypes.c_float(alpha),))
 
 
-def masked_select(x, mask, scratch_bytes=None, out_offset=0):
+def masked_select(x, mask, scratch_bytes=None, out_offset=0, check_guard=False):
     """Returns (values, count) from twg_masked_select_f32.  out_offset (in floats)
-    shifts the output pointer off its 128-byte alignment."""
+    shifts the output pointer off its 128-byte alignment.  With check_guard the output
+    buffer is pre-filled and every byte outside the k results must come back untouched."""
     L = capi.load()
     shape = torch.broadcast_shapes(x.shape, mask.shape)
     xe, me = _expanded(shape, x, mask)
@@ -107,7 +119,9 @@ def masked_select(x, mask, scratch_bytes=None, out_offset=0):
     for s in shape:
         n *= s
     ux, um = Uploaded(x), Uploaded(mask)
-    out = capi.DeviceBuffer(max(4 * n, 4) + 4 * out_offset)
+    out = capi.DeviceBuffer(max(4 * n, 4) + 4 * out_offset + 256)
+    if check_guard:
+        capi.check(L.twg_fill_bytes(out.ptr, 0xAB, out.nbytes, None))
     cnt = capi.DeviceBuffer(8)
     need = L.twg_masked_select_scratch_bytes(n)
     scratch = capi.DeviceBuffer(need if scratch_bytes is None else max(scratch_bytes, 8))
@@ -117,6 +131,11 @@ def masked_select(x, mask, scratch_bytes=None, out_offset=0):
                                  None)
     capi.check(rc)
     k = int(cnt.download((1,), torch.int64)[0])
+    if check_guard:
+        raw = out.download((out.nbytes,), torch.uint8)
+        lo, hi = 4 * out_offset, 4 * (out_offset + k)
+        assert bool((raw[:lo] == 0xAB).all()), "bytes before the output were written"
+        assert bool((raw[hi:] == 0xAB).all()), "bytes after the k results were written"
     vals = (out.download((k,), torch.float32, byte_offset=4 * out_offset) if k
             else torch.empty(0, dtype=torch.float32))
     return vals, k

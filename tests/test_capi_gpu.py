@@ -474,7 +474,7 @@ def test_masked_select_bernoulli(twg, n, p):
     _say(f"masked_select n={n} p={p}")
     x = W.select_source(n, seed=4)
     m = W.bernoulli_mask(n, p, seed=n % 1000) if 0.0 < p < 1.0 else torch.full((n,), p == 1.0)
-    vals, k = H.masked_select(x, m)
+    vals, k = H.masked_select(x, m, check_guard=True)
     ref = oracle.masked_select(x, m)
     assert k == int(m.sum()) == ref.numel()
     assert bit_equal(vals, ref)
@@ -500,7 +500,7 @@ def test_masked_select_large_tiles(twg, n, p, out_offset):
         m = W.bernoulli_mask(n, p, seed=11)
     else:
         m = torch.full((n,), p == 1.0)
-    vals, k = H.masked_select(x, m, out_offset=out_offset)
+    vals, k = H.masked_select(x, m, out_offset=out_offset, check_guard=True)
     assert k == int(m.sum())
     assert bit_equal(vals, torch.masked_select(x, m))
 
@@ -526,7 +526,7 @@ def test_masked_select_streaming_edge_patterns(twg):
             ref = torch.masked_select(x, m)
             for off in (0, 1, 31):
                 _say(f"masked_select pattern n={n} {name} out_offset={off}")
-                vals, k = H.masked_select(x, m, out_offset=off)
+                vals, k = H.masked_select(x, m, out_offset=off, check_guard=True)
                 assert k == ref.numel() and bit_equal(vals, ref), (n, name, off)
 
 
