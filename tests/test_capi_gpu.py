@@ -549,14 +549,14 @@ def test_masked_select_misaligned_broadcast_strided(twg):
     m = torch.rand(n + 3, generator=g) < 0.4
     # misaligned source / mask pointers (scalar variant of the kernel)
     for xo, mo in ((1, 0), (0, 1), (3, 2)):
-        vals, k = H.masked_select(x[xo:xo + n], m[mo:mo + n])
+        vals, k = H.masked_select(x[xo:xo + n], m[mo:mo + n], check_guard=True)
         assert bit_equal(vals, torch.masked_select(x[xo:xo + n], m[mo:mo + n]))
     # reference known answers: row mask over a matrix, transposed self
     xm = torch.tensor([[0., 1., 2.], [3., 4., 5.]])
     rm = torch.tensor([True, False, True])
-    assert torch.equal(H.masked_select(xm, rm)[0], torch.tensor([0., 2., 3., 5.]))
+    assert torch.equal(H.masked_select(xm, rm, check_guard=True)[0], torch.tensor([0., 2., 3., 5.]))
     xt = torch.arange(6.).view(3, 2).t()
-    assert torch.equal(H.masked_select(xt, rm)[0], torch.tensor([0., 4., 1., 5.]))
+    assert torch.equal(H.masked_select(xt, rm, check_guard=True)[0], torch.tensor([0., 4., 1., 5.]))
     # larger broadcast / strided cases against the oracle and ATen
     x3 = torch.rand(37, 1, 50, generator=g)
     m3 = torch.rand(1, 11, 50, generator=g) < 0.5
