@@ -287,7 +287,9 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   int64_t k = 0;  // the output shape depends on the data: this read is the op's one sync point
   TWG_CHECK(twg_memcpy_d2h(&k, count_dev, sizeof(k), nullptr));
   TORCH_CHECK(k >= 0 && k <= n, "webgpu masked_select: implausible count ", k);
-  if (k * 4 <= n) {  // do not pin a source-sized block under a small result
+  // Do not pin a source-sized block under a small result, unless the block is small
+  // anyway (then the extra copy kernel would cost more than the memory is worth).
+  if (k * 4 <= n && n * (int64_t)sizeof(float) > (int64_t(1) << 20)) {
     at::Tensor exact = at::empty({k}, self.options());
     if (k > 0)
       TWG_CHECK(twg_memcpy_d2d(exact.data_ptr(), out.const_data_ptr(), (size_t)k * sizeof(float), nullptr));
