@@ -357,6 +357,15 @@ def test_masked_select_semantics():
     assert torch.equal(torch.masked_select(t, t.ne(0)).to("cpu"), torch.tensor([1.5, -2.0]))
     assert torch.equal(torch.masked_select(t, torch.eq(t, t) & t.ne(0)).to("cpu"),
                        torch.tensor([1.5, -2.0]))
+    # int32 sources are moved bit for bit by the same kernel (patterns that would be NaNs
+    # or subnormals as floats included); other widths are refused
+    ints = torch.randint(-2 ** 31, 2 ** 31 - 1, (70001,), dtype=torch.int64).to(torch.int32)
+    ints[:4] = torch.tensor([0x7FC00001, -0x00800000, 1, -1], dtype=torch.int32)
+    im = W.bernoulli_mask(70001, 0.3, seed=9)
+    got = torch.masked_select(dev(ints), dev(im))
+    assert got.dtype == torch.int32 and torch.equal(got.cpu(), torch.masked_select(ints, im))
+    with pytest.raises(RuntimeError, match="float32 and int32"):
+        torch.masked_select(dev(ints.long()), dev(im))
 
 
 def test_random_views_through_the_dispatcher():

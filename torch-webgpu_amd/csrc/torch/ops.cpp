@@ -264,7 +264,9 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   // (csrc/bindings.cpp:42).
   TORCH_CHECK(mask.scalar_type() == at::kBool, "masked_select: expected BoolTensor for mask");
   require_on_device(self, "masked_select");
-  TORCH_CHECK(self.scalar_type() == at::kFloat, "webgpu masked_select: only float32 sources are supported, got ",
+  // The kernel moves 4-byte elements without looking at them, so int32 rides along.
+  TORCH_CHECK(self.scalar_type() == at::kFloat || self.scalar_type() == at::kInt,
+              "webgpu masked_select: only float32 and int32 sources are supported, got ",
               self.scalar_type());
   at::Tensor m = is_webgpu(mask) ? mask : mask.to(self.device());
   auto expanded = at::expand_outplace(m, self);
@@ -281,7 +283,8 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   auto *count_dev = static_cast<int64_t *>(work.data_ptr());
   void *scratch = static_cast<char *>(work.data_ptr()) + 256;
   at::Tensor out = at::empty({n}, self.options());
-  TWG_CHECK(twg_masked_select_f32(out.data_ptr<float>(), count_dev, se.const_data_ptr<float>(),
+  TWG_CHECK(twg_masked_select_f32(static_cast<float *>(out.data_ptr()), count_dev,
+                                  static_cast<const float *>(se.const_data_ptr()),
                                   static_cast<const uint8_t *>(me.const_data_ptr()), &it, scratch,
                                   scratch_bytes, nullptr));
   int64_t k = 0;  // the output shape depends on the data: this read is the op's one sync point
