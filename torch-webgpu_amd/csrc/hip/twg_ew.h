@@ -174,21 +174,15 @@ struct RowGeom {
   int64_t len;               // extent of dimension 0
   uint32_t chunks_per_row;   // blocks along one row
   int32_t nouter;            // remaining dimensions
-  uint32_t reused;           // bit k: operand k is the same row for every block (a bias)
   int64_t oshape[TWG_MAX_DIMS - 1];
   int64_t ostride[3][TWG_MAX_DIMS - 1];
 };
 
-// A row every block re-reads should stay in L2: streaming hints only for the rest.
-template <bool STREAM, typename P>
-__device__ __forceinline__ P load_row_pack(const P *p, bool reused) {
-  if constexpr (STREAM) {
-    if (!reused) return load_pack<true>(p);
-  }
-  return load_pack<false>(p);
-}
-
-template <int THREADS, int NIN, int VEC, int UNROLL, bool STREAM, bool A_BC, bool B_BC, typename Op,
+// HINTS says which accesses carry the nontemporal hint: bit 0 the store, bit 1 operand a,
+// bit 2 operand b.  A row that every block re-reads (a bias) keeps default caching so it
+// stays in L2; which operands that is has to be a compile-time fact, because a run-time
+// choice between a hinted and a plain load of one address is folded into one plain load.
+template <int THREADS, int NIN, int VEC, int UNROLL, int HINTS, bool A_BC, bool B_BC, typename Op,
           typename TO, typename TA, typename TB>
 __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
                                                     Op op) {
@@ -225,9 +219,9 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
     const int64_t e = e0 + (int64_t)u * THREADS * VEC;
     if (e < g.len) {
       if constexpr (!A_BC)
-        va[u] = load_row_pack<STREAM>(reinterpret_cast<const PA *>(arow + e), g.reused & 2u);
+        va[u] = load_pack<(HINTS & 2) != 0>(reinterpret_cast<const PA *>(arow + e));
       if constexpr (NIN == 2 && !B_BC)
-        vb[u] = load_row_pack<STREAM>(reinterpret_cast<const PB *>(brow + e), g.reused & 4u);
+        vb[u] = load_pack<(HINTS & 4) != 0>(reinterpret_cast<const PB *>(brow + e));
     }
   }
 #pragma unroll
@@ -241,7 +235,7 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
         const TB y = (NIN == 2) ? (B_BC ? bbc : vb[u].v[k]) : TB();
         r.v[k] = apply<NIN, Op, TO, TA, TB>(op, x, y);
       }
-      store_pack<STREAM && sizeof(PO) == 16>(reinterpret_cast<PO *>(orow + e), r);
+      store_pack<(HINTS & 1) != 0 && sizeof(PO) == 16>(reinterpret_cast<PO *>(orow + e), r);
     }
   }
 }
@@ -534,18 +528,24 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
     rg.oshape[d - 1] = g.shape[d];
     for (int o = 0; o < 3; ++o) rg.ostride[o][d - 1] = g.stride[o][d];
   }
+  bool reused[3] = {false, false, false};  // operand k is the same row for every block
   for (int o = 1; o <= NIN; ++o) {
-    bool same_row = true;
-    for (int d = 1; d < g.ndim; ++d) same_row = same_row && g.stride[o][d] == 0;
-    if (same_row) rg.reused |= 1u << o;
+    reused[o] = true;
+    for (int d = 1; d < g.ndim; ++d) reused[o] = reused[o] && g.stride[o][d] == 0;
   }
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
-  if (stream)
-    ew_rows<kBlock, NIN, VEC, U, true, A_BC, B_BC, Op, TO, TA, TB>
-        <<<(unsigned)(cpr * rows), kBlock, 0, s>>>(out, a, b, rg, op);
+  const unsigned grid = (unsigned)(cpr * rows);
+#define TWG_LAUNCH_ROWS(HINTS) \
+  ew_rows<kBlock, NIN, VEC, U, HINTS, A_BC, B_BC, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, rg, op)
+  if (!stream)
+    TWG_LAUNCH_ROWS(0);
+  else if (reused[1])
+    TWG_LAUNCH_ROWS(1 | 4);
+  else if (NIN == 2 && reused[2])
+    TWG_LAUNCH_ROWS(1 | 2);
   else
-    ew_rows<kBlock, NIN, VEC, U, false, A_BC, B_BC, Op, TO, TA, TB>
-        <<<(unsigned)(cpr * rows), kBlock, 0, s>>>(out, a, b, rg, op);
+    TWG_LAUNCH_ROWS(1 | 2 | 4);
+#undef TWG_LAUNCH_ROWS
   return (int)hipGetLastError();
 }
 
