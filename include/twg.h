@@ -234,6 +234,18 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
                           const uint8_t *mask, const twg_iter_t *it, void *scratch,
                           size_t scratch_bytes, twg_stream_t stream);
 
+/* The same compaction, with K delivered to the host: *count_host is valid when the
+ * call returns, while the writes to `out` are only ordered on `stream` like any
+ * other launch (work queued afterwards sees them).  The kernel stores K into pinned
+ * host memory the moment the last tile knows it and the host polls that word, which
+ * saves the separate read-back of twg_masked_select_f32 + twg_memcpy_d2h (one
+ * launch and one wait per call).  This is what the masked_select registration
+ * calls: it needs K to shape the result (csrc/bindings.cpp:42 reaches the same
+ * point through the CPU fallback). */
+int twg_masked_select_f32_count(float *out, int64_t *count_host, const float *src,
+                                const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                                size_t scratch_bytes, twg_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

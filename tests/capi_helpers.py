@@ -138,4 +138,14 @@ def masked_select(x, mask, scratch_bytes=None, out_offset=0, check_guard=False):
         assert bool((raw[hi:] == 0xAB).all()), "bytes after the k results were written"
     vals = (out.download((k,), torch.float32, byte_offset=4 * out_offset) if k
             else torch.empty(0, dtype=torch.float32))
+    if scratch_bytes is None:
+        # the entry point that hands the count to the host must agree bit for bit
+        out2 = capi.DeviceBuffer(out.nbytes)
+        k2 = ctypes.c_int64(-7)
+        capi.check(L.twg_masked_select_f32_count(out2.ptr + 4 * out_offset, ctypes.byref(k2), ux.ptr, um.ptr,
+                                                 ctypes.byref(it), scratch.ptr, scratch.nbytes, None))
+        assert k2.value == k, f"host count {k2.value} != device count {k}"
+        if k:
+            vals2 = out2.download((k,), torch.float32, byte_offset=4 * out_offset)
+            assert torch.equal(vals.view(torch.int32), vals2.view(torch.int32))
     return vals, k

@@ -162,8 +162,11 @@ __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, 
     }
     if (lane == 0) {
       *s_slot = exclusive;
+      // One 8-byte store at system scope: the count may live in host memory that the
+      // host polls while the rest of the grid is still compacting.
       if (tile == ntiles - 1)
-        *d_count = exclusive + (int64_t)tile_total + (carry_in ? *carry_in : 0);
+        __hip_atomic_store(d_count, exclusive + (int64_t)tile_total + (carry_in ? *carry_in : 0),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
   __syncthreads();

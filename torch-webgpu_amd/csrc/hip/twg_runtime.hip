@@ -588,6 +588,40 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   return 0;
 }
 
+int twg_masked_select_f32_count(float *out, int64_t *count_host, const float *src,
+                                const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                                size_t scratch_bytes, twg_stream_t stream) {
+  if (!count_host || !it) return TWG_E_INVALID_ARG;
+  int rc = ensure_init();
+  if (rc) return rc;
+  hipStream_t s = resolve_stream(stream);
+  Staging &st = staging();
+  std::lock_guard<std::mutex> lk(st.mu);
+  if ((rc = staging_prepare_locked(st))) return rc;
+  // The first 8 bytes of the mailbox receive the count.  The sentinel is no valid
+  // count; the kernel replaces it with one 8-byte store.
+  constexpr int64_t kPending = INT64_MIN;
+  int64_t *slot = reinterpret_cast<int64_t *>(st.mailbox);
+  __atomic_store_n(slot, kPending, __ATOMIC_RELEASE);
+  rc = twg_masked_select_f32(out, static_cast<int64_t *>(st.mailbox_dev), src, mask, it, scratch,
+                             scratch_bytes, stream);
+  if (rc) return rc;
+  int64_t k = kPending;
+  if (it->numel != 0) {  // an empty input clears the count bytewise: wait for the stream instead
+    for (int i = 0; i < kMailboxSpins && k == kPending; ++i) {
+      k = __atomic_load_n(slot, __ATOMIC_ACQUIRE);
+      if (k == kPending) _mm_pause();
+    }
+  }
+  if (k == kPending) {
+    TWG_HIP_TRY(hipStreamSynchronize(s));
+    k = __atomic_load_n(slot, __ATOMIC_ACQUIRE);
+    if (k == kPending) return (int)hipErrorUnknown;
+  }
+  *count_host = k;
+  return 0;
+}
+
 int twg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes, twg_stream_t stream) {
   if (nbytes == 0) return 0;
   if (!dst_dev || !src_dev) return TWG_E_INVALID_ARG;

@@ -278,17 +278,15 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   twg_iter_t it;
   fill_iter_logical(se, me, &it);
   const size_t scratch_bytes = twg_masked_select_scratch_bytes(n);
-  // one allocation: [count (8 B, padded to 256) | scratch]
-  at::Tensor work = at::empty({(int64_t)(scratch_bytes + 256)}, self.options().dtype(at::kByte));
-  auto *count_dev = static_cast<int64_t *>(work.data_ptr());
-  void *scratch = static_cast<char *>(work.data_ptr()) + 256;
+  at::Tensor work = at::empty({(int64_t)scratch_bytes}, self.options().dtype(at::kByte));
   at::Tensor out = at::empty({n}, self.options());
-  TWG_CHECK(twg_masked_select_f32(static_cast<float *>(out.data_ptr()), count_dev,
-                                  static_cast<const float *>(se.const_data_ptr()),
-                                  static_cast<const uint8_t *>(me.const_data_ptr()), &it, scratch,
-                                  scratch_bytes, nullptr));
-  int64_t k = 0;  // the output shape depends on the data: this read is the op's one sync point
-  TWG_CHECK(twg_memcpy_d2h(&k, count_dev, sizeof(k), nullptr));
+  // The output shape depends on the data: waiting for the count is the op's one sync
+  // point.  The kernel hands it over through pinned memory as soon as it is known.
+  int64_t k = 0;
+  TWG_CHECK(twg_masked_select_f32_count(static_cast<float *>(out.data_ptr()), &k,
+                                        static_cast<const float *>(se.const_data_ptr()),
+                                        static_cast<const uint8_t *>(me.const_data_ptr()), &it,
+                                        work.data_ptr(), scratch_bytes, nullptr));
   TORCH_CHECK(k >= 0 && k <= n, "webgpu masked_select: implausible count ", k);
   // Do not pin a source-sized block under a small result, unless the block is small
   // anyway (then the extra copy kernel would cost more than the memory is worth).

@@ -59,7 +59,7 @@ SYMBOLS = [
     "twg_add_f32", "twg_add_scalar_f32", "twg_mul_f32", "twg_mul_scalar_f32",
     "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided", "twg_cast",
     "twg_eq_f32", "twg_ne_scalar_f32", "twg_and_u8",
-    "twg_masked_select_scratch_bytes", "twg_masked_select_f32",
+    "twg_masked_select_scratch_bytes", "twg_masked_select_f32", "twg_masked_select_f32_count",
 ]
 
 _lib = None
@@ -114,6 +114,7 @@ def load():
     L.twg_masked_select_scratch_bytes.argtypes = [i64]
     L.twg_masked_select_scratch_bytes.restype = sz
     L.twg_masked_select_f32.argtypes = [vp, vp, vp, vp, ip, vp, sz, vp]
+    L.twg_masked_select_f32_count.argtypes = [vp, ctypes.POINTER(ctypes.c_int64), vp, vp, ip, vp, sz, vp]
     _lib = L
     return L
 
