@@ -148,9 +148,9 @@ def main():
     def run_ms(mask_buf=None):
         """The op as the dispatcher runs it: compaction with the count handed to the host
         (the call returns once the count is known; the output is stream ordered)."""
-        capi.check(L.twg_masked_select_f32_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr,
-                                                 (mask_buf or d_m).ptr, ctypes.byref(it),
-                                                 d_scratch.ptr, scratch_bytes, None))
+        capi.check(L.twg_masked_select_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr, 4,
+                                             (mask_buf or d_m).ptr, ctypes.byref(it),
+                                             d_scratch.ptr, scratch_bytes, None))
         return k_host.value
 
     bytes_add = W.BYTES_PER_ELEM["add"] * n
@@ -342,9 +342,9 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         k_host = ctypes.c_int64(-1)
 
         def full():
-            capi.check(L.twg_masked_select_f32_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr,
-                                                     d_mask.ptr, ctypes.byref(it), d_scratch.ptr,
-                                                     scratch_bytes, None))
+            capi.check(L.twg_masked_select_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr, 4,
+                                                 d_mask.ptr, ctypes.byref(it), d_scratch.ptr,
+                                                 scratch_bytes, None))
 
         ms_kernel = time_launches(launch, Wm, K)
         ms_full = time_launches(full, 1, K)

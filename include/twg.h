@@ -229,22 +229,42 @@ size_t twg_masked_select_scratch_bytes(int64_t numel);
  * the broadcast logical shape: stride[TWG_A] addresses src, stride[TWG_B]
  * addresses mask, stride[TWG_OUT] is ignored; dim 0 fastest, so logical index i
  * is the row-major index of the broadcast shape reversed.  Asynchronous: read
- * *d_count with twg_memcpy_d2h. */
+ * *d_count with twg_memcpy_d2h (or call twg_masked_select_count, below). */
 int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
                           const uint8_t *mask, const twg_iter_t *it, void *scratch,
                           size_t scratch_bytes, twg_stream_t stream);
 
-/* The same compaction, with K delivered to the host: *count_host is valid when the
- * call returns, while the writes to `out` are only ordered on `stream` like any
- * other launch (work queued afterwards sees them).  The kernel stores K into pinned
- * host memory the moment the last tile knows it and the host polls that word, which
- * saves the separate read-back of twg_masked_select_f32 + twg_memcpy_d2h (one
- * launch and one wait per call).  This is what the masked_select registration
- * calls: it needs K to shape the result (csrc/bindings.cpp:42 reaches the same
- * point through the CPU fallback). */
-int twg_masked_select_f32_count(float *out, int64_t *count_host, const float *src,
-                                const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                                size_t scratch_bytes, twg_stream_t stream);
+/* The same compaction for elements of `elem_size` = 1, 2, 4 or 8 bytes (moved without
+ * being looked at, so any dtype of that size; the CPU fallback the reference registers,
+ * csrc/bindings.cpp:42, takes every dtype), with K delivered to the host: *count_host
+ * is valid when the call returns, while the writes to `out` are only ordered on `stream`
+ * like any other launch (work queued afterwards sees them).  The kernel stores K into
+ * pinned host memory the moment the last tile knows it and the host polls that word,
+ * which saves the separate read-back of twg_masked_select_f32 + twg_memcpy_d2h (one
+ * launch and one wait per call).  This is what the masked_select registration calls:
+ * it needs K to shape the result.  `out` and `src` must be aligned to elem_size;
+ * 4-byte elements take the same kernels as twg_masked_select_f32. */
+int twg_masked_select_count(void *out, int64_t *count_host, const void *src,
+                            int32_t elem_size, const uint8_t *mask, const twg_iter_t *it,
+                            void *scratch, size_t scratch_bytes, twg_stream_t stream);
+
+/* ------------------------------------------- compare / and for every dtype */
+
+/* out[i] = (a[i] == b[i]) as a 0/1 byte for two operands of one dtype (enum
+ * twg_dtype), ATen's CPU semantics, which are what the reference's fallback gives
+ * (csrc/bindings.cpp:38-39): IEEE for floating types, exact for integers.
+ * TWG_DT_F32 runs the kernel of twg_eq_f32. */
+int twg_eq(uint8_t *out, const void *a, const void *b, int32_t dtype, const twg_iter_t *it,
+           twg_stream_t stream);
+/* out[i] = (a[i] != s) for an operand of `dtype` (csrc/bindings.cpp:36-37).  The scalar
+ * comes twice: s_f is used for floating dtypes (rounded to the dtype first, as ATen
+ * does), s_i for integral ones and bool. */
+int twg_ne_scalar(uint8_t *out, const void *a, int32_t dtype, double s_f, int64_t s_i,
+                  const twg_iter_t *it, twg_stream_t stream);
+/* out[i] = a[i] & b[i] on integers of elem_size = 1, 2, 4 or 8 bytes
+ * (csrc/bindings.cpp:40-41). */
+int twg_and(void *out, const void *a, const void *b, int32_t elem_size, const twg_iter_t *it,
+            twg_stream_t stream);
 
 #ifdef __cplusplus
 }

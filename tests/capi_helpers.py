@@ -109,43 +109,84 @@ def add(a, b, alpha=1.0, out=None):
 
 
 def masked_select(x, mask, scratch_bytes=None, out_offset=0, check_guard=False):
-    """Returns (values, count) from twg_masked_select_f32.  out_offset (in floats)
-    shifts the output pointer off its 128-byte alignment.  With check_guard the output
-    buffer is pre-filled and every byte outside the k results must come back untouched."""
+    """Returns (values, count).  float32 sources go through twg_masked_select_f32 and are
+    cross-checked against twg_masked_select_count; other dtypes go through
+    twg_masked_select_count alone.  out_offset (in elements) shifts the output pointer off
+    its 128-byte alignment.  With check_guard the output buffer is pre-filled and every byte
+    outside the k results must come back untouched."""
     L = capi.load()
     shape = torch.broadcast_shapes(x.shape, mask.shape)
     xe, me = _expanded(shape, x, mask)
     n = 1
     for s in shape:
         n *= s
+    es = x.element_size()
     ux, um = Uploaded(x), Uploaded(mask)
-    out = capi.DeviceBuffer(max(4 * n, 4) + 4 * out_offset + 256)
+    out = capi.DeviceBuffer(max(es * n, es) + es * out_offset + 256)
     if check_guard:
         capi.check(L.twg_fill_bytes(out.ptr, 0xAB, out.nbytes, None))
-    cnt = capi.DeviceBuffer(8)
     need = L.twg_masked_select_scratch_bytes(n)
     scratch = capi.DeviceBuffer(need if scratch_bytes is None else max(scratch_bytes, 8))
+    sb = scratch.nbytes if scratch_bytes is None else scratch_bytes
     it = _iter_for(shape, None, (xe, me), sort_by_out=False)
-    rc = L.twg_masked_select_f32(out.ptr + 4 * out_offset, cnt.ptr, ux.ptr, um.ptr, ctypes.byref(it),
-                                 scratch.ptr, scratch.nbytes if scratch_bytes is None else scratch_bytes,
-                                 None)
-    capi.check(rc)
-    k = int(cnt.download((1,), torch.int64)[0])
+    if x.dtype == torch.float32:
+        cnt = capi.DeviceBuffer(8)
+        capi.check(L.twg_masked_select_f32(out.ptr + es * out_offset, cnt.ptr, ux.ptr, um.ptr,
+                                           ctypes.byref(it), scratch.ptr, sb, None))
+        k = int(cnt.download((1,), torch.int64)[0])
+    else:
+        kh = ctypes.c_int64(-7)
+        capi.check(L.twg_masked_select_count(out.ptr + es * out_offset, ctypes.byref(kh), ux.ptr, es,
+                                             um.ptr, ctypes.byref(it), scratch.ptr, sb, None))
+        k = kh.value
     if check_guard:
         raw = out.download((out.nbytes,), torch.uint8)
-        lo, hi = 4 * out_offset, 4 * (out_offset + k)
+        lo, hi = es * out_offset, es * (out_offset + k)
         assert bool((raw[:lo] == 0xAB).all()), "bytes before the output were written"
         assert bool((raw[hi:] == 0xAB).all()), "bytes after the k results were written"
-    vals = (out.download((k,), torch.float32, byte_offset=4 * out_offset) if k
-            else torch.empty(0, dtype=torch.float32))
-    if scratch_bytes is None:
+    vals = (out.download((k,), x.dtype, byte_offset=es * out_offset) if k
+            else torch.empty(0, dtype=x.dtype))
+    if x.dtype == torch.float32 and scratch_bytes is None:
         # the entry point that hands the count to the host must agree bit for bit
         out2 = capi.DeviceBuffer(out.nbytes)
         k2 = ctypes.c_int64(-7)
-        capi.check(L.twg_masked_select_f32_count(out2.ptr + 4 * out_offset, ctypes.byref(k2), ux.ptr, um.ptr,
-                                                 ctypes.byref(it), scratch.ptr, scratch.nbytes, None))
+        capi.check(L.twg_masked_select_count(out2.ptr + es * out_offset, ctypes.byref(k2), ux.ptr, es,
+                                             um.ptr, ctypes.byref(it), scratch.ptr, scratch.nbytes, None))
         assert k2.value == k, f"host count {k2.value} != device count {k}"
         if k:
-            vals2 = out2.download((k,), torch.float32, byte_offset=4 * out_offset)
+            vals2 = out2.download((k,), torch.float32, byte_offset=es * out_offset)
             assert torch.equal(vals.view(torch.int32), vals2.view(torch.int32))
     return vals, k
+
+
+def compare_eq(a, b):
+    """twg_eq on two CPU tensors of one dtype (broadcast together); returns a bool tensor."""
+    L = capi.load()
+    shape = torch.broadcast_shapes(a.shape, b.shape)
+    out = torch.zeros(shape, dtype=torch.bool)
+    ae, be = _expanded(shape, a, b)
+    ua, ub, uo = Uploaded(a), Uploaded(b), Uploaded(out)
+    it = _iter_for(shape, out, (ae, be), True)
+    capi.check(L.twg_eq(uo.ptr, ua.ptr, ub.ptr, capi.DTYPES[a.dtype], ctypes.byref(it), None))
+    return uo.fetch()
+
+
+def compare_ne_scalar(a, s_f, s_i):
+    L = capi.load()
+    out = torch.zeros(tuple(a.shape), dtype=torch.bool)
+    ua, uo = Uploaded(a), Uploaded(out)
+    it = _iter_for(tuple(a.shape), out, (a,), True)
+    capi.check(L.twg_ne_scalar(uo.ptr, ua.ptr, capi.DTYPES[a.dtype], ctypes.c_double(s_f),
+                               ctypes.c_int64(s_i), ctypes.byref(it), None))
+    return uo.fetch()
+
+
+def bitwise_and(a, b):
+    L = capi.load()
+    shape = torch.broadcast_shapes(a.shape, b.shape)
+    out = torch.zeros(shape, dtype=a.dtype)
+    ae, be = _expanded(shape, a, b)
+    ua, ub, uo = Uploaded(a), Uploaded(b), Uploaded(out)
+    it = _iter_for(shape, out, (ae, be), True)
+    capi.check(L.twg_and(uo.ptr, ua.ptr, ub.ptr, a.element_size(), ctypes.byref(it), None))
+    return uo.fetch()

@@ -340,6 +340,81 @@ def test_cast_float_edge_cases(twg):
         assert rc == 0 and bit_equal(got.nan_to_num(), h.to(torch.float32).nan_to_num())
 
 
+def _compare_source(dtype, n, g):
+    """Few distinct values (so that about a fifth of the pairs match) plus the type's specials."""
+    if dtype == torch.bool:
+        return torch.rand(n, generator=g) < 0.5
+    if dtype in _INT_TYPES:
+        info = torch.iinfo(dtype)
+        t = torch.randint(0, 5, (n,), generator=g).to(dtype)
+        t[:4] = torch.tensor([info.min, info.max, info.min, 0], dtype=dtype)
+        return t
+    t = torch.randint(-2, 3, (n,), generator=g).to(dtype)
+    t[:8] = torch.tensor([0.0, -0.0, float("nan"), float("inf"), -float("inf"), 0.5, 1.0, -1.0]).to(dtype)
+    return t
+
+
+def test_eq_ne_and_every_dtype_match_aten(twg):
+    # twg_eq / twg_ne_scalar / twg_and against ATen's CPU kernels: dense, misaligned,
+    # broadcast and strided operands of every dtype
+    g = torch.Generator().manual_seed(33)
+    n = 50021
+    for dt in _INT_TYPES + _FLOAT_TYPES:
+        _say(f"eq/ne/and {dt}")
+        a, b = _compare_source(dt, n, g), _compare_source(dt, n, g)
+        b[:8] = a[:8].flip(0)  # specials against specials: NaN vs NaN, 0.0 vs -0.0, min vs max
+        b[8:16] = a[8:16]
+        assert torch.equal(H.compare_eq(a, b), torch.eq(a, b)), dt
+        assert torch.equal(H.compare_eq(a[1:], b[:-1]), torch.eq(a[1:], b[:-1])), dt
+        a2, row = a[:50000].view(250, 200), b[:200]
+        assert torch.equal(H.compare_eq(a2, row), torch.eq(a2, row)), dt
+        assert torch.equal(H.compare_eq(a2.t(), b[21:50021].view(200, 250)),
+                           torch.eq(a2.t(), b[21:50021].view(200, 250))), dt
+        if dt in _FLOAT_TYPES:
+            for s in (0.0, 1.0, 0.1, float("nan"), float("inf"), 1.0 + 2 ** -12):
+                # the reference value: ATen rounds the scalar to the tensor's dtype
+                assert torch.equal(H.compare_ne_scalar(a, s, 0), a.ne(s)), (dt, s)
+        elif dt == torch.bool:
+            for s in (0, 1):
+                assert torch.equal(H.compare_ne_scalar(a, 0.0, s), a.ne(bool(s))), (dt, s)
+        else:
+            info = torch.iinfo(dt)
+            for s in (0, 3, info.max, info.min):
+                assert torch.equal(H.compare_ne_scalar(a, 0.0, s), a.ne(s)), (dt, s)
+            assert torch.equal(H.compare_ne_scalar(a2.t(), 0.0, 3), a2.t().ne(3)), dt
+        if dt in _INT_TYPES:
+            x = _compare_source(dt, n, g)
+            if dt not in (torch.bool,):
+                x = torch.randint(0, 1 << 7, (n,), generator=g).to(dt) * (3 if dt != torch.int8 else 1)
+            y = x.flip(0).clone()
+            assert bit_equal(H.bitwise_and(x, y), torch.bitwise_and(x, y)), dt
+            assert bit_equal(H.bitwise_and(x[:50000].view(250, 200).t(), y[:250]),
+                             torch.bitwise_and(x[:50000].view(250, 200).t(), y[:250])), dt
+    L = twg.load()
+    assert L.twg_eq(None, None, None, 99, None, None) == twg.E_INVALID_ARG
+    assert L.twg_and(None, None, None, 3, None, None) == twg.E_UNSUPPORTED
+
+
+@pytest.mark.parametrize("dtype", [torch.bool, torch.uint8, torch.int16, torch.float16, torch.bfloat16,
+                                   torch.int32, torch.int64, torch.float64])
+def test_masked_select_every_element_size(twg, dtype):
+    # elements are moved, not looked at: 1, 2, 4 and 8 bytes, dense, misaligned, broadcast, strided
+    g = torch.Generator().manual_seed(34)
+    for n in (1, 63, 4096, 70001, (1 << 21) + 5):
+        _say(f"masked_select {dtype} n={n}")
+        x = (torch.randn(n, generator=g) * 1000).to(dtype)
+        m = torch.rand(n, generator=g) < 0.4
+        vals, k = H.masked_select(x, m, check_guard=True)
+        assert k == int(m.sum()) and bit_equal(vals, torch.masked_select(x, m)), (dtype, n)
+    x = (torch.randn(40004, generator=g) * 1000).to(dtype)
+    m = torch.rand(40004, generator=g) < 0.5
+    vals, _ = H.masked_select(x[1:40001], m[3:40003], out_offset=1, check_guard=True)
+    assert bit_equal(vals, torch.masked_select(x[1:40001], m[3:40003]))
+    xt = x[:40000].view(100, 400).t()
+    vals, _ = H.masked_select(xt, m[:100])
+    assert bit_equal(vals, torch.masked_select(xt, m[:100]))
+
+
 # ------------------------------------------------------------- activations
 
 def _unary(op, x, **kw):

@@ -319,8 +319,8 @@ def test_mask_ops_config4_reduced():
     assert bit_equal(dev(a).ne(0.0).to("cpu"), a.ne(0.0))
     assert bit_equal(torch.eq(dev(a).view(6, 1), dev(b).view(1, 6)).to("cpu"), torch.eq(a.view(6, 1), b.view(1, 6)))
     assert bit_equal(dev(a).abs().to("cpu"), a.abs())
-    with pytest.raises(RuntimeError):
-        torch.eq(dev(torch.ones(3, dtype=torch.int64)), dev(torch.ones(3, dtype=torch.int64)))
+    i = torch.tensor([1, 2, 1 << 40], dtype=torch.int64)
+    assert bit_equal(torch.eq(dev(i), dev(i.flip(0))).to("cpu"), torch.eq(i, i.flip(0)))
 
 
 @pytest.mark.parametrize("p", [0.0, 0.01, 0.5, 0.99, 1.0])
@@ -358,14 +358,16 @@ def test_masked_select_semantics():
     assert torch.equal(torch.masked_select(t, torch.eq(t, t) & t.ne(0)).to("cpu"),
                        torch.tensor([1.5, -2.0]))
     # int32 sources are moved bit for bit by the same kernel (patterns that would be NaNs
-    # or subnormals as floats included); other widths are refused
+    # or subnormals as floats included), and so are 1-, 2- and 8-byte elements
     ints = torch.randint(-2 ** 31, 2 ** 31 - 1, (70001,), dtype=torch.int64).to(torch.int32)
     ints[:4] = torch.tensor([0x7FC00001, -0x00800000, 1, -1], dtype=torch.int32)
     im = W.bernoulli_mask(70001, 0.3, seed=9)
     got = torch.masked_select(dev(ints), dev(im))
     assert got.dtype == torch.int32 and torch.equal(got.cpu(), torch.masked_select(ints, im))
-    with pytest.raises(RuntimeError, match="float32 and int32"):
-        torch.masked_select(dev(ints.long()), dev(im))
+    got = torch.masked_select(dev(ints.long()), dev(im))
+    assert got.dtype == torch.int64 and torch.equal(got.cpu(), torch.masked_select(ints.long(), im))
+    with pytest.raises(RuntimeError, match="16 bytes"):
+        torch.masked_select(dev(ints.to(torch.complex128)), dev(im))
 
 
 def test_random_views_through_the_dispatcher():
@@ -453,3 +455,47 @@ def test_reshape_of_strided_int64_upload():  # tests/test_reshape.py:6-14
         b = a.reshape((4, 6))
     assert b.shape == (4, 6) and b.dtype == torch.int64 and b.device.type == "webgpu"
     assert torch.equal(b.to("cpu"), a_cpu.reshape((4, 6)))
+
+
+def test_mask_ops_take_every_dtype():
+    # the reference sends eq / ne / bitwise_and / masked_select to ATen's CPU kernels
+    # (csrc/bindings.cpp:36-42), which accept any dtype and promote mixed operands
+    g = torch.Generator().manual_seed(9)
+    ints = (torch.bool, torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64)
+    floats = (torch.float16, torch.bfloat16, torch.float32, torch.float64)
+    n = 3001
+    for dt in ints + floats:
+        a = torch.randint(0, 4, (n,), generator=g).to(dt)
+        b = torch.randint(0, 4, (n,), generator=g).to(dt)
+        wa, wb = a.to("webgpu"), b.to("webgpu")
+        assert torch.equal(torch.eq(wa, wb).to("cpu"), torch.eq(a, b)), dt
+        assert torch.equal(wa.ne(1).to("cpu"), a.ne(1)), dt
+        assert torch.equal(wa.ne(0.5).to("cpu"), a.ne(0.5)), dt
+        m = torch.rand(n, generator=g) < 0.5
+        got = torch.masked_select(wa, m.to("webgpu"))
+        assert got.dtype == dt and torch.equal(got.to("cpu"), torch.masked_select(a, m)), dt
+        if dt in ints:
+            got = torch.bitwise_and(wa, wb)
+            assert got.dtype == dt and torch.equal(got.to("cpu"), torch.bitwise_and(a, b)), dt
+    # mixed dtypes follow ATen's promotion
+    i32 = torch.tensor([1, 2, 3, 16777217], dtype=torch.int32)
+    f32 = torch.tensor([1.0, 2.5, 3.0, 16777216.0])
+    assert torch.equal(torch.eq(i32.to("webgpu"), f32.to("webgpu")).to("cpu"), torch.eq(i32, f32))
+    u8 = torch.tensor([1, 2, 255, 7], dtype=torch.uint8)
+    got = torch.bitwise_and(u8.to("webgpu"), i32.to("webgpu"))
+    assert got.dtype == torch.int32 and torch.equal(got.to("cpu"), torch.bitwise_and(u8, i32))
+    bm = torch.tensor([True, False, True, True])
+    got = torch.bitwise_and(bm.to("webgpu"), u8.to("webgpu"))
+    assert got.dtype == torch.uint8 and torch.equal(got.to("cpu"), torch.bitwise_and(bm, u8))
+    assert torch.equal(bm.to("webgpu").ne(1).to("cpu"), bm.ne(1))
+    with pytest.raises(RuntimeError):
+        torch.bitwise_and(f32.to("webgpu"), f32.to("webgpu"))
+    # the scalar is converted like a C cast: wrapped around for integers
+    w = torch.tensor([44, 1], dtype=torch.uint8)
+    assert torch.equal(w.to("webgpu").ne(300).to("cpu"), w.ne(300))
+    w = torch.tensor([-1, 1], dtype=torch.int8)
+    assert torch.equal(w.to("webgpu").ne(255).to("cpu"), w.ne(255))
+    assert torch.equal(bm.to("webgpu").ne(2).to("cpu"), bm.ne(2))
+    big = torch.tensor([16777217], dtype=torch.int32)
+    assert torch.equal(big.to("webgpu").ne(16777216.0).to("cpu"), big.ne(16777216.0))
+

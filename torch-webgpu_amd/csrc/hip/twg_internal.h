@@ -36,4 +36,12 @@ struct Geom {
 // slots (2 = out + a, 3 = out + a + b).  Returns 0 or TWG_E_INVALID_ARG.
 int canonicalize(const twg_iter_t *it, int nops, Geom *g);
 
+// The compaction behind the masked_select entry points: elements of 1, 2, 4 or 8
+// bytes, count written to *d_count (device memory, or host memory the device can
+// address).  Dense 16-byte-aligned sources of 4-byte elements take the vectorised
+// kernels, everything else the one-element-per-lane kernel.
+int masked_select_launch(void *out, int64_t *d_count, const void *src, int elem_size,
+                         const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                         size_t scratch_bytes, twg_stream_t stream);
+
 }  // namespace twg

@@ -426,10 +426,12 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t
 // -------------------------------------------------------------- fallback variants
 // One element per lane: misaligned pointers (STRIDED = false) or broadcast /
 // strided source and mask addressed through div/mod index math (STRIDED = true).
+// The values are moved as T without being looked at, so T is an unsigned integer of
+// the element's size.
 
-template <bool STRIDED>
+template <bool STRIDED, typename T>
 __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
-    float *out, int64_t *d_count, const float *src, const uint8_t *mask, int64_t n,
+    T *out, int64_t *d_count, const T *src, const uint8_t *mask, int64_t n,
     uint32_t ntiles, uint32_t *ticket, uint64_t *status, MsGeom g) {
   constexpr int kWaveSpan = 64 * kSteps;
   constexpr int kTileElems = kWaveSpan * kScalarWaves;
@@ -485,7 +487,7 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     if (w < wave) wave_base += t;
     tile_total += t;
   }
-  float vals[kSteps];
+  T vals[kSteps];
 #pragma unroll
   for (int k = 0; k < kSteps; ++k)
     if (sel[k]) vals[k] = src[soff[k]];
@@ -554,12 +556,17 @@ size_t twg_masked_select_scratch_bytes(int64_t numel) {
   return kMsHeaderBytes + sizeof(uint64_t) * (size_t)(tiles > 0 ? tiles : 1);
 }
 
-int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const uint8_t *mask,
-                          const twg_iter_t *it, void *scratch, size_t scratch_bytes,
-                          twg_stream_t stream) {
+}  // extern "C"
+
+namespace twg {
+
+int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int elem_size,
+                         const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                         size_t scratch_bytes, twg_stream_t stream) {
   int rc = ensure_init();
   if (rc) return rc;
   if (!it || !d_count) return TWG_E_INVALID_ARG;
+  if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8) return TWG_E_UNSUPPORTED;
   // Only the source and mask strides matter; mirror the source strides into the
   // output slot so they never block a merge of adjacent dimensions.
   twg_iter_t local = *it;
@@ -568,14 +575,18 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
   Geom g;
   if ((rc = canonicalize(&local, 3, &g))) return rc;
   if (g.numel == 0) return twg_fill_bytes(d_count, 0, sizeof(int64_t), stream);
-  if (!out || !src || !mask || !scratch) return TWG_E_INVALID_ARG;
+  if (!out_v || !src_v || !mask || !scratch) return TWG_E_INVALID_ARG;
+  if (reinterpret_cast<uintptr_t>(out_v) % elem_size || reinterpret_cast<uintptr_t>(src_v) % elem_size)
+    return TWG_E_INVALID_ARG;
   if (scratch_bytes < twg_masked_select_scratch_bytes(g.numel)) return TWG_E_SCRATCH_SMALL;
   if (reinterpret_cast<uintptr_t>(scratch) % 8 != 0) return TWG_E_INVALID_ARG;
 
   hipStream_t s = resolve_stream(stream);
   const bool dense =
       g.ndim == 0 || (g.ndim == 1 && g.stride[TWG_A][0] == 1 && g.stride[TWG_B][0] == 1);
-  const bool vec4 = dense && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+  float *out = static_cast<float *>(out_v);  // the fast variants move 4-byte elements
+  const float *src = static_cast<const float *>(src_v);
+  const bool vec4 = elem_size == 4 && dense && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(mask) % 4 == 0 &&
                     reinterpret_cast<uintptr_t>(out) % 4 == 0;
 
@@ -611,14 +622,35 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const 
       mg.sstride[d] = g.stride[TWG_A][d];
       mg.mstride[d] = g.stride[TWG_B][d];
     }
-    if (dense)
-      ms_compact_scalar<false><<<ntiles, kScalarWaves * 64, 0, s>>>(out, d_count, src, mask,
-                                                                    g.numel, ntiles, ticket, status, mg);
-    else
-      ms_compact_scalar<true><<<ntiles, kScalarWaves * 64, 0, s>>>(out, d_count, src, mask,
-                                                                   g.numel, ntiles, ticket, status, mg);
+    auto scalar = [&](auto zero) {
+      using T = decltype(zero);
+      if (dense)
+        ms_compact_scalar<false, T><<<ntiles, kScalarWaves * 64, 0, s>>>(
+            static_cast<T *>(out_v), d_count, static_cast<const T *>(src_v), mask, g.numel, ntiles,
+            ticket, status, mg);
+      else
+        ms_compact_scalar<true, T><<<ntiles, kScalarWaves * 64, 0, s>>>(
+            static_cast<T *>(out_v), d_count, static_cast<const T *>(src_v), mask, g.numel, ntiles,
+            ticket, status, mg);
+    };
+    switch (elem_size) {
+      case 1: scalar(uint8_t{}); break;
+      case 2: scalar(uint16_t{}); break;
+      case 4: scalar(uint32_t{}); break;
+      default: scalar(uint64_t{}); break;
+    }
   }
   return (int)hipGetLastError();
+}
+
+}  // namespace twg
+
+extern "C" {
+
+int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const uint8_t *mask,
+                          const twg_iter_t *it, void *scratch, size_t scratch_bytes,
+                          twg_stream_t stream) {
+  return masked_select_launch(out, d_count, src, 4, mask, it, scratch, scratch_bytes, stream);
 }
 
 }  // extern "C"

@@ -588,9 +588,9 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   return 0;
 }
 
-int twg_masked_select_f32_count(float *out, int64_t *count_host, const float *src,
-                                const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                                size_t scratch_bytes, twg_stream_t stream) {
+int twg_masked_select_count(void *out, int64_t *count_host, const void *src, int32_t elem_size,
+                            const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                            size_t scratch_bytes, twg_stream_t stream) {
   if (!count_host || !it) return TWG_E_INVALID_ARG;
   int rc = ensure_init();
   if (rc) return rc;
@@ -603,8 +603,8 @@ int twg_masked_select_f32_count(float *out, int64_t *count_host, const float *sr
   constexpr int64_t kPending = INT64_MIN;
   int64_t *slot = reinterpret_cast<int64_t *>(st.mailbox);
   __atomic_store_n(slot, kPending, __ATOMIC_RELEASE);
-  rc = twg_masked_select_f32(out, static_cast<int64_t *>(st.mailbox_dev), src, mask, it, scratch,
-                             scratch_bytes, stream);
+  rc = masked_select_launch(out, static_cast<int64_t *>(st.mailbox_dev), src, elem_size, mask, it,
+                            scratch, scratch_bytes, stream);
   if (rc) return rc;
   int64_t k = kPending;
   if (it->numel != 0) {  // an empty input clears the count bytewise: wait for the stream instead

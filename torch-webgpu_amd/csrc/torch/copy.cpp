@@ -25,22 +25,6 @@ bool same_dense_layout(const at::Tensor &a, const at::Tensor &b) {
          a.is_non_overlapping_and_dense();
 }
 
-int twg_dtype_of(at::ScalarType t) {
-  switch (t) {
-    case at::kBool: return TWG_DT_BOOL;
-    case at::kByte: return TWG_DT_U8;
-    case at::kChar: return TWG_DT_I8;
-    case at::kShort: return TWG_DT_I16;
-    case at::kInt: return TWG_DT_I32;
-    case at::kLong: return TWG_DT_I64;
-    case at::kHalf: return TWG_DT_F16;
-    case at::kBFloat16: return TWG_DT_BF16;
-    case at::kFloat: return TWG_DT_F32;
-    case at::kDouble: return TWG_DT_F64;
-    default: return -1;
-  }
-}
-
 bool is_integral_dt(int dt) { return dt <= TWG_DT_I64 || dt == TWG_DT_I8 || dt == TWG_DT_I16; }
 
 void device_to_device(const at::Tensor &dst, const at::Tensor &src);

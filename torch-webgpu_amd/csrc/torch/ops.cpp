@@ -176,25 +176,41 @@ at::Tensor &abs_out(const at::Tensor &self, at::Tensor &out) {
 
 // ----------------------------------------------------------------- bool masks
 
+// The reference runs these three through ATen's CPU kernels (csrc/bindings.cpp:36-41),
+// which take any dtype and promote mixed operands; here the operands are converted to
+// the promoted dtype on the device and compared by a kernel of that dtype.
+
+int known_dtype(at::ScalarType t, const char *op) {
+  const int dt = twg_dtype_of(t);
+  TORCH_CHECK(dt >= 0, "webgpu ", op, ": dtype ", t, " is not supported");
+  return dt;
+}
+
+at::Tensor as_dtype(const at::Tensor &t, at::ScalarType want) {
+  return t.scalar_type() == want ? t : t.to(want);
+}
+
 at::Tensor &eq_tensor_out(const at::Tensor &self, const at::Tensor &other, at::Tensor &out) {
   require_on_device(self, "eq");
   require_on_device(other, "eq");
-  TORCH_CHECK(self.scalar_type() == at::kFloat && other.scalar_type() == at::kFloat,
-              "webgpu eq: only float32 operands are supported, got ", self.scalar_type(), " and ",
-              other.scalar_type());
   TORCH_CHECK(out.scalar_type() == at::kBool, "webgpu eq: the output must be a bool tensor");
+  const at::ScalarType common = self.scalar_type() == other.scalar_type()
+                                    ? self.scalar_type()
+                                    : at::result_type(self, other);
+  const int dt = known_dtype(common, "eq");
+  const at::Tensor a = as_dtype(self, common), b = as_dtype(other, common);
   at::TensorIteratorConfig config;
   config.set_check_mem_overlap(true);
   config.add_output(out);
-  config.add_const_input(self);
-  config.add_const_input(other);
+  config.add_const_input(a);
+  config.add_const_input(b);
   config.check_all_same_dtype(false);
   auto iter = config.build();
   if (iter.numel() == 0) return out;
   twg_iter_t it;
   fill_iter(iter, &it);
-  TWG_CHECK(twg_eq_f32(static_cast<uint8_t *>(iter.data_ptr(0)), fptr(iter, 1), fptr(iter, 2), &it,
-                       nullptr));
+  TWG_CHECK(twg_eq(static_cast<uint8_t *>(iter.data_ptr(0)), iter.data_ptr(1), iter.data_ptr(2), dt,
+                   &it, nullptr));
   return out;
 }
 
@@ -206,21 +222,42 @@ at::Tensor eq_tensor(const at::Tensor &self, const at::Tensor &other) {
 
 at::Tensor &ne_scalar_out(const at::Tensor &self, const at::Scalar &other, at::Tensor &out) {
   require_on_device(self, "ne");
-  TORCH_CHECK(self.scalar_type() == at::kFloat, "webgpu ne: only float32 is supported, got ",
-              self.scalar_type());
   TORCH_CHECK(out.scalar_type() == at::kBool, "webgpu ne: the output must be a bool tensor");
+  // ATen compares in the promoted dtype (an integer tensor against 0.5 compares as
+  // float32, a bool tensor against 2 as int64) and converts the scalar to it the way a
+  // C cast does: rounded for floating types, wrapped around for integers
+  // (uint8 44 equals 300).
+  const at::ScalarType common =
+      c10::isFloatingType(self.scalar_type()) && !other.isComplex() ? self.scalar_type()
+                                                                    : at::result_type(self, other);
+  const int dt = known_dtype(common, "ne");
+  const at::Tensor a = as_dtype(self, common);
+  double s_f = 0;
+  int64_t s_i = 0;
+  if (c10::isFloatingType(common)) {
+    s_f = other.to<double>();
+  } else {
+    const int64_t v = other.isBoolean() ? (other.to<bool>() ? 1 : 0) : other.to<int64_t>();
+    switch (common) {
+      case at::kBool: s_i = v != 0; break;
+      case at::kByte: s_i = (uint8_t)v; break;
+      case at::kChar: s_i = (int8_t)v; break;
+      case at::kShort: s_i = (int16_t)v; break;
+      case at::kInt: s_i = (int32_t)v; break;
+      default: s_i = v; break;
+    }
+  }
   at::TensorIteratorConfig config;
   config.set_check_mem_overlap(true);
   config.add_output(out);
-  config.add_const_input(self);
+  config.add_const_input(a);
   config.check_all_same_dtype(false);
   auto iter = config.build();
   if (iter.numel() == 0) return out;
   twg_iter_t it;
   fill_iter(iter, &it);
-  // ATen compares in the tensor's dtype: the scalar is rounded to float32 first
-  TWG_CHECK(twg_ne_scalar_f32(static_cast<uint8_t *>(iter.data_ptr(0)), fptr(iter, 1),
-                              other.to<float>(), &it, nullptr));
+  TWG_CHECK(twg_ne_scalar(static_cast<uint8_t *>(iter.data_ptr(0)), iter.data_ptr(1), dt, s_f, s_i,
+                          &it, nullptr));
   return out;
 }
 
@@ -232,28 +269,31 @@ at::Tensor ne_scalar(const at::Tensor &self, const at::Scalar &other) {
 at::Tensor &bitwise_and_out(const at::Tensor &self, const at::Tensor &other, at::Tensor &out) {
   require_on_device(self, "bitwise_and");
   require_on_device(other, "bitwise_and");
-  const auto dt = self.scalar_type();
-  TORCH_CHECK(dt == other.scalar_type() && dt == out.scalar_type() &&
-                  (dt == at::kBool || dt == at::kByte || dt == at::kChar),
-              "webgpu bitwise_and: operands and output must share a 1-byte dtype (bool, uint8, int8), got ",
-              self.scalar_type(), ", ", other.scalar_type(), " -> ", out.scalar_type());
+  const at::ScalarType common = self.scalar_type() == other.scalar_type()
+                                    ? self.scalar_type()
+                                    : at::result_type(self, other);
+  TORCH_CHECK(c10::isIntegralType(common, /*includeBool=*/true) && twg_dtype_of(common) >= 0,
+              "webgpu bitwise_and: integer or bool operands expected, got ", self.scalar_type(),
+              " and ", other.scalar_type());
+  TORCH_CHECK(out.scalar_type() == common, "webgpu bitwise_and: the output must have dtype ", common,
+              ", got ", out.scalar_type());
+  const at::Tensor a = as_dtype(self, common), b = as_dtype(other, common);
   at::TensorIteratorConfig config;
   config.set_check_mem_overlap(true);
   config.add_output(out);
-  config.add_const_input(self);
-  config.add_const_input(other);
+  config.add_const_input(a);
+  config.add_const_input(b);
   auto iter = config.build();
   if (iter.numel() == 0) return out;
   twg_iter_t it;
   fill_iter(iter, &it);
-  TWG_CHECK(twg_and_u8(static_cast<uint8_t *>(iter.data_ptr(0)),
-                       static_cast<const uint8_t *>(iter.data_ptr(1)),
-                       static_cast<const uint8_t *>(iter.data_ptr(2)), &it, nullptr));
+  TWG_CHECK(twg_and(iter.data_ptr(0), iter.data_ptr(1), iter.data_ptr(2),
+                    (int32_t)c10::elementSize(common), &it, nullptr));
   return out;
 }
 
 at::Tensor bitwise_and(const at::Tensor &self, const at::Tensor &other) {
-  at::Tensor out = at::empty({0}, self.options());
+  at::Tensor out = at::empty({0}, self.options().dtype(at::result_type(self, other)));
   return bitwise_and_out(self, other, out);
 }
 
@@ -264,10 +304,11 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   // (csrc/bindings.cpp:42).
   TORCH_CHECK(mask.scalar_type() == at::kBool, "masked_select: expected BoolTensor for mask");
   require_on_device(self, "masked_select");
-  // The kernel moves 4-byte elements without looking at them, so int32 rides along.
-  TORCH_CHECK(self.scalar_type() == at::kFloat || self.scalar_type() == at::kInt,
-              "webgpu masked_select: only float32 and int32 sources are supported, got ",
-              self.scalar_type());
+  // The kernel moves elements without looking at them: any dtype of 1, 2, 4 or 8 bytes.
+  const int64_t esize = (int64_t)self.element_size();
+  TORCH_CHECK(esize == 1 || esize == 2 || esize == 4 || esize == 8,
+              "webgpu masked_select: elements of ", esize, " bytes (", self.scalar_type(),
+              ") are not supported");
   at::Tensor m = is_webgpu(mask) ? mask : mask.to(self.device());
   auto expanded = at::expand_outplace(m, self);
   const at::Tensor &me = *std::get<0>(expanded);
@@ -283,17 +324,16 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   // The output shape depends on the data: waiting for the count is the op's one sync
   // point.  The kernel hands it over through pinned memory as soon as it is known.
   int64_t k = 0;
-  TWG_CHECK(twg_masked_select_f32_count(static_cast<float *>(out.data_ptr()), &k,
-                                        static_cast<const float *>(se.const_data_ptr()),
-                                        static_cast<const uint8_t *>(me.const_data_ptr()), &it,
-                                        work.data_ptr(), scratch_bytes, nullptr));
+  TWG_CHECK(twg_masked_select_count(out.data_ptr(), &k, se.const_data_ptr(), (int32_t)esize,
+                                    static_cast<const uint8_t *>(me.const_data_ptr()), &it,
+                                    work.data_ptr(), scratch_bytes, nullptr));
   TORCH_CHECK(k >= 0 && k <= n, "webgpu masked_select: implausible count ", k);
   // Do not pin a source-sized block under a small result, unless the block is small
   // anyway (then the extra copy kernel would cost more than the memory is worth).
-  if (k * 4 <= n && n * (int64_t)sizeof(float) > (int64_t(1) << 20)) {
+  if (k * 4 <= n && n * esize > (int64_t(1) << 20)) {
     at::Tensor exact = at::empty({k}, self.options());
     if (k > 0)
-      TWG_CHECK(twg_memcpy_d2d(exact.data_ptr(), out.const_data_ptr(), (size_t)k * sizeof(float), nullptr));
+      TWG_CHECK(twg_memcpy_d2d(exact.data_ptr(), out.const_data_ptr(), (size_t)(k * esize), nullptr));
     return exact;
   }
   out.unsafeGetTensorImpl()->set_sizes_contiguous({k});

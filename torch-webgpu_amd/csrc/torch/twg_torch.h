@@ -29,6 +29,23 @@ at::Allocator *get_allocator();
 
 inline bool is_webgpu(const at::Tensor &t) { return t.device().is_privateuseone(); }
 
+// enum twg_dtype of a torch dtype, -1 for those the kernels do not know.
+inline int twg_dtype_of(at::ScalarType t) {
+  switch (t) {
+    case at::kBool: return TWG_DT_BOOL;
+    case at::kByte: return TWG_DT_U8;
+    case at::kChar: return TWG_DT_I8;
+    case at::kShort: return TWG_DT_I16;
+    case at::kInt: return TWG_DT_I32;
+    case at::kLong: return TWG_DT_I64;
+    case at::kHalf: return TWG_DT_F16;
+    case at::kBFloat16: return TWG_DT_BF16;
+    case at::kFloat: return TWG_DT_F32;
+    case at::kDouble: return TWG_DT_F64;
+    default: return -1;
+  }
+}
+
 // Fill a twg_iter_t from a built TensorIterator.  TensorIterator already orders
 // dimensions fastest-first and merges adjacent ones; strides arrive in bytes
 // (csrc/ops/binary.h:55-89 does the same division).

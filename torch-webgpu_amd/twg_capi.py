@@ -59,7 +59,8 @@ SYMBOLS = [
     "twg_add_f32", "twg_add_scalar_f32", "twg_mul_f32", "twg_mul_scalar_f32",
     "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided", "twg_cast",
     "twg_eq_f32", "twg_ne_scalar_f32", "twg_and_u8",
-    "twg_masked_select_scratch_bytes", "twg_masked_select_f32", "twg_masked_select_f32_count",
+    "twg_masked_select_scratch_bytes", "twg_masked_select_f32", "twg_masked_select_count",
+    "twg_eq", "twg_ne_scalar", "twg_and",
 ]
 
 _lib = None
@@ -114,7 +115,10 @@ def load():
     L.twg_masked_select_scratch_bytes.argtypes = [i64]
     L.twg_masked_select_scratch_bytes.restype = sz
     L.twg_masked_select_f32.argtypes = [vp, vp, vp, vp, ip, vp, sz, vp]
-    L.twg_masked_select_f32_count.argtypes = [vp, ctypes.POINTER(ctypes.c_int64), vp, vp, ip, vp, sz, vp]
+    L.twg_masked_select_count.argtypes = [vp, ctypes.POINTER(ctypes.c_int64), vp, i32, vp, ip, vp, sz, vp]
+    L.twg_eq.argtypes = [vp, vp, vp, i32, ip, vp]
+    L.twg_ne_scalar.argtypes = [vp, vp, i32, ctypes.c_double, i64, ip, vp]
+    L.twg_and.argtypes = [vp, vp, vp, i32, ip, vp]
     _lib = L
     return L
 
