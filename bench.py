@@ -369,12 +369,17 @@ def config1(capi, W, L, torch, time_launches, Wm, K):
     reps = 20
 
     def wall(fn):
-        capi.sync()
-        t = time.perf_counter()
-        for _ in range(reps):
+        """Median wall time of one copy, device side finished (a mean over the repetitions
+        would carry every scheduling hiccup of the host)."""
+        ts = []
+        for i in range(reps + 3):
+            capi.sync()
+            t = time.perf_counter()
             fn()
-        capi.sync()
-        return (time.perf_counter() - t) / reps
+            capi.sync()
+            if i >= 3:
+                ts.append(time.perf_counter() - t)
+        return statistics.median(ts)
 
     t_up = wall(lambda: d_a.upload(a_h))
     t_down = wall(lambda: capi.check(L.twg_memcpy_d2h(back.data_ptr(), d_o.ptr, 4 * n1, None)))
