@@ -123,9 +123,9 @@ int twg_mem_stats(twg_mem_stats_t *out);
 /* ----------------------------------------------------------------- copies */
 
 /* Host -> device.  Replaces queue.WriteBuffer in copy_ (csrc/ops/copy.cpp:74-92).
- * Pageable host memory is staged through a ring of pinned buffers so the CPU
- * memcpy of chunk k+1 overlaps the DMA of chunk k; the host range may be reused
- * as soon as the call returns. */
+ * Pageable host memory is staged through a ring of pinned memory, in pieces sized
+ * to the copy, so the CPU memcpy of piece k+1 overlaps the DMA of piece k; the host
+ * range may be reused as soon as the call returns. */
 int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_stream_t stream);
 /* Device -> host, blocking: on return the bytes are in dst_host.  Replaces the
  * staging-buffer + MapAsync + WaitAny + memcpy sequence of cpu_copy_with_webgpu
