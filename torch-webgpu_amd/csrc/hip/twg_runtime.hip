@@ -7,6 +7,7 @@
 //   csrc/ops/copy.cpp:12-62,74-122        WriteBuffer / CopyBufferToBuffer / MapAsync
 #include <hip/hip_runtime.h>
 #include <emmintrin.h>
+#include <sys/mman.h>
 #include <unistd.h>
 
 #include <atomic>
@@ -96,6 +97,7 @@ int release_cached_locked(Pool &p) {
 constexpr int kStageSlots = 16;                    // events; a copy uses ring / piece of them
 constexpr size_t kStageRingBytes = size_t(64) << 20;
 constexpr size_t kStreamingDrainBytes = size_t(32) << 20;  // beyond what a last-level cache keeps
+constexpr size_t kHugePageHintBytes = size_t(8) << 20;      // D2H destinations from this size on
 constexpr size_t kMailboxBytes = 256;                      // largest read served by the mailbox
 constexpr int kMailboxSpins = 200000;                      // then fall back to a stream sync
 
@@ -166,9 +168,9 @@ void drain_slot(char *dst, const char *src, size_t n, bool streaming) {
 // bounds them (one core moves ~30 GB/s), so from 8 MiB on it is split into parts that the
 // caller's thread and three helpers claim one by one.  The caller starts a job, issues the
 // DMA of the neighbouring chunk meanwhile (a hipMemcpyAsync plus an event record cost it
-// ~17 us, a third of a chunk's copy time) and then joins in.  A freshly allocated
-// destination still costs its page faults (~10 GB/s): faulting it in from several threads
-// was measured 3-5x slower than from one on this host, so that is left to the drain itself.
+// ~17 us, a third of a chunk's copy time) and then joins in.  Faulting a freshly
+// allocated destination in from several threads was measured 3-5x slower than from one on
+// this host, so that is left to the drain itself (see the huge page hint in twg_memcpy_d2h).
 // The helpers are created on first use, sleep on a condition variable between copies and are
 // never joined: the team is leaked like the pools above, so nothing they touch is destroyed
 // at exit.
@@ -654,6 +656,17 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
     return 0;
   };
   const bool streaming = nbytes >= kStreamingDrainBytes;
+  if (nbytes >= kHugePageHintBytes) {
+    // A destination that was just allocated (what `t.cpu()` hands over) takes a page fault
+    // and a page of zeroing per 4 KiB, which bounds the copy at ~13 GB/s.  Asking for
+    // transparent huge pages on its 2 MiB-aligned interior makes that one fault per 2 MiB
+    // (30-39 GB/s where the system grants them on madvise); on pages that already exist the
+    // call changes nothing.  It is a hint: the result is ignored.
+    const uintptr_t two_mib = uintptr_t(2) << 20;
+    const uintptr_t lo = (reinterpret_cast<uintptr_t>(dst) + two_mib - 1) & ~(two_mib - 1);
+    const uintptr_t hi = (reinterpret_cast<uintptr_t>(dst) + nbytes) & ~(two_mib - 1);
+    if (hi > lo) (void)madvise(reinterpret_cast<void *>(lo), hi - lo, MADV_HUGEPAGE);
+  }
   // The DMA engine runs up to a ring (less one slot) ahead of the CPU draining the slots:
   // while chunk c is drained, the DMA that refills the slot drained before it is issued.
   size_t issued = 0;
