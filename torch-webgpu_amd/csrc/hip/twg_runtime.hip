@@ -596,11 +596,9 @@ int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_strea
       st.busy[slot] = false;
     }
     const bool started = host_copy_start(st.buf(slot), src + done, chunk, false, nbytes >= kTeamMinBytes);
-    if (started) {  // the team is copying: issue the previous chunk's DMA meanwhile
-      rc = issue_pending();
-      host_copy_finish(true);
-      if (rc) return rc;
-    }
+    rc = issue_pending();  // the previous chunk's DMA, while the team (if any) is copying
+    host_copy_finish(started);
+    if (rc) return rc;
     pending_slot = slot;
     pending_off = done;
     pending_len = chunk;
