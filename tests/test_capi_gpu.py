@@ -92,6 +92,33 @@ def test_copy_round_trip_fp32_and_bool(twg):
     assert bit_equal(raw[8:-8].view(torch.float32), t)
 
 
+def test_copy_sizes_around_every_staging_boundary(twg):
+    # The pinned ring is divided differently for each copy size and large copies are split
+    # over helper threads; sizes just below, at and above each switch, with ragged tails, in
+    # an order that changes the division between consecutive copies and leaves uploads in
+    # flight when the next copy starts.
+    L = twg.load()
+    g = torch.Generator().manual_seed(77)
+    mib = 1 << 20
+    sizes = [mib - 1, mib, mib + 1, 2 * mib + 3, 4 * mib, 8 * mib - 1, 8 * mib, 8 * mib + 5,
+             16 * mib - 7, 16 * mib + mib + 3, 32 * mib - 1, 32 * mib + 12, 9 * mib + 999,
+             128 * mib - 3, 128 * mib + 16 * mib + 11, 300, 64 * mib + 1]
+    raw = torch.randint(0, 256, (max(sizes) + 64,), dtype=torch.uint8, generator=g)
+    back = torch.empty(max(sizes) + 64, dtype=torch.uint8)
+    dev = twg.DeviceBuffer(max(sizes))
+    small = twg.DeviceBuffer(4096)
+    for i, nb in enumerate(sizes):
+        _say(f"copy {nb} bytes")
+        off = (i * 7) % 31
+        twg.check(L.twg_memcpy_h2d(dev.ptr, raw.data_ptr() + off, nb, None))
+        if i % 2:  # a small upload of another division right behind the large one
+            twg.check(L.twg_memcpy_h2d(small.ptr, raw.data_ptr(), 4096, None))
+        back.fill_(0xEE)
+        twg.check(L.twg_memcpy_d2h(back.data_ptr() + 3, dev.ptr, nb, None))
+        assert torch.equal(back[3:3 + nb], raw[off:off + nb]), nb
+        assert bool((back[:3] == 0xEE).all()) and bool((back[3 + nb:3 + nb + 61] == 0xEE).all()), nb
+
+
 # --------------------------------------------------------------------- add
 
 def test_add_config1_contiguous(twg):
