@@ -688,3 +688,80 @@ def test_invalid_iter_is_rejected(twg):
     it.ndim = 9
     assert L.twg_add_f32(buf.ptr, buf.ptr, buf.ptr, 1.0, ctypes.byref(it), None) == twg.E_INVALID_ARG
     assert L.twg_unary_f32(99, buf.ptr, buf.ptr, ctypes.byref(twg.dense_iter(16)), None) == twg.E_INVALID_ARG
+
+
+def test_entry_points_capture_into_a_hip_graph(twg):
+    # A caller may record the launches on a stream of its own into a HIP graph and replay
+    # them: every entry point only enqueues kernels (the scratch clear of masked_select is a
+    # fill kernel, not a memset node).  Replays, with new input contents each time and eager
+    # work in between, must reproduce the eager results bit for bit.
+    hip = ctypes.CDLL("libamdhip64.so")
+    vp = ctypes.c_void_p
+
+    def ok(rc):
+        assert rc == 0, f"HIP error {rc}"
+
+    L = twg.load()
+    stream = vp()
+    ok(hip.hipStreamCreateWithFlags(ctypes.byref(stream), 1))  # hipStreamNonBlocking
+    n = (1 << 21) + 4096 + 13
+    g = torch.Generator().manual_seed(91)
+    a_h, b_h = torch.randn(n, generator=g), torch.randn(n, generator=g)
+    m_h = torch.rand(n, generator=g) < 0.37
+    d_a, d_b, d_m = twg.to_device(a_h), twg.to_device(b_h), twg.to_device(m_h)
+    d_sum, d_act, d_eq, d_sel = (twg.DeviceBuffer(4 * n), twg.DeviceBuffer(4 * n), twg.DeviceBuffer(n),
+                                 twg.DeviceBuffer(4 * n))
+    d_cnt = twg.DeviceBuffer(8)
+    sb = L.twg_masked_select_scratch_bytes(n)
+    d_scr = twg.DeviceBuffer(sb)
+    it = twg.dense_iter(n)
+
+    def enqueue(s):
+        twg.check(L.twg_add_f32(d_sum.ptr, d_a.ptr, d_b.ptr, ctypes.c_float(1.0), ctypes.byref(it), s))
+        twg.check(L.twg_unary_f32(twg.UNARY_GELU_ERF, d_act.ptr, d_sum.ptr, ctypes.byref(it), s))
+        twg.check(L.twg_eq_f32(d_eq.ptr, d_a.ptr, d_b.ptr, ctypes.byref(it), s))
+        twg.check(L.twg_masked_select_f32(d_sel.ptr, d_cnt.ptr, d_act.ptr, d_m.ptr, ctypes.byref(it),
+                                          d_scr.ptr, sb, s))
+
+    def results():
+        k = int(d_cnt.download((1,), torch.int64)[0])
+        return (d_act.download((n,), torch.float32), d_eq.download((n,), torch.uint8),
+                k, d_sel.download((k,), torch.float32))
+
+    twg.sync()
+    ok(hip.hipStreamBeginCapture(stream, 1))  # hipStreamCaptureModeThreadLocal
+    try:
+        enqueue(stream)
+    finally:
+        graph = vp()
+        rc_end = hip.hipStreamEndCapture(stream, ctypes.byref(graph))
+    ok(rc_end)
+    graph_exec = vp()
+    ok(hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)))
+    try:
+        for rep in range(3):
+            _say(f"graph replay {rep}")
+            if rep:  # new contents in the same buffers, and unrelated eager work in between
+                a_h = torch.randn(n, generator=g)
+                a_h[::5] = b_h[::5]
+                m_h = torch.rand(n, generator=g) < (0.1 + 0.4 * rep)
+                d_a.upload(a_h)
+                d_m.upload(m_h)
+                H.add(a_h[:1000], b_h[:1000])
+            twg.sync()
+            ok(hip.hipGraphLaunch(graph_exec, stream))
+            ok(hip.hipStreamSynchronize(stream))
+            got = results()
+            for buf in (d_act, d_eq, d_sel, d_cnt):  # wipe, then the same work eagerly
+                twg.check(L.twg_fill_bytes(buf.ptr, 0xCD, buf.nbytes, None))
+            enqueue(None)
+            twg.sync()
+            want = results()
+            assert got[2] == want[2] == int(m_h.sum())
+            assert bit_equal(got[0], want[0]) and torch.equal(got[1], want[1]) and bit_equal(got[3], want[3])
+            assert torch.equal(got[1].bool(), torch.eq(a_h, b_h))
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
+        hip.hipStreamDestroy(stream)
+
