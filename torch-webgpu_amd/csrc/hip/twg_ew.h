@@ -120,45 +120,63 @@ __device__ __forceinline__ TO apply(const Op &op, TA a, TB b) {
 }
 
 // ------------------------------------------------------------- ew_contig
-// One pack per lane, no loop: on MI355X a grid of very many short-lived blocks
-// streams faster (add: 6.4-6.7 TB/s) than a persistent grid-stride loop sized to
-// the 256 CUs (5.4 TB/s).  Block size matters too, and the best one was measured per
-// shape of traffic at 2^28 elements:
-//   same width in and out (add, activations, and): 64 lanes (add 83% of peak, 80% at 256);
-//   two float4 in, one dword of bools out (eq): 64 lanes (83%; 81% at 256, 80% at 1024);
-//   8 bytes out per lane (float32 -> half): 64 lanes (87%; 82% at 256);
-//   one pack in, at most a dword out (ne.Scalar, float32 -> bool): 1024 lanes (80%;
-//     78-79.5% at 128..512; a 64-lane block moves too little, 73%: the grid then
+// No loop: on MI355X a grid of very many short-lived single-wavefront blocks streams
+// faster (add: 6.4-6.7 TB/s) than a persistent grid-stride loop sized to the 256 CUs
+// (5.4 TB/s).  How much one block moves matters too; measured per shape of traffic at 2^28
+// elements (packs per lane x lanes):
+//   same width in and out (add, activations, and): 1 x 64 (add 83% of peak; 80% with
+//     2 x 64 or 1 x 256, 77% with 4 x 64);
+//   two float4 in, one dword of bools out (eq): 1 x 64 (89%; 84% with 2 x 64);
+//   8 bytes out per lane (float32 -> half): 1 x 64 (87%; 84% with 2 x 64);
+//   one pack in, at most a dword out (ne.Scalar, float32 -> bool): 2 x 64 (90%; 88% with
+//     4 x 64, 80% with 1 x 1024; 1 x 64 moves too little per block, 73%: the grid then
 //     launches no faster than ~4.5 blocks per ns);
-//   output wider than input (bool -> float32): 1024 lanes (74.5%; 71% at 256, 66% at 64).
+//   output wider than input (bool -> float32): 4 x 64 (78%; 75% with 1 x 1024 or 2 x 64,
+//     67% with 1 x 64).
+struct ContigShape {
+  int threads, packs;
+};
 template <int NIN, int VEC, typename TO, typename TA>
-constexpr int contig_block_size() {
-  if (sizeof(TO) > sizeof(TA)) return 1024;
-  if (NIN == 1 && sizeof(TO) * VEC <= 4) return 1024;
-  return 64;
+constexpr ContigShape contig_shape() {
+  if (sizeof(TO) > sizeof(TA)) return {64, 4};
+  if (NIN == 1 && sizeof(TO) * VEC <= 4) return {64, 2};
+  return {64, 1};
 }
 
 template <int THREADS, int NIN, int VEC, bool STREAM, typename Op, typename TO, typename TA,
-          typename TB>
+          typename TB, int U = 1>
 __global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const TB *b,
                                                      int64_t numel, Op op) {
   using PO = Pack<TO, VEC>;
   using PA = Pack<TA, VEC>;
   using PB = Pack<TB, VEC>;
   const int64_t nvec = numel / VEC;
-  const int64_t i = (int64_t)blockIdx.x * THREADS + threadIdx.x;
-  if (i < nvec) {
-    const PA va = load_pack<STREAM, PA, true>(reinterpret_cast<const PA *>(a) + i);
-    PB vb;
-    if constexpr (NIN == 2) vb = load_pack<STREAM, PB, true>(reinterpret_cast<const PB *>(b) + i);
-    PO r;
+  // pack k of lane l sits at base + k * THREADS + l: every load and store instruction of
+  // the block covers THREADS consecutive packs
+  const int64_t base = (int64_t)blockIdx.x * (THREADS * U) + threadIdx.x;
+  PA va[U];
+  PB vb[U];
 #pragma unroll
-    for (int k = 0; k < VEC; ++k)
-      r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
-    // the nontemporal hint pays for stores of 8 and 16 bytes per lane (float32 -> half:
-    // 87% vs 84% of peak); one dword of bools per lane streams faster with a plain store
-    // (ne: 83% vs 79%)
-    store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = base + k * THREADS;
+    if (i < nvec) {
+      va[k] = load_pack<STREAM, PA, true>(reinterpret_cast<const PA *>(a) + i);
+      if constexpr (NIN == 2) vb[k] = load_pack<STREAM, PB, true>(reinterpret_cast<const PB *>(b) + i);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = base + k * THREADS;
+    if (i < nvec) {
+      PO r;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        r.v[e] = apply<NIN, Op, TO, TA, TB>(op, va[k].v[e], NIN == 2 ? vb[k].v[e] : TB());
+      // the nontemporal hint pays for stores of 8 and 16 bytes per lane (float32 -> half:
+      // 87% vs 84% of peak); one dword of bools per lane streams faster with a plain store
+      // (ne: 83% vs 79%)
+      store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+    }
   }
   if constexpr (VEC > 1) {  // the last numel % VEC elements
     if (blockIdx.x == gridDim.x - 1) {
@@ -663,19 +681,20 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
                         (NIN == 1 || aligned_to(b, sizeof(TB) * VEC));
     const bool stream =
         g.numel * (int64_t)(sizeof(TO) + sizeof(TA) + (NIN == 2 ? sizeof(TB) : 0)) > kStreamBytes;
-    constexpr int kBlock = contig_block_size<NIN, VEC, TO, TA>();
+    constexpr ContigShape kShape = contig_shape<NIN, VEC, TO, TA>();
+    constexpr int kBlock = kShape.threads, kPacks = kShape.packs;
     const int64_t packs = vec_ok ? (g.numel + VEC - 1) / VEC : g.numel;
-    const int64_t blocks = (packs + kBlock - 1) / kBlock;
+    const int64_t blocks = (packs + kBlock * kPacks - 1) / (kBlock * kPacks);
     if (blocks > INT32_MAX) return TWG_E_UNSUPPORTED;
     const unsigned grid = (unsigned)blocks;
     if (vec_ok && stream)
-      ew_contig<kBlock, NIN, VEC, true, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, VEC, true, Op, TO, TA, TB, kPacks><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     else if (vec_ok)
-      ew_contig<kBlock, NIN, VEC, false, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, VEC, false, Op, TO, TA, TB, kPacks><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     else if (stream)
-      ew_contig<kBlock, NIN, 1, true, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, 1, true, Op, TO, TA, TB, kPacks><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     else
-      ew_contig<kBlock, NIN, 1, false, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
+      ew_contig<kBlock, NIN, 1, false, Op, TO, TA, TB, kPacks><<<grid, kBlock, 0, s>>>(out, a, b, g.numel, op);
     return (int)hipGetLastError();
   }
 
