@@ -80,6 +80,15 @@ def test_copy_round_trip_fp32_and_bool(twg):
             twg.check(L.twg_memcpy_d2h(back.data_ptr() + 5, small.ptr + off, nb, None))
             assert torch.equal(back[5:5 + nb], raw[off:off + nb])
             assert bool((back[:5] == 0xEE).all()) and bool((back[5 + nb:] == 0xEE).all())
+    # uploads of a few bytes travel as a kernel argument: every size around the switch, at odd
+    # device and host offsets, must leave the neighbouring bytes alone
+    for nb in (1, 2, 3, 4, 8, 63, 64, 65, 255, 256, 257, 300, 1023, 1024, 1025, 1500):
+        for off in (0, 1, 5):
+            twg.check(L.twg_fill_bytes(small.ptr, 0xEE, 4096, None))
+            twg.check(L.twg_memcpy_h2d(small.ptr + 16 + off, raw.data_ptr() + 3 + off, nb, None))
+            back = small.download((2048,), torch.uint8)
+            assert torch.equal(back[16 + off:16 + off + nb], raw[3 + off:3 + off + nb]), (nb, off)
+            assert bool((back[:16 + off] == 0xEE).all()) and bool((back[16 + off + nb:] == 0xEE).all())
     # device -> device and fill
     t = torch.randn(4097, generator=g)
     src = twg.to_device(t)

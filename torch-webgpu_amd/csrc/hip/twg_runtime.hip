@@ -329,6 +329,27 @@ __global__ __launch_bounds__(64) void mailbox_kernel(uint8_t *box, const uint8_t
   }
 }
 
+// Uploads of a few bytes (a scalar, a shape) travel as a kernel argument: the launch copies
+// them, so the host range is free at once and no staging slot, DMA or event is involved
+// (~4 us of host time against ~20 us through the ring).
+constexpr size_t kSmallUploadBytes = 1024;
+template <int BYTES>
+struct SmallPayload {
+  uint8_t bytes[BYTES];
+};
+template <int BYTES>
+__global__ __launch_bounds__(64) void upload_small_kernel(uint8_t *dst, SmallPayload<BYTES> p,
+                                                          uint32_t n) {
+  for (uint32_t i = threadIdx.x; i < n; i += 64) dst[i] = p.bytes[i];
+}
+template <int BYTES>
+int upload_small(void *dst, const void *src, size_t n, hipStream_t s) {
+  SmallPayload<BYTES> p;
+  std::memcpy(p.bytes, src, n);
+  upload_small_kernel<BYTES><<<1, 64, 0, s>>>(static_cast<uint8_t *>(dst), p, (uint32_t)n);
+  return (int)hipGetLastError();
+}
+
 __global__ void fill_bytes_kernel(uint8_t *dst, uint8_t v, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t step = (size_t)gridDim.x * blockDim.x;
@@ -571,6 +592,9 @@ int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_strea
   int rc = ensure_init();
   if (rc) return rc;
   hipStream_t s = resolve_stream(stream);
+  if (nbytes <= 64) return upload_small<64>(dst_dev, src_host, nbytes, s);  // scalars
+  if (nbytes <= 256) return upload_small<256>(dst_dev, src_host, nbytes, s);
+  if (nbytes <= kSmallUploadBytes) return upload_small<kSmallUploadBytes>(dst_dev, src_host, nbytes, s);
   Staging &st = staging();
   std::lock_guard<std::mutex> lk(st.mu);
   if ((rc = staging_prepare_locked(st))) return rc;
