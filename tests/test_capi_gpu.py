@@ -72,10 +72,10 @@ def test_copy_round_trip_fp32_and_bool(twg):
         assert torch.equal(back[off:off + nb], raw[off:off + nb])
         assert bool((back[:off] == 0xEE).all()) and bool((back[off + nb:] == 0xEE).all())
         dev.free()
-    # reads of a few bytes (<= 256) take a different route back than larger ones
-    small = twg.to_device(raw[:4096])
-    for nb in (1, 3, 8, 255, 256, 257, 1025):
-        for off in (0, 1, 7):
+    # reads of up to 16 KiB take a different route back than larger ones
+    small = twg.to_device(raw[:65536])
+    for nb in (1, 3, 8, 255, 256, 257, 1025, 4096, 16383, 16384, 16385, 20000):
+        for off in (0, 1, 4, 7):
             back = torch.full((nb + 16,), 0xEE, dtype=torch.uint8)
             twg.check(L.twg_memcpy_d2h(back.data_ptr() + 5, small.ptr + off, nb, None))
             assert torch.equal(back[5:5 + nb], raw[off:off + nb])

@@ -98,7 +98,7 @@ constexpr int kStageSlots = 16;                    // events; a copy uses ring /
 constexpr size_t kStageRingBytes = size_t(64) << 20;
 constexpr size_t kStreamingDrainBytes = size_t(32) << 20;  // beyond what a last-level cache keeps
 constexpr size_t kHugePageHintBytes = size_t(8) << 20;      // D2H destinations from this size on
-constexpr size_t kMailboxBytes = 256;                      // largest read served by the mailbox
+constexpr size_t kMailboxBytes = 16384;                     // largest read served by the mailbox
 constexpr int kMailboxSpins = 200000;                      // then fall back to a stream sync
 
 // Bytes a copy of nbytes moves per DMA.  Each hipMemcpyAsync + event record costs ~17 us
@@ -318,12 +318,24 @@ int staging_divide_locked(Staging &s, size_t nbytes, bool to_device) {
   return 0;
 }
 
-// Copy n <= kMailboxBytes bytes into the mailbox, then publish the sequence number.
-// One wavefront, so the release below orders every lane's payload stores.
-__global__ __launch_bounds__(64) void mailbox_kernel(uint8_t *box, const uint8_t *src, uint32_t n,
-                                                     uint32_t seq) {
-  for (uint32_t i = threadIdx.x; i < n; i += 64) box[i] = src[i];
-  if (threadIdx.x == 0) {
+// Copy n <= kMailboxBytes bytes into the mailbox, then publish the sequence number.  Every
+// lane's payload stores are made visible system-wide before the barrier, the release store of
+// the sequence word comes after it.
+constexpr int kMailboxLanes = 256;
+__global__ __launch_bounds__(kMailboxLanes) void mailbox_kernel(uint8_t *box, const uint8_t *src,
+                                                                uint32_t n, uint32_t seq) {
+  const uint32_t t = threadIdx.x;
+  uint32_t done = 0;
+  if ((reinterpret_cast<uintptr_t>(src) & 3u) == 0) {  // the box itself is 64-byte aligned
+    const uint32_t words = n >> 2;
+    for (uint32_t i = t; i < words; i += kMailboxLanes)
+      reinterpret_cast<uint32_t *>(box)[i] = reinterpret_cast<const uint32_t *>(src)[i];
+    done = words << 2;
+  }
+  for (uint32_t i = done + t; i < n; i += kMailboxLanes) box[i] = src[i];
+  __threadfence_system();
+  __syncthreads();
+  if (t == 0) {
     __hip_atomic_store(reinterpret_cast<uint32_t *>(box + kMailboxBytes), seq, __ATOMIC_RELEASE,
                        __HIP_MEMORY_SCOPE_SYSTEM);
   }
@@ -648,7 +660,7 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   const char *src = static_cast<const char *>(src_dev);
   if (nbytes <= kMailboxBytes) {
     const uint32_t seq = ++st.mailbox_seq;
-    mailbox_kernel<<<1, 64, 0, s>>>(reinterpret_cast<uint8_t *>(st.mailbox_dev),
+    mailbox_kernel<<<1, kMailboxLanes, 0, s>>>(reinterpret_cast<uint8_t *>(st.mailbox_dev),
                                     reinterpret_cast<const uint8_t *>(src), (uint32_t)nbytes, seq);
     TWG_HIP_TRY(hipGetLastError());
     const uint32_t *flag = reinterpret_cast<const uint32_t *>(st.mailbox + kMailboxBytes);
