@@ -388,7 +388,7 @@ def config1(capi, W, L, torch, time_launches, Wm, K):
     d = {"elements": n1, "add_kernel_us": round(statistics.median(ms) * 1e3, 2),
          "h2d_4MiB_us": round(t_up * 1e6, 1), "h2d_GBps": round(4 * n1 / t_up / 1e9, 2),
          "d2h_4MiB_us": round(t_down * 1e6, 1), "d2h_GBps": round(4 * n1 / t_down / 1e9, 2),
-         "note": "pageable host memory through the pinned staging ring; result equals the CPU sum"}
+         "note": "pageable host memory through the pinned ring (up: DMA per piece, down: streamed by workgroups); median of single copies; result equals the CPU sum"}
     log(f"  config 1 (2^20): add {d['add_kernel_us']} us, H2D {d['h2d_GBps']} GB/s, D2H {d['d2h_GBps']} GB/s")
     return d
 
