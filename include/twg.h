@@ -261,6 +261,9 @@ int twg_eq(uint8_t *out, const void *a, const void *b, int32_t dtype, const twg_
  * does), s_i for integral ones and bool. */
 int twg_ne_scalar(uint8_t *out, const void *a, int32_t dtype, double s_f, int64_t s_i,
                   const twg_iter_t *it, twg_stream_t stream);
+/* out[i] = |a[i]| for every dtype but bool (csrc/bindings.cpp:35), out of a's dtype.
+ * TWG_DT_F32 runs twg_unary_f32(TWG_UNARY_ABS). */
+int twg_abs(void *out, const void *a, int32_t dtype, const twg_iter_t *it, twg_stream_t stream);
 /* out[i] = a[i] & b[i] on integers of elem_size = 1, 2, 4 or 8 bytes
  * (csrc/bindings.cpp:40-41). */
 int twg_and(void *out, const void *a, const void *b, int32_t elem_size, const twg_iter_t *it,

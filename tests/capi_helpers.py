@@ -190,3 +190,14 @@ def bitwise_and(a, b):
     it = _iter_for(shape, out, (ae, be), True)
     capi.check(L.twg_and(uo.ptr, ua.ptr, ub.ptr, a.element_size(), ctypes.byref(it), None))
     return uo.fetch()
+
+
+def abs_any(a, out=None):
+    L = capi.load()
+    if out is None:
+        out = torch.zeros(tuple(a.shape), dtype=a.dtype)
+    ua, uo = Uploaded(a), Uploaded(out)
+    it = _iter_for(tuple(a.shape), out, (a,), True)
+    rc = L.twg_abs(uo.ptr, ua.ptr, capi.DTYPES[a.dtype], ctypes.byref(it), None)
+    return rc, (uo.fetch() if rc == 0 else None)
+

@@ -426,6 +426,21 @@ def test_eq_ne_and_every_dtype_match_aten(twg):
             assert bit_equal(H.bitwise_and(x, y), torch.bitwise_and(x, y)), dt
             assert bit_equal(H.bitwise_and(x[:50000].view(250, 200).t(), y[:250]),
                              torch.bitwise_and(x[:50000].view(250, 200).t(), y[:250])), dt
+    # abs: every dtype but bool; integers wrap at their minimum, NaN and -0.0 lose their sign
+    for dt in _INT_TYPES + _FLOAT_TYPES:
+        a = _compare_source(dt, n, g)
+        if dt in _FLOAT_TYPES:
+            a = -a
+        elif dt not in (torch.bool, torch.uint8):
+            a = a - 2
+            a[0] = torch.iinfo(dt).min
+        rc, got = H.abs_any(a)
+        if dt == torch.bool:
+            assert rc == twg.E_UNSUPPORTED
+            continue
+        assert rc == 0 and bit_equal(got, a.abs()), dt
+        rc, got = H.abs_any(a[:50000].view(250, 200).t(), out=torch.zeros(200, 500, dtype=dt)[:, ::2])
+        assert rc == 0 and bit_equal(got, a[:50000].view(250, 200).t().abs()), dt
     L = twg.load()
     assert L.twg_eq(None, None, None, 99, None, None) == twg.E_INVALID_ARG
     assert L.twg_and(None, None, None, 3, None, None) == twg.E_UNSUPPORTED

@@ -474,6 +474,10 @@ def test_mask_ops_take_every_dtype():
         m = torch.rand(n, generator=g) < 0.5
         got = torch.masked_select(wa, m.to("webgpu"))
         assert got.dtype == dt and torch.equal(got.to("cpu"), torch.masked_select(a, m)), dt
+        if dt != torch.bool:
+            neg = (a.to(torch.float64) - 2).to(dt) if dt != torch.uint8 else a
+            got = neg.to("webgpu").abs()
+            assert got.dtype == dt and torch.equal(got.to("cpu"), neg.abs()), dt
         if dt in ints:
             got = torch.bitwise_and(wa, wb)
             assert got.dtype == dt and torch.equal(got.to("cpu"), torch.bitwise_and(a, b)), dt

@@ -1,7 +1,8 @@
-// eq / ne.Scalar / bitwise_and for every dtype (twg_eq, twg_ne_scalar, twg_and).
+// eq / ne.Scalar / bitwise_and / abs for every dtype (twg_eq, twg_ne_scalar, twg_and,
+// twg_abs).
 //
 // The reference sends these ops to ATen's CPU kernels through a boxed fallback
-// (csrc/bindings.cpp:36-41), so it accepts any dtype; the float32 / bool kernels of
+// (csrc/bindings.cpp:35-41), so it accepts any dtype; the float32 / bool kernels of
 // twg_elementwise.hip cover the shapes that are measured, these cover the rest with the
 // same launch logic (dense and general strided kernels).  Semantics are ATen's: IEEE
 // comparison for floating types (NaN != NaN, -0 == +0), exact for integers; half and
@@ -27,6 +28,34 @@ template <typename T>
 struct AndAnyOp {
   __device__ __forceinline__ T operator()(T a, T b) const { return a & b; }
 };
+
+// |x| in the element's own type: integers wrap at the minimum as ATen's do (abs(INT_MIN) =
+// INT_MIN); half and bfloat16 clear their sign bit, so NaN payloads survive.
+template <typename T>
+struct AbsAnyOp {
+  __device__ __forceinline__ T operator()(T a) const {
+    if constexpr (std::is_same<T, BFloat16>::value) {
+      return BFloat16{(uint16_t)(a.bits & 0x7FFFu)};
+    } else if constexpr (std::is_same<T, Half>::value) {
+      uint16_t b;
+      __builtin_memcpy(&b, &a, 2);
+      b &= 0x7FFFu;
+      Half r;
+      __builtin_memcpy(&r, &b, 2);
+      return r;
+    } else if constexpr (std::is_same<T, double>::value) {
+      return fabs(a);
+    } else {
+      using U = typename std::make_unsigned<T>::type;
+      return a < 0 ? (T)(U(0) - (U)a) : a;
+    }
+  }
+};
+template <typename T>
+int abs_any(void *out, const void *a, const twg_iter_t *it, twg_stream_t stream) {
+  return launch_ew<1, AbsAnyOp<T>, T, T, T, /*ALL_SHAPES=*/false>(
+      static_cast<T *>(out), static_cast<const T *>(a), nullptr, it, AbsAnyOp<T>{}, stream);
+}
 
 template <typename T>
 int eq_any(uint8_t *out, const void *a, const void *b, const twg_iter_t *it, twg_stream_t stream) {
@@ -109,6 +138,24 @@ int twg_and(void *out, const void *a, const void *b, int32_t elem_size, const tw
     case 4: return and_any<uint32_t>(out, a, b, it, stream);
     case 8: return and_any<uint64_t>(out, a, b, it, stream);
     default: return TWG_E_UNSUPPORTED;
+  }
+}
+
+int twg_abs(void *out, const void *a, int32_t dtype, const twg_iter_t *it, twg_stream_t stream) {
+  switch (dtype) {
+    case TWG_DT_F32:
+      return twg_unary_f32(TWG_UNARY_ABS, static_cast<float *>(out), static_cast<const float *>(a),
+                           it, stream);
+    case TWG_DT_U8: return twg_copy_strided(out, a, 1, it, stream);  // nothing to do
+    case TWG_DT_I8: return abs_any<int8_t>(out, a, it, stream);
+    case TWG_DT_I16: return abs_any<int16_t>(out, a, it, stream);
+    case TWG_DT_I32: return abs_any<int32_t>(out, a, it, stream);
+    case TWG_DT_I64: return abs_any<int64_t>(out, a, it, stream);
+    case TWG_DT_F16: return abs_any<Half>(out, a, it, stream);
+    case TWG_DT_BF16: return abs_any<BFloat16>(out, a, it, stream);
+    case TWG_DT_F64: return abs_any<double>(out, a, it, stream);
+    case TWG_DT_BOOL: return TWG_E_UNSUPPORTED;  // ATen has no abs of bool either
+    default: return TWG_E_INVALID_ARG;
   }
 }
 

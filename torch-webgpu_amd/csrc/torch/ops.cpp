@@ -170,7 +170,21 @@ at::Tensor &silu_out(const at::Tensor &self, at::Tensor &out) {
   return out;
 }
 at::Tensor &abs_out(const at::Tensor &self, at::Tensor &out) {
-  unary_f32(TWG_UNARY_ABS, self, out, "abs");
+  // any real dtype, as behind the reference's CPU fallback (csrc/bindings.cpp:35)
+  require_on_device(self, "abs");
+  const int dt = twg_dtype_of(self.scalar_type());
+  TORCH_CHECK(dt >= 0 && self.scalar_type() != at::kBool, "webgpu abs: dtype ", self.scalar_type(),
+              " is not supported");
+  at::TensorIteratorConfig config;
+  config.set_check_mem_overlap(true);
+  config.add_output(out);
+  config.add_const_input(self);
+  config.check_all_same_dtype(true);
+  auto iter = config.build();
+  if (iter.numel() == 0) return out;
+  twg_iter_t it;
+  fill_iter(iter, &it);
+  TWG_CHECK(twg_abs(iter.data_ptr(0), iter.data_ptr(1), dt, &it, nullptr));
   return out;
 }
 

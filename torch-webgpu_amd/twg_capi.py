@@ -60,7 +60,7 @@ SYMBOLS = [
     "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided", "twg_cast",
     "twg_eq_f32", "twg_ne_scalar_f32", "twg_and_u8",
     "twg_masked_select_scratch_bytes", "twg_masked_select_f32", "twg_masked_select_count",
-    "twg_eq", "twg_ne_scalar", "twg_and",
+    "twg_eq", "twg_ne_scalar", "twg_and", "twg_abs",
 ]
 
 _lib = None
@@ -119,6 +119,7 @@ def load():
     L.twg_eq.argtypes = [vp, vp, vp, i32, ip, vp]
     L.twg_ne_scalar.argtypes = [vp, vp, i32, ctypes.c_double, i64, ip, vp]
     L.twg_and.argtypes = [vp, vp, vp, i32, ip, vp]
+    L.twg_abs.argtypes = [vp, vp, i32, ip, vp]
     _lib = L
     return L
 
