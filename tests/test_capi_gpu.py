@@ -7,6 +7,7 @@ oracle), relu, copy, eq, ne, bitwise_and and masked_select (length and order);
 closed form.
 """
 import ctypes
+import os
 import itertools
 
 import pytest
@@ -126,6 +127,37 @@ def test_copy_sizes_around_every_staging_boundary(twg):
         twg.check(L.twg_memcpy_d2h(back.data_ptr() + 3, dev.ptr, nb, None))
         assert torch.equal(back[3:3 + nb], raw[off:off + nb]), nb
         assert bool((back[:3] == 0xEE).all()) and bool((back[3 + nb:3 + nb + 61] == 0xEE).all()), nb
+
+
+def test_copies_with_a_small_pinned_ring(twg):
+    # TWG_STAGE_RING_MIB shrinks the pinned ring (what the library also does by itself when
+    # 64 MiB cannot be pinned): every copy size must still round-trip.  The variable is read
+    # when the ring is created, hence a process of its own.
+    import subprocess
+    import sys
+    code = r"""
+import sys, ctypes, torch
+sys.path.insert(0, sys.argv[1])
+import twg_capi as capi
+L = capi.load(); capi.init()
+g = torch.Generator().manual_seed(5)
+mib = 1 << 20
+raw = torch.randint(0, 256, (40 * mib + 200,), dtype=torch.uint8, generator=g)
+back = torch.empty_like(raw)
+dev = capi.DeviceBuffer(raw.numel())
+for nb in (300, 70000, mib + 1, 3 * mib + 7, 4 * mib, 4 * mib + 1, 9 * mib + 5, 40 * mib + 99):
+    capi.check(L.twg_memcpy_h2d(dev.ptr, raw.data_ptr() + 1, nb - 1, None))
+    back.fill_(0xEE)
+    capi.check(L.twg_memcpy_d2h(back.data_ptr() + 2, dev.ptr, nb - 1, None))
+    assert torch.equal(back[2:nb + 1], raw[1:nb]), nb
+    assert int(back[1]) == 0xEE and int(back[nb + 1]) == 0xEE, nb
+print("small ring ok")
+"""
+    env = dict(os.environ, TWG_STAGE_RING_MIB="4")
+    pkg = os.path.dirname(os.path.abspath(twg.__file__))
+    r = subprocess.run([sys.executable, "-c", code, pkg], env=env, capture_output=True, text=True,
+                       timeout=150)
+    assert r.returncode == 0 and "small ring ok" in r.stdout, r.stdout + r.stderr
 
 
 # --------------------------------------------------------------------- add

@@ -122,7 +122,8 @@ size_t piece_for(size_t nbytes, bool to_device) {
 struct Staging {
   std::mutex mu;
   bool ready = false;
-  char *base = nullptr;  // one pinned allocation of kStageRingBytes
+  char *base = nullptr;  // one pinned allocation of ring_bytes
+  size_t ring_bytes = 0;  // kStageRingBytes, or a quarter of it where that much cannot be pinned
   // The ring as the copy in progress divides it: `slots` pieces of `piece` bytes.
   size_t piece = 0;
   int slots = 0;
@@ -289,8 +290,18 @@ int staging_prepare_locked(Staging &s) {
   if (s.ready) return 0;
   // coherent: small downloads are stored into the ring by a kernel and read by the host while
   // that kernel is still running
-  TWG_HIP_TRY(hipHostMalloc((void **)&s.base, kStageRingBytes,
-                            hipHostMallocCoherent | hipHostMallocMapped));
+  s.ring_bytes = kStageRingBytes;
+  if (const char *mib = getenv("TWG_STAGE_RING_MIB")) {  // hosts that can pin little memory
+    const long v = atol(mib);
+    if (v >= 4 && v <= 64) s.ring_bytes = (size_t)v << 20;
+  }
+  hipError_t e = hipHostMalloc((void **)&s.base, s.ring_bytes, hipHostMallocCoherent | hipHostMallocMapped);
+  if (e == hipErrorOutOfMemory) {  // a tight limit on pinned memory: a smaller ring still works
+    (void)hipGetLastError();
+    s.ring_bytes = s.ring_bytes / 4 < (size_t(4) << 20) ? size_t(4) << 20 : s.ring_bytes / 4;
+    e = hipHostMalloc((void **)&s.base, s.ring_bytes, hipHostMallocCoherent | hipHostMallocMapped);
+  }
+  TWG_HIP_TRY(e);
   for (int i = 0; i < kStageSlots; ++i)
     TWG_HIP_TRY(hipEventCreateWithFlags(&s.ev[i], hipEventDisableTiming));
   TWG_HIP_TRY(hipHostMalloc((void **)&s.mailbox, kMailboxBytes + 64,
@@ -320,12 +331,13 @@ int staging_drain_locked(Staging &s) {
 // Divide the ring for a copy of nbytes.  Slots of another size overlap the old ones, so
 // DMAs still reading those are waited for first.
 int staging_divide_locked(Staging &s, size_t nbytes, bool to_device) {
-  const size_t piece = piece_for(nbytes, to_device);
+  size_t piece = piece_for(nbytes, to_device);
+  if (piece > s.ring_bytes / 4) piece = s.ring_bytes / 4;
   if (piece != s.piece) {
     int rc = staging_drain_locked(s);
     if (rc) return rc;
     s.piece = piece;
-    const size_t fit = kStageRingBytes / piece;
+    const size_t fit = s.ring_bytes / piece;
     s.slots = fit < (size_t)kStageSlots ? (int)fit : kStageSlots;
   }
   return 0;
@@ -368,7 +380,6 @@ constexpr uint32_t kFlowMaxPieces = (uint32_t)(kFlowMaxBytes / kFlowPiece);
 constexpr int kFlowBlocks = 8;
 constexpr int kFlowLanes = 1024;
 static_assert(kFlowMaxPieces * sizeof(uint32_t) <= kFlowFlagBytes, "one flag per piece");
-static_assert(kFlowMaxBytes <= kStageRingBytes, "a small download fits the ring");
 
 template <typename V>
 __device__ __forceinline__ uint32_t flow_copy(uint8_t *dst, const uint8_t *src, uint32_t len,
@@ -736,7 +747,7 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
     std::memcpy(dst, st.mailbox, nbytes);
     return 0;
   }
-  if (nbytes <= kFlowMaxBytes) {
+  if (nbytes <= kFlowMaxBytes && nbytes <= st.ring_bytes) {
     const uint32_t seq = ++st.flow_seq;
     const uint32_t npieces = (uint32_t)((nbytes + kFlowPiece - 1) / kFlowPiece);
     const int blocks = npieces < (uint32_t)kFlowBlocks ? (int)npieces : kFlowBlocks;
