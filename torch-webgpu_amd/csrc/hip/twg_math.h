@@ -72,11 +72,11 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
 // formed as a rounded product plus its exact FMA residual, and the exponent is
 // split the same way, so the result keeps about 4e-7 relative error down into
 // the far negative tail where x*Phi(x) is ~1e-38 (plain 0.5*x*(1+erf(x/sqrt 2))
-// has lost every digit by x = -6).  Below 2^-96 the exponential is evaluated 64
-// binades up and the result scaled back, so subnormal results are rounded once.
+// has lost every digit by x = -6).  The exponential is evaluated 64 binades up and
+// the result scaled back at the end, so subnormal results are rounded once.
 //   x > 0:  x * (1 - Phi(-a)) = x * (1 - q);     x <= 0:  x * q.
-// gelu(+-0) = +-0, gelu(NaN) = NaN, gelu(+inf) = +inf, gelu(-inf) = NaN,
-// gelu(x <= -14.2) = -0.
+// gelu(+-0) = +-0, gelu(NaN) = NaN, gelu(+inf) = +inf, gelu(x <= -14.2) = -0 for finite x
+// (the argument of Phi is clamped at 15, so -inf comes back as -inf).
 __device__ __forceinline__ float gelu_erf_f32(float x) {
   const float a = fminf(fabsf(x), 15.0f);
   const float t = hw_rcp(__fmaf_rn(0.35f, a, 1.0f));
@@ -97,14 +97,15 @@ __device__ __forceinline__ float gelu_erf_f32(float x) {
   const float u_hi = __fmul_rn(-s_hi, kLog2eHi);
   float u_lo = __fmaf_rn(-s_hi, kLog2eHi, -u_hi);
   u_lo = __fmaf_rn(-s_hi, kLog2eLo, u_lo);
-  const bool tiny = u_hi < -96.0f;
-  const float e = hw_exp2(u_hi + (tiny ? 64.0f : 0.0f));
-  const float corr = 1.0f + __fmaf_rn(kLn2, u_lo, -s_lo);
-  const float q = (e * corr) * g;  // Phi(-a), times 2^64 when tiny
-  const float xs = tiny ? x * 0x1p-64f : x;
+  // The exponential is always taken 64 binades up (u_hi >= -163 because a <= 15, so the
+  // argument stays above v_exp_f32's flush threshold of -126) and the factor 2^-64 is
+  // applied last: results that are subnormal are then rounded exactly once.
+  const float e = hw_exp2(u_hi + 64.0f);
+  const float eg = e * g;
+  const float q = __fmaf_rn(eg, __fmaf_rn(kLn2, u_lo, -s_lo), eg);  // Phi(-a) * 2^64
   // x > 0 (not >=) so that -0.0 takes the product branch and keeps its sign;
-  // x * (1 - q) rather than x - x*q so that +inf stays +inf (q is never 0 here).
-  return (x > 0.0f) ? x * (1.0f - q) : xs * q;
+  // x * (1 - Phi(-a)) rather than x - x*Phi(-a) so that +inf stays +inf.
+  return (x > 0.0f) ? x * __fmaf_rn(q, -0x1p-64f, 1.0f) : (x * q) * 0x1p-64f;
 }
 
 }  // namespace twg
