@@ -54,7 +54,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this op path is single-GPU (no collectives, nothing to shard in one "
-            "process); run with --gpus 1.  How it would shard is described in DESIGN.md.")
+            "process); run with --gpus 1.  Across GPUs every op would split along the flattened "
+            "element axis with no exchange; masked_select adds one scan of the per-GPU counts.")
         sys.exit(2)
 
     import torch
