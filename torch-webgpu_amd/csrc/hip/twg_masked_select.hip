@@ -41,8 +41,11 @@ namespace {
 
 constexpr int kSteps = 8;           // steps of 256 elements per wavefront (tile variants)
 constexpr int kWaveElems = 256 * kSteps;
-constexpr int kScalarWaves = 4;     // fallback variants: one element per lane
-constexpr int kMsMinTile = 64 * kScalarWaves * kSteps;  // smallest tile of any variant
+constexpr int kScalarWaves = 16;    // fallback variants: one element per lane,
+constexpr int kScalarSteps = 16;    //   16 wavefronts x 16 steps of 64 elements per tile
+constexpr int kScalarTile = 64 * kScalarWaves * kScalarSteps;
+constexpr int kMsMinTile = 256 * kSteps * 4;  // smallest tile of any variant (ms_compact_vec<4>)
+static_assert(kScalarTile >= kMsMinTile, "the scratch is sized for kMsMinTile-element tiles");
 constexpr size_t kMsHeaderBytes = 256;                  // tickets and carry, padded
 constexpr int kLookPerLane = 4;                         // look-back window = 64 * 4 tiles
 
@@ -433,7 +436,7 @@ template <bool STRIDED, typename T>
 __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     T *out, int64_t *d_count, const T *src, const uint8_t *mask, int64_t n,
     uint32_t ntiles, uint32_t *ticket, uint64_t *status, MsGeom g) {
-  constexpr int kWaveSpan = 64 * kSteps;
+  constexpr int kWaveSpan = 64 * kScalarSteps;
   constexpr int kTileElems = kWaveSpan * kScalarWaves;
 
   __shared__ uint32_t s_tile;
@@ -448,12 +451,12 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
   const uint32_t tile = s_tile;
   const int64_t wstart = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
 
-  bool sel[kSteps];
-  uint32_t loff[kSteps];
-  int64_t soff[kSteps];
+  bool sel[kScalarSteps];
+  uint32_t loff[kScalarSteps];
+  int64_t soff[kScalarSteps];
   uint32_t wtotal = 0;
 #pragma unroll
-  for (int k = 0; k < kSteps; ++k) {
+  for (int k = 0; k < kScalarSteps; ++k) {
     const int64_t e = wstart + k * 64 + lane;
     bool f = false;
     soff[k] = e;
@@ -487,14 +490,14 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     if (w < wave) wave_base += t;
     tile_total += t;
   }
-  T vals[kSteps];
+  T vals[kScalarSteps];
 #pragma unroll
-  for (int k = 0; k < kSteps; ++k)
+  for (int k = 0; k < kScalarSteps; ++k)
     if (sel[k]) vals[k] = src[soff[k]];
   const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &s_base, nullptr);
   const int64_t wpos = base + wave_base;
 #pragma unroll
-  for (int k = 0; k < kSteps; ++k)
+  for (int k = 0; k < kScalarSteps; ++k)
     if (sel[k]) out[wpos + loff[k]] = vals[k];
 }
 
@@ -604,7 +607,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
     return launch_stream<8, 1>(m);
   }
 
-  const int64_t tile = vec4 ? kSmallTile : (int64_t)kMsMinTile;
+  const int64_t tile = vec4 ? kSmallTile : (int64_t)kScalarTile;
   const int64_t ntiles64 = tiles_of(g.numel, tile);
   if (ntiles64 > INT32_MAX) return TWG_E_UNSUPPORTED;
   const uint32_t ntiles = (uint32_t)ntiles64;
