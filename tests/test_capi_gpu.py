@@ -326,6 +326,32 @@ def test_random_geometries(twg):
         assert rc == 0 and bit_equal(got, ad.to(torch.float32)), dt
 
 
+def test_short_rows_with_a_small_broadcast_operand(twg):
+    # [rows, len] with len below one block's span plus a row vector or a per-row value on
+    # either side of a non-commutative form: the flat kernel, and its fallbacks when the row
+    # length is not a multiple of 4 or a pointer is misaligned
+    g = torch.Generator().manual_seed(41)
+    for rows, ln in ((1000, 4), (333, 8), (4097, 16), (70, 60), (5000, 64), (257, 100), (300, 252),
+                     (129, 62), (64, 256)):
+        _say(f"short rows {rows}x{ln}")
+        big = torch.randn(rows, ln, generator=g)
+        rowv = torch.randn(ln, generator=g)
+        colv = torch.randn(rows, 1, generator=g)
+        for small in (rowv, colv, colv[::2].repeat_interleave(2, 0)[:rows], torch.randn(1, 1, generator=g)):
+            assert bit_equal(H.add(big, small, alpha=-2.5), oracle.add(big, small.expand_as(big), alpha=-2.5))
+            assert bit_equal(H.add(small, big, alpha=-2.5), oracle.add(small.expand_as(big), big, alpha=-2.5))
+            assert torch.equal(H.binary("twg_eq_f32", big, small, out_dtype=torch.bool), torch.eq(big, small))
+        # a strided per-row operand (every third value of a longer vector)
+        col3 = torch.randn(3 * rows, generator=g)[::3].unsqueeze(1)
+        assert bit_equal(H.binary("twg_mul_f32", big, col3), big * col3)
+        # misaligned dense operand and misaligned row vector
+        flat = torch.randn(rows * ln + 1, generator=g)
+        big1 = flat[1:].view(rows, ln)
+        assert bit_equal(H.add(big1, rowv), big1 + rowv)
+        rowv1 = torch.randn(ln + 1, generator=g)[1:]
+        assert bit_equal(H.add(big, rowv1), big + rowv1)
+
+
 def test_mul_and_fused_add_relu(twg):
     g = torch.Generator().manual_seed(6)
     a = torch.randn(70001, generator=g)

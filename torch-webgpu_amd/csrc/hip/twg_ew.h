@@ -40,6 +40,8 @@ constexpr int kThreads = 256;  // 4 wavefronts of 64
 // keep default caching so a following op can hit in L2 / Infinity Cache.
 constexpr int64_t kStreamBytes = int64_t(64) << 20;
 
+inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+
 // ------------------------------------------------------------------ packs
 
 template <typename T, int N>
@@ -180,6 +182,91 @@ __global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const
       const int64_t e = nvec * VEC + threadIdx.x;
       if (e < numel) out[e] = apply<NIN, Op, TO, TA, TB>(op, a[e], NIN == 2 ? b[e] : TB());
     }
+  }
+}
+
+// --------------------------------------------------------------- ew_flat_bc
+// A dense 2-D operand and output with rows shorter than one block's span, plus a small
+// operand broadcast along one of the two dimensions (a bias over [rows, 64], a per-row
+// scale): walking whole rows would leave most lanes of a block idle (30% of peak at 64
+// elements per row), so the dense side is walked as one flat array, like ew_contig, and the
+// small operand is indexed by column (e % len) or by row (e / len) per pack.  It stays in
+// cache and carries no nontemporal hint.  BC_A: operand a is the small one; BC_ROW: it is a
+// row vector (unit stride along dimension 0), otherwise one value per row.
+template <bool BC_A, bool BC_ROW, bool STREAM, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(64) void ew_flat_bc(TO *out, const TA *a, const TB *b, uint32_t numel,
+                                                 uint32_t len, int64_t bc_stride, Op op) {
+  constexpr int VEC = 4;
+  using PO = Pack<TO, VEC>;
+  using PA = Pack<TA, VEC>;
+  using PB = Pack<TB, VEC>;
+  const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+  const uint32_t e0 = i * VEC;  // len is a multiple of VEC: a pack never crosses a row end
+  if (e0 >= numel) return;
+  PA va;
+  PB vb;
+  if constexpr (BC_A) {
+    vb = load_pack<STREAM, PB, true>(reinterpret_cast<const PB *>(b) + i);
+    if constexpr (BC_ROW) {
+      va = load_pack<false>(reinterpret_cast<const PA *>(a + e0 % len));
+    } else {
+      const TA x = a[(int64_t)(e0 / len) * bc_stride];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) va.v[k] = x;
+    }
+  } else {
+    va = load_pack<STREAM, PA, true>(reinterpret_cast<const PA *>(a) + i);
+    if constexpr (BC_ROW) {
+      vb = load_pack<false>(reinterpret_cast<const PB *>(b + e0 % len));
+    } else {
+      const TB x = b[(int64_t)(e0 / len) * bc_stride];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) vb.v[k] = x;
+    }
+  }
+  PO r;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) r.v[k] = op(va.v[k], vb.v[k]);
+  store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+}
+
+// Returns TWG_E_UNSUPPORTED when the geometry is not of that kind.
+template <typename Op, typename TO, typename TA, typename TB>
+int launch_flat_bc(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  if constexpr (sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    const int64_t len = g.shape[0];
+    if (g.ndim != 2 || len >= 256 || len % 4 != 0 || g.numel > (int64_t)UINT32_MAX - 1024)
+      return TWG_E_UNSUPPORTED;
+    auto dense = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == len; };
+    auto row_vec = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == 0; };
+    auto col_vec = [&](int o) { return g.stride[o][0] == 0 && g.stride[o][1] >= 0; };
+    if (!dense(0) || !aligned_to(out, sizeof(TO) * 4)) return TWG_E_UNSUPPORTED;
+    const bool bc_a = !dense(1);
+    const int small = bc_a ? 1 : 2, big = bc_a ? 2 : 1;
+    if (!dense(big) || !(row_vec(small) || col_vec(small))) return TWG_E_UNSUPPORTED;
+    const void *big_p = bc_a ? (const void *)b : (const void *)a;
+    const void *small_p = bc_a ? (const void *)a : (const void *)b;
+    const bool bc_row = row_vec(small);
+    if (!aligned_to(big_p, 16) || (bc_row && !aligned_to(small_p, 16))) return TWG_E_UNSUPPORTED;
+    const bool stream = g.numel * (int64_t)(sizeof(TO) + 4) > kStreamBytes;
+    const unsigned grid = (unsigned)((g.numel / 4 + 63) / 64);
+    const uint32_t n32 = (uint32_t)g.numel, len32 = (uint32_t)len;
+    const int64_t bs = g.stride[small][1];
+#define TWG_FLAT(BA, BR)                                                                         \
+  do {                                                                                           \
+    if (stream)                                                                                  \
+      ew_flat_bc<BA, BR, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, n32, len32, bs, op); \
+    else                                                                                         \
+      ew_flat_bc<BA, BR, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, n32, len32, bs, op); \
+  } while (0)
+    if (bc_a && bc_row) TWG_FLAT(true, true);
+    else if (bc_a) TWG_FLAT(true, false);
+    else if (bc_row) TWG_FLAT(false, true);
+    else TWG_FLAT(false, false);
+#undef TWG_FLAT
+    return (int)hipGetLastError();
   }
 }
 
@@ -483,7 +570,6 @@ __global__ __launch_bounds__(kThreads) void ew_generic(TO *out, const TA *a, con
 
 // -------------------------------------------------------------- dispatch
 
-inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
 // One element per lane for the general strided kernel too: a grid capped at 8 workgroups per
 // CU with a grid-stride loop was measured up to 20% slower (all operands stepped: 1.83 against
@@ -702,6 +788,11 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
   }
 
   if constexpr (ALL_SHAPES) {
+    // (i') short dense rows with one small broadcast operand: walked flat
+    if constexpr (NIN == 2) {
+      const int r = launch_flat_bc<Op, TO, TA, TB>(out, a, b, g, op, s);
+      if (r != TWG_E_UNSUPPORTED) return r;
+    }
     if (g.ndim >= 1 && g.stride[0][0] == 1) {
       const int64_t sa0 = g.stride[1][0];
       const int64_t sb0 = (NIN == 2) ? g.stride[2][0] : 1;
