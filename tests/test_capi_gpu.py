@@ -352,6 +352,32 @@ def test_short_rows_with_a_small_broadcast_operand(twg):
         assert bit_equal(H.add(big, rowv1), big + rowv1)
 
 
+def test_short_unit_stride_rows_in_strided_arrangements(twg):
+    # rows of 32..252 elements that are unit-stride (or broadcast) in every operand but laid
+    # out with gaps, permuted outer dimensions or mixed broadcasts: the packed general kernel,
+    # and the element-wise one where a pack would be misaligned
+    g = torch.Generator().manual_seed(43)
+    base = torch.randn(40, 6, 8, 128, generator=g)
+    other = torch.randn(40, 8, 6, 64, generator=g)
+    x = base[..., :64]                       # sliced rows
+    y = other.permute(0, 2, 1, 3)            # permuted outer dimensions
+    for a, b in ((x, y), (y, x), (x, x[:, :1]), (x[:, :, :1], y), (x, torch.randn(64, generator=g)),
+                 (base[..., 32:96], y), (base[..., 4:68], y), (base[..., 1:65], y)):
+        assert bit_equal(H.add(a, b, alpha=0.75), oracle.add(a.expand(40, 6, 8, 64), b.expand(40, 6, 8, 64), alpha=0.75))
+        assert torch.equal(H.binary("twg_eq_f32", a, b, out_dtype=torch.bool), torch.eq(a, b))
+        out = torch.zeros(40, 6, 8, 96)[..., 16:80]
+        assert bit_equal(H.add(a, b, out=out), a + b)
+    import twg_capi as C
+    assert bit_equal(H.unary("twg_unary_f32", x, pre=(C.UNARY_RELU,)), torch.relu(x))
+    got = H.unary("twg_unary_f32", y, pre=(C.UNARY_GELU_ERF,), out=torch.zeros(40, 6, 8, 128)[..., 64:])
+    assert rel_err_ok(got, closed_form64("gelu_erf", y))[0]
+    for ln in (32, 36, 100, 252):
+        z = torch.randn(300, 256, generator=g)[:, :ln]
+        w = torch.randn(300, 1, generator=g)
+        assert bit_equal(H.binary("twg_mul_f32", z, w), z * w)
+        assert bit_equal(H.binary("twg_mul_f32", w, z), w * z)
+
+
 def test_mul_and_fused_add_relu(twg):
     g = torch.Generator().manual_seed(6)
     a = torch.randn(70001, generator=g)
