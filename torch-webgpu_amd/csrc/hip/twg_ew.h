@@ -190,44 +190,65 @@ __global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const
 // operand broadcast along one of the two dimensions (a bias over [rows, 64], a per-row
 // scale): walking whole rows would leave most lanes of a block idle (30% of peak at 64
 // elements per row), so the dense side is walked as one flat array, like ew_contig, and the
-// small operand is indexed by column (e % len) or by row (e / len) per pack.  It stays in
+// small operand is indexed by column (e % len) or by row (e / len): once per pack when the
+// row length is a multiple of the pack (EXACT), element by element otherwise.  It stays in
 // cache and carries no nontemporal hint.  BC_A: operand a is the small one; BC_ROW: it is a
 // row vector (unit stride along dimension 0), otherwise one value per row.
-template <bool BC_A, bool BC_ROW, bool STREAM, typename Op, typename TO, typename TA, typename TB>
+template <bool BC_A, bool BC_ROW, bool EXACT, bool STREAM, typename Op, typename TO, typename TA,
+          typename TB>
 __global__ __launch_bounds__(64) void ew_flat_bc(TO *out, const TA *a, const TB *b, uint32_t numel,
                                                  uint32_t len, int64_t bc_stride, Op op) {
   constexpr int VEC = 4;
   using PO = Pack<TO, VEC>;
   using PA = Pack<TA, VEC>;
   using PB = Pack<TB, VEC>;
+  using TS = typename std::conditional<BC_A, TA, TB>::type;  // element type of the small operand
+  const TS *small = BC_A ? reinterpret_cast<const TS *>(a) : reinterpret_cast<const TS *>(b);
   const uint32_t i = blockIdx.x * 64u + threadIdx.x;
-  const uint32_t e0 = i * VEC;  // len is a multiple of VEC: a pack never crosses a row end
-  if (e0 >= numel) return;
-  PA va;
-  PB vb;
-  if constexpr (BC_A) {
-    vb = load_pack<STREAM, PB, true>(reinterpret_cast<const PB *>(b) + i);
-    if constexpr (BC_ROW) {
-      va = load_pack<false>(reinterpret_cast<const PA *>(a + e0 % len));
-    } else {
-      const TA x = a[(int64_t)(e0 / len) * bc_stride];
+  const uint32_t e0 = i * VEC;
+  if (e0 + VEC <= numel) {
+    // the four values of the small operand that go with elements e0..e0+3
+    Pack<TS, VEC> vs;
+    if constexpr (EXACT) {  // len is a multiple of VEC: a pack never crosses a row end
+      if constexpr (BC_ROW) {
+        vs = load_pack<false>(reinterpret_cast<const Pack<TS, VEC> *>(small + e0 % len));
+      } else {
+        const TS x = small[(int64_t)(e0 / len) * bc_stride];
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) va.v[k] = x;
+        for (int k = 0; k < VEC; ++k) vs.v[k] = x;
+      }
+    } else {
+      uint32_t row = e0 / len, col = e0 - row * len;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        vs.v[k] = BC_ROW ? small[col] : small[(int64_t)row * bc_stride];
+        if (++col == len) {
+          col = 0;
+          ++row;
+        }
+      }
     }
-  } else {
-    va = load_pack<STREAM, PA, true>(reinterpret_cast<const PA *>(a) + i);
-    if constexpr (BC_ROW) {
-      vb = load_pack<false>(reinterpret_cast<const PB *>(b + e0 % len));
+    PA va;
+    PB vb;
+    if constexpr (BC_A) {
+      vb = load_pack<STREAM, PB, true>(reinterpret_cast<const PB *>(b) + i);
+      va = vs;
     } else {
-      const TB x = b[(int64_t)(e0 / len) * bc_stride];
+      va = load_pack<STREAM, PA, true>(reinterpret_cast<const PA *>(a) + i);
+      vb = vs;
+    }
+    PO r;
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) vb.v[k] = x;
+    for (int k = 0; k < VEC; ++k) r.v[k] = op(va.v[k], vb.v[k]);
+    store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+  } else if (e0 < numel) {  // the last numel % VEC elements (never with EXACT)
+    for (uint32_t e = e0; e < numel; ++e) {
+      const uint32_t row = e / len, col = e - row * len;
+      const TS x = BC_ROW ? small[col] : small[(int64_t)row * bc_stride];
+      if constexpr (BC_A) out[e] = op(x, b[e]);
+      else out[e] = op(a[e], x);
     }
   }
-  PO r;
-#pragma unroll
-  for (int k = 0; k < VEC; ++k) r.v[k] = op(va.v[k], vb.v[k]);
-  store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
 }
 
 // Returns TWG_E_UNSUPPORTED when the geometry is not of that kind.
@@ -237,8 +258,9 @@ int launch_flat_bc(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
     return TWG_E_UNSUPPORTED;
   } else {
     const int64_t len = g.shape[0];
-    if (g.ndim != 2 || len >= 256 || len % 4 != 0 || g.numel > (int64_t)UINT32_MAX - 1024)
+    if (g.ndim != 2 || len >= 256 || len < 4 || g.numel > (int64_t)UINT32_MAX - 1024)
       return TWG_E_UNSUPPORTED;
+    const bool exact = len % 4 == 0;
     auto dense = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == len; };
     auto row_vec = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == 0; };
     auto col_vec = [&](int o) { return g.stride[o][0] == 0 && g.stride[o][1] >= 0; };
@@ -249,22 +271,29 @@ int launch_flat_bc(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
     const void *big_p = bc_a ? (const void *)b : (const void *)a;
     const void *small_p = bc_a ? (const void *)a : (const void *)b;
     const bool bc_row = row_vec(small);
-    if (!aligned_to(big_p, 16) || (bc_row && !aligned_to(small_p, 16))) return TWG_E_UNSUPPORTED;
+    if (!aligned_to(big_p, 16) || (exact && bc_row && !aligned_to(small_p, 16)))
+      return TWG_E_UNSUPPORTED;
     const bool stream = g.numel * (int64_t)(sizeof(TO) + 4) > kStreamBytes;
-    const unsigned grid = (unsigned)((g.numel / 4 + 63) / 64);
+    const unsigned grid = (unsigned)(((g.numel + 3) / 4 + 63) / 64);
     const uint32_t n32 = (uint32_t)g.numel, len32 = (uint32_t)len;
     const int64_t bs = g.stride[small][1];
-#define TWG_FLAT(BA, BR)                                                                         \
+#define TWG_FLAT2(BA, BR, EX)                                                                    \
   do {                                                                                           \
     if (stream)                                                                                  \
-      ew_flat_bc<BA, BR, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, n32, len32, bs, op); \
+      ew_flat_bc<BA, BR, EX, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, n32, len32, bs, op); \
     else                                                                                         \
-      ew_flat_bc<BA, BR, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, n32, len32, bs, op); \
+      ew_flat_bc<BA, BR, EX, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, n32, len32, bs, op); \
+  } while (0)
+#define TWG_FLAT(BA, BR)          \
+  do {                            \
+    if (exact) TWG_FLAT2(BA, BR, true); \
+    else TWG_FLAT2(BA, BR, false);      \
   } while (0)
     if (bc_a && bc_row) TWG_FLAT(true, true);
     else if (bc_a) TWG_FLAT(true, false);
     else if (bc_row) TWG_FLAT(false, true);
     else TWG_FLAT(false, false);
+#undef TWG_FLAT2
 #undef TWG_FLAT
     return (int)hipGetLastError();
   }
