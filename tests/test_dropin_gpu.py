@@ -503,3 +503,30 @@ def test_mask_ops_take_every_dtype():
     big = torch.tensor([16777217], dtype=torch.int32)
     assert torch.equal(big.to("webgpu").ne(16777216.0).to("cpu"), big.ne(16777216.0))
 
+
+def test_masked_select_lays_out_large_strided_operands_densely():
+    # from 2^16 elements on, broadcast masks and strided sources are made dense on the device
+    # before the compaction; order and values must be those of the logical row-major walk.
+    # The views are built on the device with the same calls as on the CPU.
+    g = torch.Generator().manual_seed(12)
+    R, C = 512, 256
+    x = torch.randn(R, C, generator=g)
+    wide = torch.randn(R, 2 * C, generator=g)
+    m_rc = torch.rand(R, C, generator=g) < 0.5
+    m_cr = torch.rand(C, R, generator=g) < 0.3
+    m_c = torch.rand(C, generator=g) < 0.5
+    m_r1 = torch.rand(R, 1, generator=g) < 0.5
+    cases = (
+        (x, lambda t: t, m_c, lambda t: t),
+        (x, lambda t: t, m_r1, lambda t: t),
+        (x, lambda t: t.t(), m_cr, lambda t: t),
+        (wide, lambda t: t[:, :C], m_rc, lambda t: t),
+        (wide, lambda t: t[:, 1::2], m_cr, lambda t: t.t()),
+        (x, lambda t: t[:1], m_rc, lambda t: t),            # source broadcast over the mask
+    )
+    for src, sv, m, mv in cases:
+        want = torch.masked_select(sv(src), mv(m))
+        d_src, d_m = sv(dev(src)), mv(dev(m))
+        assert d_src.stride() == sv(src).stride() and d_m.stride() == mv(m).stride()
+        got = torch.masked_select(d_src, d_m)
+        assert bit_equal(got.to("cpu"), want), (d_src.shape, d_src.stride(), d_m.stride())
