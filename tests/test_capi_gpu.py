@@ -332,7 +332,8 @@ def test_short_rows_with_a_small_broadcast_operand(twg):
     # length is not a multiple of 4 or a pointer is misaligned
     g = torch.Generator().manual_seed(41)
     for rows, ln in ((1000, 4), (333, 8), (4097, 16), (70, 60), (5000, 64), (257, 100), (300, 252),
-                     (129, 62), (64, 256), (1001, 5), (77, 63), (401, 10), (3, 7), (50, 3), (1, 9)):
+                     (129, 62), (64, 256), (1001, 5), (77, 63), (401, 10), (3, 7), (50, 3), (1, 9),
+                     (37, 320), (9, 1001), (5, 4092), (3, 4096), (2, 5000)):
         _say(f"short rows {rows}x{ln}")
         big = torch.randn(rows, ln, generator=g)
         rowv = torch.randn(ln, generator=g)

@@ -186,10 +186,11 @@ __global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const
 }
 
 // --------------------------------------------------------------- ew_flat_bc
-// A dense 2-D operand and output with rows shorter than one block's span, plus a small
-// operand broadcast along one of the two dimensions (a bias over [rows, 64], a per-row
-// scale): walking whole rows would leave most lanes of a block idle (30% of peak at 64
-// elements per row), so the dense side is walked as one flat array, like ew_contig, and the
+// A dense 2-D operand and output plus a small operand broadcast along one of the two
+// dimensions (a bias over [rows, 64], one value per row).  Walking whole rows, one block per
+// 256-element row chunk, leaves lanes idle whenever the row length is not a multiple of
+// that (30% of peak at 64 elements per row, 66% at 320..1000), so up to 4096 elements per
+// row the dense side is walked as one flat array, like ew_contig (83% at any length), and the
 // small operand is indexed by column (e % len) or by row (e / len): once per pack when the
 // row length is a multiple of the pack (EXACT), element by element otherwise.  It stays in
 // cache and carries no nontemporal hint.  BC_A: operand a is the small one; BC_ROW: it is a
@@ -258,7 +259,7 @@ int launch_flat_bc(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
     return TWG_E_UNSUPPORTED;
   } else {
     const int64_t len = g.shape[0];
-    if (g.ndim != 2 || len >= 256 || len < 4 || g.numel > (int64_t)UINT32_MAX - 1024)
+    if (g.ndim != 2 || len >= 4096 || len < 4 || g.numel > (int64_t)UINT32_MAX - 1024)
       return TWG_E_UNSUPPORTED;
     const bool exact = len % 4 == 0;
     auto dense = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == len; };
