@@ -128,6 +128,8 @@ def masked_select(x, mask, scratch_bytes=None, out_offset=0, check_guard=False):
     need = L.twg_masked_select_scratch_bytes(n)
     scratch = capi.DeviceBuffer(need if scratch_bytes is None else max(scratch_bytes, 8))
     sb = scratch.nbytes if scratch_bytes is None else scratch_bytes
+    # the scratch may hold anything on entry: the library clears what it needs
+    capi.check(L.twg_fill_bytes(scratch.ptr, 0xA5, scratch.nbytes, None))
     it = _iter_for(shape, None, (xe, me), sort_by_out=False)
     if x.dtype == torch.float32:
         cnt = capi.DeviceBuffer(8)

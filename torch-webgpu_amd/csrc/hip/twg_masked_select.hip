@@ -332,8 +332,11 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t
   __shared__ MsShared<WAVES> sh;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
+  // A launch of a single tile needs no ticket (and no cleared scratch: nothing is looked back at).
   if (threadIdx.x == 0)
-    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh.tile = ntiles == 1
+                  ? 0u
+                  : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t tile = sh.tile;
   // tile bases are wavefront-uniform; everything per lane is a 32-bit offset
@@ -446,7 +449,9 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   if (threadIdx.x == 0)
-    s_tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_tile = ntiles == 1
+                 ? 0u
+                 : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t tile = s_tile;
   const int64_t wstart = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
@@ -611,7 +616,9 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
   const int64_t ntiles64 = tiles_of(g.numel, tile);
   if (ntiles64 > INT32_MAX) return TWG_E_UNSUPPORTED;
   const uint32_t ntiles = (uint32_t)ntiles64;
-  if ((rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
+  // one tile takes no ticket and looks back at nothing: the scratch may hold anything
+  if (ntiles > 1 &&
+      (rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
     return rc;
 
   if (vec4) {
