@@ -379,6 +379,28 @@ def test_short_unit_stride_rows_in_strided_arrangements(twg):
         assert bit_equal(H.binary("twg_mul_f32", w, z), w * z)
 
 
+def test_dense_operand_with_gathered_small_operand(twg):
+    # output and one input dense, the other broadcast or strided over up to four dimensions
+    # with short or ragged rows (a channel bias over [N, C, 7, 7] and the like): the flat
+    # kernel that gathers the small operand, on either side of a non-commutative form
+    g = torch.Generator().manual_seed(47)
+    for shape in ((9, 10, 7, 7), (6, 5, 3, 27), (33, 81), (4, 7, 9, 5), (5, 3, 2, 2), (2, 300, 3)):
+        big = torch.randn(*shape, generator=g)
+        nd = len(shape)
+        for keep in itertools.product((True, False), repeat=nd):
+            if all(keep):
+                continue
+            small = torch.randn(*[s if k else 1 for s, k in zip(shape, keep)], generator=g)
+            _say(f"gathered operand {shape} + {tuple(small.shape)}")
+            assert bit_equal(H.add(big, small, alpha=1.5), oracle.add(big, small.expand(shape), alpha=1.5))
+            assert bit_equal(H.add(small, big, alpha=1.5), oracle.add(small.expand(shape), big, alpha=1.5))
+            assert torch.equal(H.binary("twg_eq_f32", small, big, out_dtype=torch.bool), torch.eq(small, big))
+        # a strided (not broadcast) small side: every other element of a wider tensor
+        wide = torch.randn(*shape[:-1], 2 * shape[-1], generator=g)
+        assert bit_equal(H.binary("twg_mul_f32", big, wide[..., ::2]), big * wide[..., ::2])
+        assert bit_equal(H.binary("twg_mul_f32", wide[..., 1::2], big), wide[..., 1::2] * big)
+
+
 def test_mul_and_fused_add_relu(twg):
     g = torch.Generator().manual_seed(6)
     a = torch.randn(70001, generator=g)

@@ -300,6 +300,143 @@ int launch_flat_bc(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
   }
 }
 
+// --------------------------------------------------------------- ew_flat_nd
+// The same idea for up to four dimensions and any layout of the other operand: output and
+// one input dense (walked flat, one pack per lane), the other input gathered element by
+// element at the offset its own strides give (a channel bias over [N, C, 7, 7], a
+// [B, 1, T, 1] factor).  The lane decomposes its first element index once and steps the
+// coordinates for the other three.  Dimensions beyond ndim are padded with an extent that
+// is never reached and stride 0.
+struct FlatNdGeom {
+  uint32_t numel;
+  uint32_t shape[4];
+  int32_t stride[4];  // of the gathered operand, in elements
+};
+
+template <bool BC_A, bool STREAM, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(64) void ew_flat_nd(TO *out, const TA *a, const TB *b, FlatNdGeom g,
+                                                 Op op) {
+  constexpr int VEC = 4;
+  using PO = Pack<TO, VEC>;
+  using PA = Pack<TA, VEC>;
+  using PB = Pack<TB, VEC>;
+  using TS = typename std::conditional<BC_A, TA, TB>::type;
+  const TS *small = BC_A ? reinterpret_cast<const TS *>(a) : reinterpret_cast<const TS *>(b);
+  const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+  const uint32_t e0 = i * VEC;
+  if (e0 >= g.numel) return;
+  uint32_t c0, c1, c2;
+  int32_t off;
+  {
+    uint32_t rem = e0, q = rem / g.shape[0];
+    c0 = rem - q * g.shape[0];
+    rem = q;
+    q = rem / g.shape[1];
+    c1 = rem - q * g.shape[1];
+    rem = q;
+    q = rem / g.shape[2];
+    c2 = rem - q * g.shape[2];
+    off = (int32_t)c0 * g.stride[0] + (int32_t)c1 * g.stride[1] + (int32_t)c2 * g.stride[2] +
+          (int32_t)q * g.stride[3];
+  }
+  if (e0 + VEC <= g.numel) {
+    Pack<TS, VEC> vs;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      vs.v[k] = small[off];
+      off += g.stride[0];
+      if (++c0 == g.shape[0]) {  // carry into the next dimensions
+        c0 = 0;
+        off += g.stride[1] - (int32_t)g.shape[0] * g.stride[0];
+        if (++c1 == g.shape[1]) {
+          c1 = 0;
+          off += g.stride[2] - (int32_t)g.shape[1] * g.stride[1];
+          if (++c2 == g.shape[2]) {
+            c2 = 0;
+            off += g.stride[3] - (int32_t)g.shape[2] * g.stride[2];
+          }
+        }
+      }
+    }
+    PA va;
+    PB vb;
+    if constexpr (BC_A) {
+      vb = load_pack<STREAM, PB, true>(reinterpret_cast<const PB *>(b) + i);
+      va = vs;
+    } else {
+      va = load_pack<STREAM, PA, true>(reinterpret_cast<const PA *>(a) + i);
+      vb = vs;
+    }
+    PO r;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) r.v[k] = op(va.v[k], vb.v[k]);
+    store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+  } else {  // the last numel % VEC elements
+    for (uint32_t e = e0; e < g.numel; ++e) {
+      const TS x = small[off];
+      if constexpr (BC_A) out[e] = op(x, b[e]);
+      else out[e] = op(a[e], x);
+      off += g.stride[0];
+      if (++c0 == g.shape[0]) {
+        c0 = 0;
+        off += g.stride[1] - (int32_t)g.shape[0] * g.stride[0];
+        if (++c1 == g.shape[1]) {
+          c1 = 0;
+          off += g.stride[2] - (int32_t)g.shape[1] * g.stride[1];
+          if (++c2 == g.shape[2]) {
+            c2 = 0;
+            off += g.stride[3] - (int32_t)g.shape[2] * g.stride[2];
+          }
+        }
+      }
+    }
+  }
+}
+
+// Returns TWG_E_UNSUPPORTED when the geometry is not of that kind.
+template <typename Op, typename TO, typename TA, typename TB>
+int launch_flat_nd(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  if constexpr (sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    if (g.ndim < 2 || g.ndim > 4 || g.numel > (int64_t)UINT32_MAX - 1024) return TWG_E_UNSUPPORTED;
+    auto dense = [&](int o) {
+      int64_t want = 1;
+      for (int d = 0; d < g.ndim; ++d) {
+        if (g.stride[o][d] != want) return false;
+        want *= g.shape[d];
+      }
+      return true;
+    };
+    if (!dense(0) || !aligned_to(out, sizeof(TO) * 4)) return TWG_E_UNSUPPORTED;
+    const bool bc_a = !dense(1);
+    const int small = bc_a ? 1 : 2, big = bc_a ? 2 : 1;
+    if (!dense(big)) return TWG_E_UNSUPPORTED;
+    if (!aligned_to(bc_a ? (const void *)b : (const void *)a, 16)) return TWG_E_UNSUPPORTED;
+    FlatNdGeom fg{};
+    fg.numel = (uint32_t)g.numel;
+    int64_t span = 0;
+    for (int d = 0; d < 4; ++d) {
+      fg.shape[d] = d < g.ndim ? (uint32_t)g.shape[d] : 0x80000000u;
+      fg.stride[d] = 0;
+      if (d < g.ndim) {
+        const int64_t st = g.stride[small][d];
+        if (st > INT32_MAX / 2 || st < -(INT32_MAX / 2)) return TWG_E_UNSUPPORTED;
+        span += (st < 0 ? -st : st) * (g.shape[d] - 1);
+        fg.stride[d] = (int32_t)st;
+      }
+    }
+    if (span > INT32_MAX / 2) return TWG_E_UNSUPPORTED;  // offsets and their carries fit 32 bits
+    const bool stream = g.numel * (int64_t)(sizeof(TO) + 4) > kStreamBytes;
+    const unsigned grid = (unsigned)(((g.numel + 3) / 4 + 63) / 64);
+    if (bc_a && stream) ew_flat_nd<true, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, fg, op);
+    else if (bc_a) ew_flat_nd<true, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, fg, op);
+    else if (stream) ew_flat_nd<false, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, fg, op);
+    else ew_flat_nd<false, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, fg, op);
+    return (int)hipGetLastError();
+  }
+}
+
 // --------------------------------------------------------------- ew_rows
 
 struct RowGeom {
@@ -934,15 +1071,23 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
   }
 
   if constexpr (ALL_SHAPES) {
-    // (i') short dense rows with one small broadcast operand: walked flat
+    // (i-a) dense rows with one small broadcast operand: walked flat
     if constexpr (NIN == 2) {
       const int r = launch_flat_bc<Op, TO, TA, TB>(out, a, b, g, op, s);
       if (r != TWG_E_UNSUPPORTED) return r;
     }
-    // (i'') short unit-stride rows in any arrangement: one pack per lane, div/mod per pack
+    // (i-b) short unit-stride rows in any arrangement: one pack per lane, div/mod per pack
     {
       const int r = launch_generic_vec<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
       if (r != TWG_E_UNSUPPORTED) return r;
+    }
+    // (i-c) rows too short or too ragged for one block per 256-element row chunk: if the
+    // output and one input are dense, walk them flat and gather the other input
+    if constexpr (NIN == 2) {
+      if (g.shape[0] < 256 || g.shape[0] % 4 != 0) {
+        const int r = launch_flat_nd<Op, TO, TA, TB>(out, a, b, g, op, s);
+        if (r != TWG_E_UNSUPPORTED) return r;
+      }
     }
     if (g.ndim >= 1 && g.stride[0][0] == 1) {
       const int64_t sa0 = g.stride[1][0];
@@ -977,6 +1122,11 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
         }
       }
     }
+  }
+  // (iii-b) output and one input dense, the other gathered: flat walk, up to four dimensions
+  if constexpr (ALL_SHAPES && NIN == 2) {
+    const int r = launch_flat_nd<Op, TO, TA, TB>(out, a, b, g, op, s);
+    if (r != TWG_E_UNSUPPORTED) return r;
   }
   // (iv) anything else
   return launch_generic<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
