@@ -427,6 +427,14 @@ int launch_flat_nd(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
       }
     }
     if (span > INT32_MAX / 2) return TWG_E_UNSUPPORTED;  // offsets and their carries fit 32 bits
+    // Gathering pays only where neighbouring lanes read neighbouring (or the same) memory: a
+    // step of at most 4 elements along dimension 0, or an operand small enough to sit in L2.
+    // A full-size operand permuted so that dimension 0 strides far (a transpose) read this way
+    // fetches a cache line per element (8% of peak): that is the tile kernels' case.
+    {
+      const int64_t s0 = g.stride[small][0] < 0 ? -g.stride[small][0] : g.stride[small][0];
+      if (s0 > 4 && (span + 1) * 4 > (int64_t(256) << 10)) return TWG_E_UNSUPPORTED;
+    }
     const bool stream = g.numel * (int64_t)(sizeof(TO) + 4) > kStreamBytes;
     const unsigned grid = (unsigned)(((g.numel + 3) / 4 + 63) / 64);
     if (bc_a && stream) ew_flat_nd<true, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, fg, op);
