@@ -51,6 +51,9 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-op sweep of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of op names to run in the sweep")
+    ap.add_argument("--geometries", action="store_true",
+                    help="instead of the benchmark: time add over families of broadcast and permuted "
+                         "operands (~2^25 elements each) and print their spread as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this op path is single-GPU (no collectives, nothing to shard in one "
@@ -64,6 +67,9 @@ def main():
 
     L = capi.load()
     capi.init()
+    if args.geometries:
+        print(json.dumps(geometry_families(capi, L)), flush=True)
+        return
     dev_name, cus, mem = capi.device_info()
     log(f"device: {dev_name}  CUs={cus}  mem={mem / 2**30:.0f} GiB")
     n = 1 << args.log2n
@@ -257,6 +263,82 @@ def main():
         "device": {"name": dev_name, "compute_units": cus},
     }
     print(json.dumps(out), flush=True)
+
+
+def geometry_families(capi, L):
+    """add.Tensor on ~2^25 fp32 elements with (a) the second operand broadcast in every possible
+    way over a set of 2- to 4-dimensional shapes and (b) the first operand stored in every
+    permutation of its dimensions.  Reports algorithmic bytes / time as % of the HBM peak: the
+    slowest patterns and the median of each family.  Wall-clock over 5 launches, device synced."""
+    import itertools
+
+    def contig(shape):
+        st, acc = [], 1
+        for s in reversed(shape):
+            st.append(acc)
+            acc *= s
+        return list(reversed(st))
+
+    def timed(shape, a_st, b_st, nb):
+        n = 1
+        for s in shape:
+            n *= s
+        da, db, do = capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * max(nb, 1)), capi.DeviceBuffer(4 * n)
+        it = capi.make_iter(shape, contig(shape), a_st, b_st)
+
+        def run():
+            capi.check(L.twg_add_f32(do.ptr, da.ptr, db.ptr, ctypes.c_float(1.0), ctypes.byref(it), None))
+        for _ in range(2):
+            run()
+        capi.sync()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            run()
+        capi.sync()
+        t = (time.perf_counter() - t0) / 5
+        return round((8 * n + 4 * nb) / t / 1e9 / HBM_PEAK_GBS * 100, 1), round(t * 1e3, 4)
+
+    fam = {}
+    rows_ = []
+    for shape in ([2048, 256, 7, 7], [512, 256, 14, 14], [128, 64, 56, 56], [32, 16, 1024, 64],
+                  [32, 16, 256, 256], [16, 2048, 1000], [256, 197, 768], [5792, 5792], [512, 768, 3, 27]):
+        for keep in itertools.product((True, False), repeat=len(shape)):
+            if all(keep) or not any(keep):
+                continue
+            bshape = [s if k else 1 for s, k in zip(shape, keep)]
+            b_st = [st if k else 0 for st, k in zip(contig(bshape), keep)]
+            nb = 1
+            for s in bshape:
+                nb *= s
+            pct, ms = timed(shape, contig(shape), b_st, nb)
+            rows_.append({"pct_hbm_peak": pct, "ms": ms, "a": shape, "b": bshape})
+    rows_.sort(key=lambda r: r["pct_hbm_peak"])
+    fam["broadcast_second_operand"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
+                                       "slowest": rows_[:5]}
+    log(f"broadcast family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
+        f"slowest {rows_[0]['pct_hbm_peak']}%")
+    rows_ = []
+    for shape in ([32, 16, 1024, 64], [64, 128, 64, 64], [256, 197, 768], [512, 3, 224, 96], [128, 56, 56, 96]):
+        nd = len(shape)
+        n = 1
+        for s in shape:
+            n *= s
+        for perm in itertools.permutations(range(nd)):
+            if list(perm) == list(range(nd)):
+                continue
+            phys = contig([shape[p] for p in perm])
+            a_st = [0] * nd
+            for pos, p in enumerate(perm):
+                a_st[p] = phys[pos]
+            pct, ms = timed(shape, a_st, contig(shape), n)
+            rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "a_memory_order": list(perm)})
+    rows_.sort(key=lambda r: r["pct_hbm_peak"])
+    fam["permuted_first_operand"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
+                                     "slowest": rows_[:5]}
+    log(f"permutation family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
+        f"slowest {rows_[0]['pct_hbm_peak']}%")
+    return {"geometry_families": fam, "elements_per_pattern": "about 2^25", "op": "add.Tensor fp32",
+            "bytes": "4 B per element read per full operand + 4 B written; a broadcast operand counts its own size"}
 
 
 def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summarize,
