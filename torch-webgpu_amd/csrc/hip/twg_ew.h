@@ -921,10 +921,18 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
     rg.oshape[d - 1] = g.shape[d];
     for (int o = 0; o < 3; ++o) rg.ostride[o][d - 1] = g.stride[o][d];
   }
-  bool reused[3] = {false, false, false};  // operand k is the same row for every block
+  // operand k is read again and again (broadcast along an outer dimension) and small enough
+  // to stay in the last-level cache (256 MB): it keeps default caching while the streamed
+  // operands carry the hint
+  bool reused[3] = {false, false, false};
   for (int o = 1; o <= NIN; ++o) {
-    reused[o] = true;
-    for (int d = 1; d < g.ndim; ++d) reused[o] = reused[o] && g.stride[o][d] == 0;
+    bool again = false;
+    int64_t footprint = (o == 1 ? sizeof(TA) : sizeof(TB)) * (g.stride[o][0] != 0 ? g.shape[0] : 1);
+    for (int d = 1; d < g.ndim; ++d) {
+      if (g.stride[o][d] == 0) again = again || g.shape[d] > 1;
+      else footprint *= g.shape[d];
+    }
+    reused[o] = again && footprint <= (int64_t(64) << 20);
   }
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
   const unsigned grid = (unsigned)(cpr * rows);
