@@ -41,6 +41,7 @@ extern "C" {
 #define TWG_E_UNSUPPORTED (-2)   /* valid request this build has no kernel for */
 #define TWG_E_SCRATCH_SMALL (-3) /* masked_select scratch buffer too small */
 #define TWG_E_OVERLAP (-4)       /* reserved */
+#define TWG_E_TOO_LARGE (-5)     /* more elements than an entry point with a fixed limit takes */
 
 typedef struct ihipStream_t *twg_stream_t; /* == hipStream_t */
 typedef struct ihipEvent_t *twg_event_t;   /* == hipEvent_t  */
@@ -233,6 +234,21 @@ size_t twg_masked_select_scratch_bytes(int64_t numel);
 int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
                           const uint8_t *mask, const twg_iter_t *it, void *scratch,
                           size_t scratch_bytes, twg_stream_t stream);
+
+/* twg_masked_select_f32 for callers that cannot allocate device memory (code under HIP
+ * graph capture, serving loops with a fixed memory plan, harnesses that forbid hipMalloc):
+ * same kernels, same results, but the tickets and status words live in a device array
+ * that is part of the library's code object (1 MiB + 256 B per GPU, held until the process
+ * ends) instead of a caller-provided scratch buffer.  It has no counterpart in the
+ * reference.  The call allocates nothing and frees nothing once the library is
+ * initialised (call twg_init() first: initialisation itself creates the stream).
+ * it->numel may be at most TWG_MS_STATIC_MAX_NUMEL; larger inputs return TWG_E_TOO_LARGE.
+ * All calls on one GPU share the one array: calls that overlap in time (on different
+ * streams) race; calls on one stream are ordered and each clears what it needs. */
+#define TWG_MS_STATIC_MAX_NUMEL (INT64_C(1) << 30)
+int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
+                                 const uint8_t *mask, const twg_iter_t *it,
+                                 twg_stream_t stream);
 
 /* The same compaction for elements of `elem_size` = 1, 2, 4 or 8 bytes (moved without
  * being looked at, so any dtype of that size; the CPU fallback the reference registers,

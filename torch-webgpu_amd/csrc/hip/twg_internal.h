@@ -44,4 +44,9 @@ int masked_select_launch(void *out, int64_t *d_count, const void *src, int elem_
                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
                          size_t scratch_bytes, twg_stream_t stream);
 
+
+// Look up the address the current device gives the masked_select scratch array that is
+// part of the code object.  Run once per device by the library's init.
+int static_scratch_setup();
+
 }  // namespace twg

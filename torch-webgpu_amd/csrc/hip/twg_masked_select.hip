@@ -655,12 +655,54 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
 
 }  // namespace twg
 
+// ------------------------------------------------- scratch that is never allocated
+// Tickets, carry and status words of twg_masked_select_f32_static live in this array
+// instead of a buffer the caller allocates.  The name below is a host-side handle, not a
+// device address: the address each device gives its copy is looked up once per device
+// (static_scratch_setup, run by the library's init) and only that pointer is ever handed
+// to a kernel or a fill.
+constexpr size_t kStaticScratchBytes =
+    kMsHeaderBytes + sizeof(uint64_t) * (size_t)(TWG_MS_STATIC_MAX_NUMEL / kMsMinTile);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace twg {
+namespace {
+constexpr int kMaxDevices = 16;
+void *g_static_scratch[kMaxDevices] = {};  // per device; written during init only
+}  // namespace
+
+int static_scratch_setup() {
+  int dev = -1;
+  TWG_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return TWG_E_UNSUPPORTED;
+  void *ptr = nullptr;
+  TWG_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr || reinterpret_cast<uintptr_t>(ptr) % 256 != 0) return TWG_E_INVALID_ARG;
+  g_static_scratch[dev] = ptr;
+  return 0;
+}
+}  // namespace twg
+
 extern "C" {
 
 int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const uint8_t *mask,
                           const twg_iter_t *it, void *scratch, size_t scratch_bytes,
                           twg_stream_t stream) {
   return masked_select_launch(out, d_count, src, 4, mask, it, scratch, scratch_bytes, stream);
+}
+
+int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
+                                 const uint8_t *mask, const twg_iter_t *it,
+                                 twg_stream_t stream) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (!it) return TWG_E_INVALID_ARG;
+  if (it->numel > TWG_MS_STATIC_MAX_NUMEL) return TWG_E_TOO_LARGE;
+  int dev = -1;
+  TWG_HIP_TRY(hipGetDevice(&dev));
+  void *ptr = (dev >= 0 && dev < kMaxDevices) ? g_static_scratch[dev] : nullptr;
+  if (!ptr) return TWG_E_UNSUPPORTED;  // not the device the library was initialised on
+  return masked_select_launch(out, d_count, src, 4, mask, it, ptr, kStaticScratchBytes, stream);
 }
 
 }  // extern "C"

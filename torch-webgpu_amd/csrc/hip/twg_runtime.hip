@@ -55,6 +55,10 @@ void do_init() {
     r.status = (int)e;
     return;
   }
+  if (int rc = static_scratch_setup()) {
+    r.status = rc;
+    return;
+  }
   r.status = 0;
 }
 
@@ -516,6 +520,7 @@ const char *twg_error_string(int code) {
     case TWG_E_UNSUPPORTED: return "twg: unsupported request";
     case TWG_E_SCRATCH_SMALL: return "twg: scratch buffer too small";
     case TWG_E_OVERLAP: return "twg: overlapping ranges";
+    case TWG_E_TOO_LARGE: return "twg: input larger than this entry point's fixed limit";
     case -1000: return "twg: not initialised";
     default: break;
   }
