@@ -238,7 +238,7 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
 /* twg_masked_select_f32 for callers that cannot allocate device memory (code under HIP
  * graph capture, serving loops with a fixed memory plan, harnesses that forbid hipMalloc):
  * same kernels, same results, but the tickets and status words live in a device array
- * that is part of the library's code object (1 MiB + 256 B per GPU, held until the process
+ * that is part of the library's code object (2 MiB + 384 B per GPU, held until the process
  * ends) instead of a caller-provided scratch buffer.  It has no counterpart in the
  * reference.  The call allocates nothing and frees nothing once the library is
  * initialised (call twg_init() first: initialisation itself creates the stream).

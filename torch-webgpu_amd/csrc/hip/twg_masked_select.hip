@@ -47,7 +47,26 @@ constexpr int kScalarTile = 64 * kScalarWaves * kScalarSteps;
 constexpr int kMsMinTile = 256 * kSteps * 4;  // smallest tile of any variant (ms_compact_vec<4>)
 static_assert(kScalarTile >= kMsMinTile, "the scratch is sized for kMsMinTile-element tiles");
 constexpr size_t kMsHeaderBytes = 256;                  // tickets and carry, padded
-constexpr int kLookPerLane = 4;                         // look-back window = 64 * 4 tiles
+// Smallest tile of the streaming variant (8 wavefronts x 8 steps x 256 elements) and the
+// status words the scratch must hold: one per kMsMinTile elements for the small-tile
+// variants, or kStreamStatusStride per streaming tile plus the few tiles of its remainder
+// launch (less than one streaming tile, at most 16 small tiles).
+constexpr int64_t kStreamMinTile = 8 * 2048;
+constexpr size_t ms_scratch_bytes(int64_t numel) {
+  if (numel < 0) numel = 0;
+  const size_t small = (size_t)((numel + kMsMinTile - 1) / kMsMinTile);
+  const size_t big = (size_t)(numel / kStreamMinTile) * 4 + 16;  // 4 == kStreamStatusStride
+  return kMsHeaderBytes + sizeof(uint64_t) * (small > big ? small : big);
+}
+constexpr int kLookPerLane = 4;   // look-back window of the small-tile variants = 64 * 4 tiles
+// The streaming variant has few, large tiles: its wavefronts poll the status words of 64
+// predecessors per round instead of 256 and keep the words 32 bytes apart, so that the
+// store that publishes one tile's word does not contend with the polls of its neighbours'
+// words in the same 128-byte line (measured at 2^28 elements: +1.5 points at every density;
+// 16 or 64 bytes apart, or a 128-tile window, changed nothing more).
+constexpr int kStreamLookPerLane = 1;
+constexpr int kStreamStatusStride = 4;  // in 8-byte words (ms_scratch_bytes assumes 4)
+static_assert(kStreamStatusStride == 4, "ms_scratch_bytes sizes the scratch for a stride of 4");
 
 constexpr uint64_t kFlagShift = 62;
 constexpr uint64_t kFlagAggregate = 1ull << kFlagShift;
@@ -106,18 +125,19 @@ __device__ __forceinline__ void wave_offsets(uint32_t c, uint32_t &below, uint32
 // (4 status words per lane, nearest first), waits until all of them have published
 // at least an aggregate, and stops at the nearest one that carries an inclusive
 // prefix.
+template <int LPL, int STRIDE>
 __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t tile, int lane) {
   int64_t exclusive = 0;
   int64_t look = (int64_t)tile - 1 - lane;  // lane's nearest candidate
   while (true) {
-    uint64_t st[kLookPerLane];
+    uint64_t st[LPL];
     while (true) {
       bool pending = false;
 #pragma unroll
-      for (int q = 0; q < kLookPerLane; ++q) {
+      for (int q = 0; q < LPL; ++q) {
         const int64_t idx = look - 64 * q;
         // slots before tile 0 behave like an inclusive prefix of 0
-        st[q] = (idx >= 0) ? status_load(status + idx) : kFlagInclusive;
+        st[q] = (idx >= 0) ? status_load(status + idx * STRIDE) : kFlagInclusive;
         pending |= (st[q] >> kFlagShift) == 0;
       }
       if (__ballot(pending) == 0) break;
@@ -126,7 +146,7 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
     int64_t part = 0;
     bool done = false;
 #pragma unroll
-    for (int q = 0; q < kLookPerLane; ++q) {
+    for (int q = 0; q < LPL; ++q) {
       if (!done) {
         const uint64_t incl = __ballot((st[q] >> kFlagShift) == 2);
         const int64_t val = (int64_t)(st[q] & kValueMask);
@@ -141,7 +161,7 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
     }
     exclusive += wave_sum_i64(part);
     if (done) return exclusive;
-    look -= 64 * kLookPerLane;
+    look -= 64 * LPL;
   }
 }
 
@@ -149,19 +169,19 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
 // with all threads; returns the tile's exclusive prefix to all of them.  s_slot is
 // one int64 of LDS.  The last tile also writes the grand total, plus *carry_in if a
 // previous launch compacted the elements before this one's.
+template <int LPL = kLookPerLane, int STRIDE = 1>
 __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, uint32_t ntiles,
                                                uint32_t tile_total, int64_t *d_count,
                                                int64_t *s_slot, const int64_t *carry_in) {
   const int lane = threadIdx.x & 63;
   if (threadIdx.x < 64) {  // wave 0
+    uint64_t *mine = status + (size_t)tile * STRIDE;
     if (lane == 0)
-      status_store(status + tile,
-                   (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
+      status_store(mine, (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
     int64_t exclusive = 0;
     if (tile != 0) {
-      exclusive = look_back(status, tile, lane);
-      if (lane == 0)
-        status_store(status + tile, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+      exclusive = look_back<LPL, STRIDE>(status, tile, lane);
+      if (lane == 0) status_store(mine, kFlagInclusive | (uint64_t)(exclusive + tile_total));
     }
     if (lane == 0) {
       *s_slot = exclusive;
@@ -253,7 +273,8 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
   f32x4 vals[kDepth];
 #pragma unroll
   for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
-  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
+  const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(
+      status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
 
   // ---- 3. stream: compact a step into the ring, refill its register for kDepth steps
   //         later, write out the lines the step completed.  Position p of this
@@ -538,7 +559,9 @@ int launch_stream(const MsLaunch &m) {
   const int64_t rem = m.numel - nbig * kTile;
   const int64_t nrem = (rem + kSmallTile - 1) / kSmallTile;
   if (nbig > INT32_MAX) return TWG_E_UNSUPPORTED;
-  int rc = twg_fill_bytes(m.scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (size_t)(nbig + nrem),
+  // status words: the big tiles' first, kStreamStatusStride apart, then the remainder's
+  const size_t big_words = (size_t)nbig * kStreamStatusStride;
+  int rc = twg_fill_bytes(m.scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (big_words + (size_t)nrem),
                           m.stream);
   if (rc) return rc;
   hipStream_t s = resolve_stream(m.stream);
@@ -547,7 +570,7 @@ int launch_stream(const MsLaunch &m) {
   if (rem)
     ms_compact_vec<kSmallWaves><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
         m.out, m.d_count, m.src + nbig * kTile, m.mask + nbig * kTile, rem, (uint32_t)nrem,
-        m.ticket + 1, m.status + nbig, m.carry);
+        m.ticket + 1, m.status + big_words, m.carry);
   return (int)hipGetLastError();
 }
 
@@ -559,9 +582,7 @@ using namespace twg;
 extern "C" {
 
 size_t twg_masked_select_scratch_bytes(int64_t numel) {
-  if (numel < 0) numel = 0;
-  const int64_t tiles = (numel + kMsMinTile - 1) / kMsMinTile;
-  return kMsHeaderBytes + sizeof(uint64_t) * (size_t)(tiles > 0 ? tiles : 1);
+  return ms_scratch_bytes(numel);
 }
 
 }  // extern "C"
@@ -661,8 +682,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
 // device address: the address each device gives its copy is looked up once per device
 // (static_scratch_setup, run by the library's init) and only that pointer is ever handed
 // to a kernel or a fill.
-constexpr size_t kStaticScratchBytes =
-    kMsHeaderBytes + sizeof(uint64_t) * (size_t)(TWG_MS_STATIC_MAX_NUMEL / kMsMinTile);
+constexpr size_t kStaticScratchBytes = twg::ms_scratch_bytes(TWG_MS_STATIC_MAX_NUMEL);
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace twg {
