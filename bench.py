@@ -50,6 +50,8 @@ def main():
     ap.add_argument("--log2n", type=int, default=28, help="log2 of the element count (28 = the named config)")
     ap.add_argument("--no-sweep", action="store_true", help="skip the per-op sweep of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-dispatcher", action="store_true",
+                    help="skip the lines timed through device=\"webgpu\" (torch dispatcher, result allocated per call)")
     ap.add_argument("--only", default="", help="comma list of op names to run in the sweep")
     ap.add_argument("--geometries", action="store_true",
                     help="instead of the benchmark: time add over families of broadcast and permuted "
@@ -103,9 +105,21 @@ def main():
         per_launch.batch_avg = s.elapsed_ms(e) / reps
         return per_launch
 
+    # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE + WRITE_SIZE, each scaled by a
+    # transfer of known size); recorded figures, not re-measured by this run
+    traffic = {}
+    tr = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if os.path.exists(tr):
+        with open(tr) as f:
+            for line in f:
+                if "=" in line and not line.startswith("#"):
+                    k, v = line.split("=")
+                    traffic[k.strip()] = int(v)
+
     def summarize(name, kernel, nbytes, ms_list, nelem, extra=None):
         avg = getattr(ms_list, "batch_avg", None) or sum(ms_list) / len(ms_list)
         med = statistics.median(ms_list)
+        moved = traffic.get(f"{name}@2^{args.log2n}")
         d = {
             "op": name, "kernel": kernel, "elements": nelem, "bytes": nbytes,
             "avg_ms": round(avg, 5), "median_ms": round(med, 5), "min_ms": round(min(ms_list), 5),
@@ -116,10 +130,18 @@ def main():
             "GBps_median": round(nbytes / med / 1e6, 1),
             "Gelem_per_s": round(nelem / avg / 1e6, 2),
             "pct_hbm_peak": round(nbytes / avg / 1e6 / HBM_PEAK_GBS * 100, 2),
+            # the same time against the bytes the kernel really moved over HBM (recorded
+            # FETCH_SIZE + WRITE_SIZE): below the algorithmic figure where source lines
+            # without a selected element are never fetched
+            "traffic": moved,
+            "pct_hbm_peak_on_traffic": (round(moved / avg / 1e6 / HBM_PEAK_GBS * 100, 2)
+                                        if moved else None),
         }
         if extra:
             d.update(extra)
-        log(f"  {name:28s} {d['avg_ms']:9.4f} ms  {d['GBps']:8.1f} GB/s  {d['pct_hbm_peak']:6.2f}% of peak")
+        on_traffic = (f"  ({d['pct_hbm_peak_on_traffic']:6.2f}% on measured traffic)"
+                      if moved else "")
+        log(f"  {name:28s} {d['avg_ms']:9.4f} ms  {d['GBps']:8.1f} GB/s  {d['pct_hbm_peak']:6.2f}% of peak{on_traffic}")
         return d
 
     f32 = ctypes.c_float
@@ -207,19 +229,9 @@ def main():
         "algorithmic_bytes_per_launch": dominant["bytes"],
         "avg_launch_ms": dominant["avg_ms"],
     }
-    # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE + WRITE_SIZE, each scaled by
-    # the plain copy kernel); a recorded figure, not re-measured by this run
-    traffic = {}
-    tr = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
-    if os.path.exists(tr):
-        with open(tr) as f:
-            for line in f:
-                if "=" in line and not line.startswith("#"):
-                    k, v = line.split("=")
-                    traffic[k.strip()] = int(v)
-    roofline["traffic"] = traffic.get(dominant["op"] + f"@2^{args.log2n}")
-    for d in head:
-        d["traffic"] = traffic.get(d["op"] + f"@2^{args.log2n}")
+    roofline["traffic"] = dominant["traffic"]
+    roofline["frac_on_traffic"] = (round(dominant["pct_hbm_peak_on_traffic"] / 100, 4)
+                                   if dominant["traffic"] else None)
 
     # ------------------------------------------------------------ sweep of the other configs
     del a_h, b_h
@@ -234,6 +246,14 @@ def main():
         result_sweep = sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summarize,
                              d_out, d_cnt, d_scratch, scratch_bytes, d_src, d_x, it, cnt_host, want)
     ops += result_sweep
+
+    # ------------------------------------------------------------ the product path itself
+    disp = None
+    if not args.no_dispatcher and not only:
+        # release what the C-ABI legs hold first; the dispatcher legs upload their own tensors
+        by_name = {d["op"]: d for d in ops}
+        disp = dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, by_name,
+                                x_h, src_h, m50_h, k50)
 
     # ------------------------------------------------------------ config 1: small add + transfers
     small = None
@@ -259,10 +279,66 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "config1_small_add_and_transfers": small,
+        "dispatcher": disp,
         "ops": ops,
         "device": {"name": dev_name, "compute_units": cus},
     }
     print(json.dumps(out), flush=True)
+
+
+def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, by_name,
+                     x_h, src_h, m_h, k50):
+    """The same ops as a user runs them: `a + b`, `F.gelu(x)`, `torch.eq(p, q)`,
+    `torch.masked_select(x, m)` on device="webgpu" tensors through the torch dispatcher, the
+    result allocated by each call (caching allocator) and, for masked_select, the count
+    waited for and the result shaped.  Timed with events on the library's stream, calls issued
+    back to back; `vs_c_abi` is this time over the C-ABI line of the same op."""
+    import torch.nn.functional as F
+    import torch_webgpu  # noqa: F401
+    res = []
+
+    def line(name, fn, nbytes, ref_ms):
+        # freshly allocated device memory is slower on its first few passes (the driver maps
+        # it on first touch), and these legs upload their own operands: warm up longer
+        ms = time_launches(fn, max(Wm, 2 * K), K)
+        avg = ms.batch_avg
+        d = {"op": name, "avg_ms": round(avg, 5), "GBps": round(nbytes / avg / 1e6, 1),
+             "pct_hbm_peak": round(nbytes / avg / 1e6 / HBM_PEAK_GBS * 100, 2),
+             "c_abi_ms": ref_ms, "vs_c_abi": round(avg / ref_ms, 4) if ref_ms else None}
+        log(f"  {name:28s} {avg:9.4f} ms  {d['GBps']:8.1f} GB/s  {d['pct_hbm_peak']:6.2f}% of peak"
+            f"  ({d['vs_c_abi']} x the C-ABI line)")
+        res.append(d)
+
+    def c_abi(name, key="avg_ms"):
+        d = by_name.get(name)
+        return d.get(key) if d else None
+
+    log("through the dispatcher (device=\"webgpu\") ...")
+    a_h, b_h = W.add_contiguous(n, seed=0)
+    a, b = a_h.to("webgpu"), b_h.to("webgpu")
+    del a_h, b_h
+    line("add", lambda: a + b, 12 * n, c_abi("add"))
+    line("eq", lambda: torch.eq(a, b), 9 * n, c_abi("eq"))
+    del b
+    x = x_h.view(rows, cols).to("webgpu")
+    line("gelu", lambda: F.gelu(x), 8 * n, c_abi("gelu"))
+    line("silu", lambda: F.silu(x), 8 * n, c_abi("silu"))
+    del x
+    # config 3b built on the device: as_strided view with transposed strides + contiguous tensor
+    r3 = 1 << (args.log2n // 2 - 1)
+    c3 = n // r3
+    at = torch.as_strided(a.view(r3, c3), (c3, r3), (1, c3))
+    c = src_h.view(c3, r3).to("webgpu")
+    line("add_transposed", lambda: at + c, 12 * n, c_abi("add_transposed"))
+    del at, a, c
+    src, m = src_h.to("webgpu"), m_h.to("webgpu")
+    got = torch.masked_select(src, m)
+    if got.numel() != k50:
+        raise RuntimeError(f"dispatcher masked_select: {got.numel()} != {k50}")
+    del got
+    line("masked_select_p0.50", lambda: torch.masked_select(src, m), W.masked_select_bytes(n, k50),
+         c_abi("masked_select_p0.50", "op_ms_with_count_readback"))
+    return res
 
 
 def geometry_families(capi, L):
@@ -543,19 +619,23 @@ def cpu_baseline(torch, W, n, x_h, src_h, m_h, step_bytes, bytes_add, bytes_gelu
             model = [l.split(":", 1)[1].strip() for l in f if l.startswith("model name")][0]
     except Exception:
         model = "unknown"
+    # The reference's CPU path is ATen's CPU kernels: its boxed fallback runs them for eq, ne,
+    # bitwise_and and masked_select (csrc/bindings.cpp:27-43), and they are the stated baseline
+    # for every op here.  The single-threaded C restatement of the WGSL arithmetic is nested.
     return {
-        "value": round(step_bytes / step_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-        "sample": f"C oracle (oracle/twg_oracle.c), 1 thread: add on 2^{ns_add.bit_length() - 1}, "
-                  f"gelu on 2^{ns_gelu.bit_length() - 1}, masked_select on 2^{ns_ms.bit_length() - 1} "
-                  "elements, median of 3; per-op GB/s combined into the time of one 2^28 step",
-        "per_op": port,
-        "torch_cpu": {
-            "value": round(step_bytes / step_t / 1e9, 2), "unit": "GB/s", "cores": threads,
-            "cpu_model": model,
-            "sample": f"torch.add / F.gelu / torch.masked_select on 2^{nt.bit_length() - 1} elements, "
-                      "median of 5 (ATen's CPU kernel is the reference's own masked_select)",
-            "per_op": dict({"add_GBps": round(ga, 2), "gelu_GBps": round(gg, 2),
-                            "masked_select_GBps": round(gm, 2)}, **others),
+        "value": round(step_bytes / step_t / 1e9, 2), "unit": "GB/s", "cores": threads,
+        "kind": "reference_cpu", "cpu_model": model,
+        "sample": f"ATen CPU kernels (torch.add, F.gelu, torch.masked_select) on 2^{nt.bit_length() - 1} "
+                  f"elements each, {threads} threads, median of 5; per-op GB/s combined into the "
+                  "time of one step",
+        "per_op": dict({"add_GBps": round(ga, 2), "gelu_GBps": round(gg, 2),
+                        "masked_select_GBps": round(gm, 2)}, **others),
+        "c_port": {
+            "value": round(step_bytes / step_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"oracle/twg_oracle.c, 1 thread: add on 2^{ns_add.bit_length() - 1}, gelu on "
+                      f"2^{ns_gelu.bit_length() - 1}, masked_select on 2^{ns_ms.bit_length() - 1} "
+                      "elements, median of 3",
+            "per_op": port,
         },
     }
 

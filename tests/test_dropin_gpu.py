@@ -530,3 +530,38 @@ def test_masked_select_lays_out_large_strided_operands_densely():
         assert d_src.stride() == sv(src).stride() and d_m.stride() == mv(m).stride()
         got = torch.masked_select(d_src, d_m)
         assert bit_equal(got.to("cpu"), want), (d_src.shape, d_src.stride(), d_m.stride())
+
+
+# ------------------------------------------------------------ overlap and out= checks
+
+def test_shifted_self_copy_raises_instead_of_corrupting():
+    # two dense views of one storage, one element apart: ATen raises a partial-overlap
+    # error for this copy on the CPU, and the device path must not memcpy over itself
+    x_h = torch.arange(1000, dtype=torch.float32)
+    with pytest.raises(RuntimeError, match="single memory location|overlap"):
+        y = x_h.clone()
+        y[1:].copy_(y[:-1])
+    x = dev(x_h)
+    with pytest.raises(RuntimeError, match="single memory location|overlap"):
+        x[1:].copy_(x[:-1])
+    assert bit_equal(x.to("cpu"), x_h)           # nothing was written
+    x[:].copy_(x)                                # the same range onto itself is a no-op
+    assert bit_equal(x.to("cpu"), x_h)
+    a, b = x[:500], x[500:]                      # disjoint halves still copy
+    a.copy_(b)
+    assert bit_equal(x.to("cpu")[:500], x_h[500:])
+
+
+def test_masked_select_out_is_validated():
+    src_h = W.select_source(5000, seed=7)
+    m_h = W.bernoulli_mask(5000, 0.3)
+    src, m = dev(src_h), dev(m_h)
+    with pytest.raises(RuntimeError, match="same scalar type"):
+        torch.masked_select(src, m, out=torch.empty(0, dtype=torch.float64, device="webgpu"))
+    with pytest.raises(RuntimeError):
+        torch.masked_select(src, m, out=torch.empty(0))          # a CPU tensor as out
+    with pytest.raises(RuntimeError, match="single memory location|overlap"):
+        torch.masked_select(src, m, out=src)
+    out = torch.empty(3, device="webgpu")
+    torch.masked_select(src, m, out=out)
+    assert bit_equal(out.to("cpu"), torch.masked_select(src_h, m_h))

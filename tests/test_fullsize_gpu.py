@@ -142,3 +142,42 @@ def test_beyond_32bit_element_indices(twg):
     vals, k = H.masked_select(a, m)
     ref = torch.masked_select(a, m)
     assert k == ref.numel() and torch.equal(vals, ref)
+
+
+# ------------------------------------------------ the same sizes through the dispatcher
+
+def test_full_transposed_add_through_the_dispatcher(twg):
+    # config 3b built on the device: the [8192, 32768] tensor viewed through as_strided with
+    # transposed strides plus a contiguous [32768, 8192] tensor, added by `at + c` behind
+    # device="webgpu" (at::TensorIterator picks the layout and the iteration order)
+    import torch_webgpu  # noqa: F401
+    _say("full-size config 3b through device=\"webgpu\"")
+    a_h, bias_h, c_h = W.broadcast_add_inputs(8192, 32768, seed=2)
+    a, bias, c = a_h.to("webgpu"), bias_h.to("webgpu"), c_h.to("webgpu")
+    assert bit_equal((a + bias).to("cpu"), a_h + bias_h)                          # 3a
+    at = torch.as_strided(a, (32768, 8192), (1, 32768))
+    assert at.device.type == "webgpu" and at.stride() == (1, 32768)
+    r = at + c
+    ref = a_h.as_strided((32768, 8192), (1, 32768)) + c_h
+    assert r.shape == ref.shape and r.stride() == ref.stride()
+    assert bit_equal(r.to("cpu"), ref)
+    del r
+    r2 = c + at                                                                   # operands swapped
+    assert bit_equal(r2.to("cpu"), ref)
+
+
+@pytest.mark.parametrize("kind", ["p0.01", "p0.5", "p0.99", "clustered"])
+def test_full_masked_select_through_the_dispatcher(twg, kind):
+    import torch_webgpu  # noqa: F401
+    _say(f"full-size masked_select through device=\"webgpu\": 2^28, mask {kind}")
+    x_h = W.select_source(N, seed=4)
+    m_h = W.clustered_mask(N, 4096) if kind == "clustered" else W.bernoulli_mask(N, float(kind[1:]))
+    x, m = x_h.to("webgpu"), m_h.to("webgpu")
+    r = torch.masked_select(x, m)
+    assert r.device.type == "webgpu" and r.dim() == 1
+    ref = torch.masked_select(x_h, m_h)
+    assert r.numel() == ref.numel() == int(m_h.sum())
+    assert bit_equal(r.to("cpu"), ref)
+    # a second call right behind the first reuses the freed blocks of the pool
+    r2 = torch.masked_select(x, m)
+    assert bit_equal(r2.to("cpu"), ref)

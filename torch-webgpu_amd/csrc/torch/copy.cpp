@@ -11,6 +11,8 @@
 #include <ATen/ops/copy_native.h>
 #include <torch/library.h>
 
+#include <ATen/MemoryOverlap.h>
+
 #include "twg_torch.h"
 
 namespace torch_webgpu {
@@ -67,8 +69,12 @@ void device_to_device(const at::Tensor &dst, const at::Tensor &src) {
     return;
   }
   if (same_dense_layout(dst, src)) {  // csrc/ops/copy.cpp:95-122
-    if (dst.data_ptr() != src.data_ptr())
+    if (dst.data_ptr() != src.data_ptr()) {
+      // x[1:].copy_(x[:-1]): two dense views of one storage, shifted.  The device copy takes
+      // disjoint ranges only; ATen raises for a partial overlap and so does this path.
+      at::assert_no_partial_overlap(dst, src);
       TWG_CHECK(twg_memcpy_d2d(dst.data_ptr(), src.data_ptr(), nbytes_of(dst), nullptr));
+    }
     return;
   }
   // csrc/ops/copy.cpp:123-134

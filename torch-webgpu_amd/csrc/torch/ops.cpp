@@ -8,6 +8,7 @@
 //                                          masked_select: boxed CPU fallbacks there,
 //                                          device kernels here
 //   csrc/ops/webgpu_ops.cpp:47-66          webgpu:: custom ops and the autograd fallthrough
+#include <ATen/MemoryOverlap.h>
 #include <ATen/ExpandUtils.h>
 #include <ATen/native/TensorIterator.h>
 #include <torch/library.h>
@@ -363,6 +364,14 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
 }
 
 at::Tensor &masked_select_out(const at::Tensor &self, const at::Tensor &mask, at::Tensor &out) {
+  // ATen's checks for the out= form (aten/src/ATen/native/TensorAdvancedIndexing.cpp,
+  // masked_select_out_impl): same dtype, same device, no overlap with the inputs.
+  require_on_device(out, "masked_select");
+  TORCH_CHECK(out.scalar_type() == self.scalar_type(),
+              "masked_select(): self and result must have the same scalar type");
+  at::assert_no_internal_overlap(out);
+  at::assert_no_overlap(out, self);
+  at::assert_no_overlap(out, mask);
   at::Tensor r = ops::masked_select(self, mask);
   out.resize_(r.sizes());
   out.copy_(r);
