@@ -345,7 +345,8 @@ def geometry_families(capi, L):
     """add.Tensor on ~2^25 fp32 elements with (a) the second operand broadcast in every possible
     way over a set of 2- to 4-dimensional shapes and (b) the first operand stored in every
     permutation of its dimensions.  Reports algorithmic bytes / time as % of the HBM peak: the
-    slowest patterns and the median of each family.  Wall-clock over 5 launches, device synced."""
+    slowest patterns and the median of each family.  Median of three batches of 10 launches,
+    each batch between one pair of events on the library's stream."""
     import itertools
 
     def contig(shape):
@@ -364,14 +365,19 @@ def geometry_families(capi, L):
 
         def run():
             capi.check(L.twg_add_f32(do.ptr, da.ptr, db.ptr, ctypes.c_float(1.0), ctypes.byref(it), None))
-        for _ in range(2):
+        for _ in range(3):
             run()
         capi.sync()
-        t0 = time.perf_counter()
-        for _ in range(5):
-            run()
-        capi.sync()
-        t = (time.perf_counter() - t0) / 5
+        batches = []
+        for _ in range(3):  # median of three batches of 10 launches between one event pair
+            e0, e1 = capi.Event(), capi.Event()
+            e0.record()
+            for _ in range(10):
+                run()
+            e1.record()
+            capi.sync()
+            batches.append(e0.elapsed_ms(e1) / 10)
+        t = statistics.median(batches) / 1e3
         return round((8 * n + 4 * nb) / t / 1e9 / HBM_PEAK_GBS * 100, 1), round(t * 1e3, 4)
 
     fam = {}
@@ -390,7 +396,7 @@ def geometry_families(capi, L):
             rows_.append({"pct_hbm_peak": pct, "ms": ms, "a": shape, "b": bshape})
     rows_.sort(key=lambda r: r["pct_hbm_peak"])
     fam["broadcast_second_operand"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
-                                       "slowest": rows_[:5]}
+                                       "slowest": rows_[:5], "all": rows_}
     log(f"broadcast family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
         f"slowest {rows_[0]['pct_hbm_peak']}%")
     rows_ = []
@@ -410,7 +416,7 @@ def geometry_families(capi, L):
             rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "a_memory_order": list(perm)})
     rows_.sort(key=lambda r: r["pct_hbm_peak"])
     fam["permuted_first_operand"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
-                                     "slowest": rows_[:5]}
+                                     "slowest": rows_[:5], "all": rows_}
     log(f"permutation family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
         f"slowest {rows_[0]['pct_hbm_peak']}%")
     return {"geometry_families": fam, "elements_per_pattern": "about 2^25", "op": "add.Tensor fp32",

@@ -248,6 +248,46 @@ def test_add_transposed_operand(twg, rows, cols):
     assert bit_equal(H.add(at3, c3), at3 + c3)
 
 
+@pytest.mark.parametrize("shape,order", [
+    # an operand stored with a short innermost extent that is another dimension than the
+    # output's innermost one, the next memory dimension yet another: (3 channels, a head
+    # size of 16, 56) x (20..40) walked as one transposed dimension
+    ((6, 3, 20, 96), (3, 0, 2, 1)), ((6, 3, 20, 96), (0, 3, 2, 1)), ((5, 16, 24, 64), (3, 0, 2, 1)),
+    ((3, 56, 9, 96), (0, 3, 2, 1)), ((4, 3, 37, 260), (3, 0, 2, 1)), ((2, 7, 33, 300), (0, 3, 2, 1)),
+    ((2, 3, 5, 20), (3, 0, 2, 1)),
+    # batched transposes whose extents and row pitches are not multiples of 4
+    ((4, 197, 72), (0, 2, 1)), ((3, 66, 259), (0, 2, 1)), ((2, 261, 35), (0, 2, 1)),
+    ((5, 19, 1030), (0, 2, 1)), ((300, 77), (1, 0)), ((67, 513), (1, 0)),
+    # dimension 0 of 96..192 elements: the 128 x 64 tile shape
+    ((3, 40, 7, 96), (3, 2, 1, 0)), ((2, 70, 160), (2, 1, 0)), ((130, 192), (1, 0)),
+    # stored [.., x, c] with a short c, wanted [.., c, x]: strips through LDS
+    ((5, 3, 40, 96), (0, 2, 3, 1)), ((5, 3, 40, 96), (2, 0, 3, 1)), ((3, 1000), (1, 0)),
+    ((4, 4, 1027), (0, 2, 1)), ((2, 16, 700), (0, 2, 1)), ((2, 32, 301), (0, 2, 1)),
+    ((2, 33, 300), (0, 2, 1)), ((7, 2, 5000), (0, 2, 1)), ((3, 5, 255), (0, 2, 1)),
+])
+def test_add_permuted_operand_tiles(twg, shape, order):
+    # `a` is stored with its dimensions in `order` (outermost first) and viewed in the logical
+    # order; b and the output are contiguous.  Also with a in the second slot, with both inputs
+    # permuted alike, and from storage offsets that break 16-byte alignment.
+    g = torch.Generator().manual_seed(sum(shape) + order[0])
+    phys = [shape[d] for d in order]
+    inv = [order.index(d) for d in range(len(shape))]
+    for off in (0, 1, 3):
+        base = torch.randn(off + torch.Size(phys).numel(), generator=g)[off:].view(*phys)
+        a = base.permute(*inv)
+        assert tuple(a.shape) == tuple(shape)
+        b = torch.randn(off + torch.Size(shape).numel(), generator=g)[off:].view(*shape)
+        ref = oracle.add(a, b, alpha=0.75)
+        assert bit_equal(H.add(a, b, alpha=0.75), ref)
+        assert bit_equal(H.add(b, a, alpha=0.75), oracle.add(b, a, alpha=0.75))
+        a2 = (base * 0.5 + 1.0).permute(*inv)
+        assert bit_equal(H.add(a, a2, alpha=-1.25), oracle.add(a, a2, alpha=-1.25))
+        out = torch.zeros(off + torch.Size(shape).numel())[off:].view(*shape)
+        assert bit_equal(H.add(a, b, out=out), oracle.add(a, b))
+        r = H.unary("twg_unary_f32", a, pre=(ctypes.c_int(1),))          # relu, contiguous output
+        assert bit_equal(r, torch.relu(a))
+
+
 def test_add_generic_strides_bruteforce(twg):
     g = torch.Generator().manual_seed(5)
     sizes = [3, 4, 2, 5]

@@ -524,6 +524,12 @@ constexpr int kTile = 64;
 struct TileGeom {
   int64_t n0, nt;          // extents of dimension 0 and of the transposed dimension t
   int64_t s0[3], st[3];    // strides along those two, per operand
+  // ew_tile_any only: t may be the product of two dimensions, q (outer, extent nt / psplit,
+  // strides st) and p (inner, extent psplit, strides sp), that lie back to back in the
+  // memory of the transposed operands (their offset along t is the index itself) but not in
+  // the other operands.  psplit == 1: t is one dimension.
+  int64_t sp[3];
+  uint32_t psplit;
   uint32_t tiles0, tilest; // tile counts
   int32_t nbatch;          // remaining dimensions
   int64_t bshape[TWG_MAX_DIMS - 2];
@@ -709,6 +715,236 @@ __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, con
       for (int c = 0; c < 4; ++c)
         o.v[c] = apply<NIN, Op, TO, TA, TB>(op, va[p].v[c], NIN == 2 ? vb[p].v[c] : TB());
       store_pack<true>(reinterpret_cast<PO *>(out + off_o + d0 + tt * g.st[0]), o);
+    }
+  }
+}
+
+// The same tile kernel without its alignment conditions.  Wide global loads and stores need
+// only 4-byte alignment on this hardware, so rows whose pitch is not a multiple of 4 elements
+// (a batched [197, 768] transpose) still move as 16-byte packs; extents that are not multiples
+// of 4 end in packs that are handled element by element.  The transposed dimension may be
+// the product of two dimensions (TileGeom::psplit): an operand stored as [.., q, p] with a short
+// innermost extent p (3 channels, 16, 56) is read in unit-stride runs across q and p, while
+// the output rows are addressed by (t / p, t % p).
+typedef uint32_t U32x4A4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <typename T>
+__device__ __forceinline__ Pack<T, 4> load4_any(const T *p) {
+  const U32x4A4 r = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4 *>(p));
+  Pack<T, 4> out;
+  __builtin_memcpy(&out, &r, 16);
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ void store4_any(T *p, const Pack<T, 4> &x) {
+  U32x4A4 r;
+  __builtin_memcpy(&r, &x, 16);
+  __builtin_nontemporal_store(r, reinterpret_cast<U32x4A4 *>(p));
+}
+// up to 4 elements from p, `valid` of them inside the extent
+template <typename T>
+__device__ __forceinline__ Pack<T, 4> load4_edge(const T *p, int64_t valid) {
+  if (valid >= 4) return load4_any(p);
+  Pack<T, 4> out;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out.v[c] = c < valid ? p[c] : T();
+  return out;
+}
+
+template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO, typename TA,
+          typename TB, int THREADS>
+__global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, const TB *b,
+                                                        TileGeom g, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  constexpr int kPitch = TD0 + 4;
+  __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
+  __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
+
+  uint32_t bid = blockIdx.x;
+  const uint32_t t0i = bid % g.tiles0;
+  bid /= g.tiles0;
+  const uint32_t tti = bid % g.tilest;
+  int64_t r = bid / g.tilest;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const int64_t q = r / g.bshape[d];
+    const int64_t c = r - q * g.bshape[d];
+    r = q;
+    off_o += c * g.bstride[0][d];
+    off_a += c * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
+  }
+  const int64_t base0 = (int64_t)t0i * TD0;
+  const int64_t baset = (int64_t)tti * TT;
+
+  // transposed operands: 4 elements along t per lane -> LDS[t][d0]
+  constexpr int kLanesT = TT / 4, kRowsT = THREADS / kLanesT, kPassT = TD0 / kRowsT;
+  static_assert(TT % 4 == 0 && THREADS % kLanesT == 0 && TD0 % kRowsT == 0, "tile shape");
+  {
+    const int tx = threadIdx.x % kLanesT, ty = threadIdx.x / kLanesT;
+    const int64_t tt = baset + 4 * tx;
+    const int64_t left = g.nt - tt;  // elements of this lane's pack inside the extent
+    if constexpr (A_T) {
+      PA v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t d0 = base0 + ty + kRowsT * p;
+        if (d0 < g.n0 && left > 0) v[p] = load4_edge(a + off_a + d0 * g.s0[1] + tt, left);
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (base0 + rr < g.n0 && left > 0) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sa[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+    if constexpr (NIN == 2 && B_T) {
+      PB v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t d0 = base0 + ty + kRowsT * p;
+        if (d0 < g.n0 && left > 0) v[p] = load4_edge(b + off_b + d0 * g.s0[2] + tt, left);
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (base0 + rr < g.n0 && left > 0) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sb[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+  }
+
+  // everything else: 4 elements along dimension 0 per lane
+  constexpr int kLanes0 = TD0 / 4, kRows0 = THREADS / kLanes0, kPass0 = TT / kRows0;
+  static_assert(TD0 % 4 == 0 && THREADS % kLanes0 == 0 && TT % kRows0 == 0, "tile shape");
+  const int tx = threadIdx.x % kLanes0, ty = threadIdx.x / kLanes0;
+  const int64_t d0 = base0 + 4 * tx;
+  const int64_t left0 = g.n0 - d0;
+  // offset of row tt of operand o: a plain stride, or (tt / p, tt % p) on two of them
+  auto row_off = [&](int64_t tt, int o) -> int64_t {
+    if (g.psplit <= 1) return tt * g.st[o];
+    const uint32_t q = (uint32_t)tt / g.psplit;
+    const uint32_t rem = (uint32_t)tt - q * g.psplit;
+    return (int64_t)q * g.st[o] + (int64_t)rem * g.sp[o];
+  };
+  PA va[kPass0];
+  PB vb[kPass0];
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int64_t tt = baset + ty + kRows0 * p;
+    if (left0 > 0 && tt < g.nt) {
+      if constexpr (!A_T) va[p] = load4_edge(a + off_a + d0 + row_off(tt, 1), left0);
+      if constexpr (NIN == 2 && !B_T) vb[p] = load4_edge(b + off_b + d0 + row_off(tt, 2), left0);
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int rr = ty + kRows0 * p;
+    const int64_t tt = baset + rr;
+    if (left0 > 0 && tt < g.nt) {
+      if constexpr (A_T) va[p] = *reinterpret_cast<const PA *>(&sa[rr][4 * tx]);
+      if constexpr (NIN == 2 && B_T) vb[p] = *reinterpret_cast<const PB *>(&sb[rr][4 * tx]);
+      PO o;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        o.v[c] = apply<NIN, Op, TO, TA, TB>(op, va[p].v[c], NIN == 2 ? vb[p].v[c] : TB());
+      TO *dst = out + off_o + d0 + row_off(tt, 0);
+      if (left0 >= 4) {
+        store4_any(dst, o);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (c < left0) dst[c] = o.v[c];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------ ew_deint
+// An operand stored as [.., x, c] with a short innermost extent c (3 colour channels, a handful
+// of heads) against an output laid out [.., c, x]: the operand's stride along dimension 0 is the
+// extent of c.  A block reads a strip of TX * c consecutive elements with 16-byte loads, parks
+// it in LDS as it lies in memory, and writes c runs of TX output elements, picking the strip up
+// with a stride of c.  (Through the gather kernel these layouts ran at 51% of HBM peak.)
+constexpr int kDeintLds = 8192;  // elements of one strip at most
+
+template <int NIN, bool A_D, bool B_D, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                     uint32_t tx_elems, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  __shared__ __attribute__((aligned(16))) TA sa[A_D ? kDeintLds : 4];
+  __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_D) ? kDeintLds : 4];
+
+  uint32_t bid = blockIdx.x;
+  const uint32_t t0i = bid % g.tiles0;
+  int64_t r = bid / g.tiles0;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const int64_t q = r / g.bshape[d];
+    const int64_t c = r - q * g.bshape[d];
+    r = q;
+    off_o += c * g.bstride[0][d];
+    off_a += c * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
+  }
+  const uint32_t P = (uint32_t)g.nt;
+  const int64_t x0 = (int64_t)t0i * tx_elems;
+  const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)tx_elems ? g.n0 - x0 : (int64_t)tx_elems);
+  const uint32_t strip = nx * P;  // consecutive elements of a deinterleaved operand
+  if constexpr (A_D) {
+    const TA *src = a + off_a + x0 * (int64_t)P;
+    for (uint32_t i = 4 * threadIdx.x; i < strip; i += 4 * kThreads)
+      *reinterpret_cast<PA *>(&sa[i]) = load4_edge(src + i, (int64_t)strip - i);
+  }
+  if constexpr (NIN == 2 && B_D) {
+    const TB *src = b + off_b + x0 * (int64_t)P;
+    for (uint32_t i = 4 * threadIdx.x; i < strip; i += 4 * kThreads)
+      *reinterpret_cast<PB *>(&sb[i]) = load4_edge(src + i, (int64_t)strip - i);
+  }
+  __syncthreads();
+  const uint32_t packs = (nx + 3) / 4;  // per channel
+  for (uint32_t idx = threadIdx.x; idx < packs * P; idx += kThreads) {
+    const uint32_t c = idx / packs, j = idx - c * packs;
+    const uint32_t x = 4 * j;
+    const int64_t left = (int64_t)nx - x;
+    PA va;
+    PB vb;
+    if constexpr (A_D) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) va.v[k] = k < left ? sa[(x + k) * P + c] : TA();
+    } else {
+      va = load4_edge(a + off_a + x0 + x + (int64_t)c * g.st[1], left);
+    }
+    if constexpr (NIN == 2) {
+      if constexpr (B_D) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) vb.v[k] = k < left ? sb[(x + k) * P + c] : TB();
+      } else {
+        vb = load4_edge(b + off_b + x0 + x + (int64_t)c * g.st[2], left);
+      }
+    }
+    PO o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
+    TO *dst = out + off_o + x0 + x + (int64_t)c * g.st[0];
+    if (left >= 4) {
+      store4_any(dst, o);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (k < left) dst[k] = o.v[k];
     }
   }
 }
@@ -965,20 +1201,31 @@ int launch_rows(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStre
   return launch_rows_v<NIN, 1, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
 }
 
+// t: the dimension the transposed operands have their unit stride along; or, with pin >= 1,
+// the outer one of two dimensions (t, pin) that lie back to back in those operands' memory
+// (unit stride along pin, stride shape[pin] along t) and are walked as one.
 template <int NIN, typename Op, typename TO, typename TA, typename TB>
 int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
-                hipStream_t s) {
+                hipStream_t s, int pin = -1) {
   TileGeom tg{};
   tg.n0 = g.shape[0];
   tg.nt = g.shape[t];
+  tg.psplit = 1;
   for (int o = 0; o < 3; ++o) {
     tg.s0[o] = g.stride[o][0];
     tg.st[o] = g.stride[o][t];
+    tg.sp[o] = 0;
+  }
+  if (pin >= 1) {
+    if (g.shape[t] * g.shape[pin] >= (int64_t(1) << 31)) return TWG_E_UNSUPPORTED;
+    tg.nt = g.shape[t] * g.shape[pin];
+    tg.psplit = (uint32_t)g.shape[pin];
+    for (int o = 0; o < 3; ++o) tg.sp[o] = g.stride[o][pin];
   }
   int64_t batch = 1;
   tg.nbatch = 0;
   for (int d = 1; d < g.ndim; ++d) {
-    if (d == t) continue;
+    if (d == t || d == pin) continue;
     tg.bshape[tg.nbatch] = g.shape[d];
     for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
     tg.nbatch++;
@@ -1006,9 +1253,46 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       ok = ok && (b_t ? (tg.st[2] == 1 && tg.s0[2] % 4 == 0) : (tg.s0[2] == 1 && tg.st[2] % 4 == 0));
     for (int d = 0; d < tg.nbatch && ok; ++d)
       for (int o = 0; o <= NIN; ++o) ok = ok && tg.bstride[o][d] % 4 == 0;
+    ok = ok && pin < 0;
+    // tile shape by the extent of dimension 0: 256 x 32 from 256 on, 128 x 64 where a 128-wide
+    // tile wastes no more lanes than two 64-wide ones (96: 54% -> 6x% of peak), else 64 x 64
+    const bool wide = tg.n0 >= 256;
+    const bool mid = !wide && tg.n0 > 64 && (tg.n0 % 128 == 0 || tg.n0 % 128 > 64);
+    if (!ok) {
+      // The same tiles without the alignment conditions, and with (t, pin) walked as one
+      // dimension: needs the unit strides only.
+      auto unit_t = [&](int o) {
+        return pin >= 1 ? (tg.sp[o] == 1 && tg.st[o] == (int64_t)tg.psplit) : tg.st[o] == 1;
+      };
+      bool any = tg.s0[0] == 1 && (a_t ? unit_t(1) : tg.s0[1] == 1);
+      if (NIN == 2) any = any && (b_t ? unit_t(2) : tg.s0[2] == 1);
+      if (any) {
+        if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid)) return TWG_E_UNSUPPORTED;
+        const bool big = g.numel >= (int64_t(1) << 27);
+#define TWG_LAUNCH_TILE_ANY(AT, BT)                                                              \
+  do {                                                                                           \
+    if (wide && big)                                                                             \
+      ew_tile_any<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 1024><<<grid, 1024, 0, s>>>(out, a, b, tg, op); \
+    else if (wide)                                                                               \
+      ew_tile_any<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else if (mid)                                                                                \
+      ew_tile_any<NIN, AT, BT, 128, 64, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else                                                                                         \
+      ew_tile_any<NIN, AT, BT, 64, 64, Op, TO, TA, TB, kThreads><<<grid, kThreads, 0, s>>>(out, a, b, tg, op); \
+  } while (0)
+        if (a_t && b_t) {
+          if constexpr (NIN == 2) TWG_LAUNCH_TILE_ANY(true, true);
+        } else if (a_t) {
+          TWG_LAUNCH_TILE_ANY(true, false);
+        } else {
+          if constexpr (NIN == 2) TWG_LAUNCH_TILE_ANY(false, true);
+        }
+#undef TWG_LAUNCH_TILE_ANY
+        return (int)hipGetLastError();
+      }
+    }
     if (ok) {
-      const bool wide = tg.n0 >= 256;
-      if (!set_tiles(wide ? 256 : 64, wide ? 32 : 64, &grid)) return TWG_E_UNSUPPORTED;
+      if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid)) return TWG_E_UNSUPPORTED;
       // 256x32 tiles: 512 lanes per tile measured 2-4 points ahead of 256 from 2^22 to 2^26
       // elements (67% -> 71% at 2^24), 1024 lanes another point ahead at 2^28 (77.6%)
       const bool big = g.numel >= (int64_t(1) << 27);
@@ -1018,6 +1302,8 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 1024><<<grid, 1024, 0, s>>>(out, a, b, tg, op); \
     else if (wide)                                                                               \
       ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else if (mid)                                                                                \
+      ew_tile_vec<NIN, AT, BT, 128, 64, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
     else                                                                                         \
       ew_tile_vec<NIN, AT, BT, 64, 64, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);  \
   } while (0)
@@ -1033,6 +1319,7 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     }
   }
 
+  if (pin >= 1) return TWG_E_UNSUPPORTED;  // the dword kernel walks one dimension only
   if (!set_tiles(kTile, kTile, &grid)) return TWG_E_UNSUPPORTED;
   if (a_t && b_t) {
     if constexpr (NIN == 2)
@@ -1044,6 +1331,57 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       ew_tile<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
   }
   return (int)hipGetLastError();
+}
+
+// Dimension 0 (extent X) and dimension pd (short extent P) form one unit-stride run of X * P
+// elements in the operands marked *_d, while the output and the other operands have their unit
+// stride along dimension 0.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool a_d, bool b_d,
+                 Op op, hipStream_t s) {
+  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    const int64_t P = g.shape[pd];
+    if (P < 2 || P > 32 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
+    auto run_of = [&](int o) { return g.stride[o][pd] == 1 && g.stride[o][0] == P; };
+    if (a_d ? !run_of(1) : g.stride[1][0] != 1) return TWG_E_UNSUPPORTED;
+    if (NIN == 2 && (b_d ? !run_of(2) : g.stride[2][0] != 1)) return TWG_E_UNSUPPORTED;
+    TileGeom tg{};
+    tg.n0 = g.shape[0];
+    tg.nt = P;
+    for (int o = 0; o < 3; ++o) {
+      tg.s0[o] = g.stride[o][0];
+      tg.st[o] = g.stride[o][pd];
+    }
+    int64_t batch = 1;
+    tg.nbatch = 0;
+    for (int d = 1; d < g.ndim; ++d) {
+      if (d == pd) continue;
+      tg.bshape[tg.nbatch] = g.shape[d];
+      for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+      tg.nbatch++;
+      batch *= g.shape[d];
+    }
+    // strip length: 1024 elements of dimension 0 while the strip fits the LDS array
+    uint32_t tx = 1024;
+    while ((int64_t)tx * P > kDeintLds) tx /= 2;
+    const int64_t tiles0 = (tg.n0 + tx - 1) / tx;
+    if (tiles0 > INT32_MAX || tiles0 * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+    tg.tiles0 = (uint32_t)tiles0;
+    tg.tilest = 1;
+    const unsigned grid = (unsigned)(tiles0 * batch);
+    if (a_d && b_d) {
+      if constexpr (NIN == 2)
+        ew_deint<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, op);
+    } else if (a_d) {
+      ew_deint<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, op);
+    } else {
+      if constexpr (NIN == 2)
+        ew_deint<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, op);
+    }
+    return (int)hipGetLastError();
+  }
 }
 
 // Pick the kernel for a canonical geometry.  ALL_SHAPES = false keeps only the dense
@@ -1120,6 +1458,51 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
           r = launch_rows<NIN, false, false, Op, TO, TA, TB>(out, a, b, g, op, s);
         }
         if (r != TWG_E_UNSUPPORTED) return r;
+      }
+      // (iii-00) an input stored [.., x, c] with a short c against an output stored [.., c, x]
+      // (strips of fewer than 256 output elements per channel run no faster than the gather)
+      if (g.ndim >= 2 && g.shape[0] >= 256) {
+        const bool a_x = sa0 != 0 && sa0 != 1, b_x = NIN == 2 && sb0 != 0 && sb0 != 1;
+        if (a_x || b_x) {
+          const int o = a_x ? 1 : 2;
+          int pd = -1;
+          for (int d = 1; d < g.ndim; ++d)
+            if (g.stride[o][d] == 1 && g.shape[d] == g.stride[o][0]) pd = d;
+          if (pd >= 1) {
+            int r = launch_deint<NIN, Op, TO, TA, TB>(out, a, b, g, pd, a_x, b_x, op, s);
+            if (r != TWG_E_UNSUPPORTED) return r;
+          }
+        }
+      }
+      // (iii-0) an input whose two innermost memory dimensions are both other dimensions than
+      // dimension 0, the inner one short (3 channels, a head size): walked as one transposed
+      // dimension so that the tiles stay full
+      if (g.ndim >= 3 && g.shape[0] >= 16) {
+        const bool a_x = sa0 != 0 && sa0 != 1, b_x = NIN == 2 && sb0 != 0 && sb0 != 1;
+        auto pair_of = [&](int o, int *pd, int *qd) {
+          *pd = *qd = -1;
+          for (int d = 1; d < g.ndim; ++d)
+            if (g.stride[o][d] == 1) *pd = d;
+          if (*pd < 0) return false;
+          for (int d = 1; d < g.ndim; ++d)
+            if (d != *pd && g.stride[o][d] == g.shape[*pd]) *qd = d;
+          return *qd >= 1;
+        };
+        int pa = -1, qa = -1, pb = -1, qb = -1;
+        const bool a_pair = a_x && pair_of(1, &pa, &qa);
+        const bool b_pair = b_x && pair_of(2, &pb, &qb);
+        int pd = -1, qd = -1;
+        if (a_x && b_x) {
+          if (a_pair && b_pair && pa == pb && qa == qb) { pd = pa; qd = qa; }
+        } else if (a_pair) {
+          pd = pa; qd = qa;
+        } else if (b_pair) {
+          pd = pb; qd = qb;
+        }
+        if (pd >= 1 && g.shape[pd] < 128 && g.shape[pd] * g.shape[qd] >= 32) {
+          int r = launch_tile<NIN, Op, TO, TA, TB>(out, a, b, g, qd, a_x, b_x, op, s, pd);
+          if (r != TWG_E_UNSUPPORTED) return r;
+        }
       }
       // (iii) an input with its unit stride along another dimension
       if (g.ndim >= 2 && g.shape[0] >= 16) {
