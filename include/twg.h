@@ -104,12 +104,25 @@ int twg_event_elapsed_ms(float *ms, twg_event_t start, twg_event_t stop);
  * WebGPUCachingHostDeleter (csrc/core/webgpu_allocator.cpp:10-29), which create
  * and destroy one Dawn buffer per tensor.  Blocks are rounded up (512 B below
  * 1 MiB, 2 MiB above), kept on per-size free lists when freed and handed out
- * again without touching hipMalloc.  Reuse is safe without events because all
- * work runs in order on one stream.  n == 0 yields *p == NULL and success
+ * again without touching hipMalloc.  A block belongs to the library's in-order
+ * stream: freed, it is reusable at once, because every later launch on that
+ * stream runs after the work that still uses it (the reference gets the same
+ * from Dawn's single queue).  n == 0 yields *p == NULL and success
  * (csrc/core/webgpu_allocator.cpp:33-38). */
 int twg_malloc(void **p, size_t n);
 int twg_free(void *p);
-/* Return every cached (unused) block to the driver. */
+/* Tell the allocator that the block containing p is used by work queued on
+ * `stream`, a stream of the caller's (every entry point takes one).  When such a
+ * block is freed it is neither reused nor released until that work has finished:
+ * twg_free records an event on each recorded stream and the block waits for them
+ * (bytes_pending in twg_mem_stats).  Without this call a block used on another
+ * stream than the library's must not be freed before the caller has synchronised
+ * that stream.  If the stream is being captured into a graph at the time of the
+ * free, the block is held until twg_empty_cache.  No counterpart in the reference
+ * (one queue).  NULL or the library's stream: nothing to do, returns 0. */
+int twg_record_stream(const void *p, twg_stream_t stream);
+/* Return every cached (unused) block to the driver; waits for the library's
+ * stream and for the recorded streams of freed blocks first. */
 int twg_empty_cache(void);
 
 typedef struct twg_mem_stats {
@@ -118,6 +131,7 @@ typedef struct twg_mem_stats {
   int64_t n_device_mallocs; /* hipMalloc calls so far */
   int64_t n_cache_hits;   /* twg_malloc calls served from a free list */
   int64_t n_allocs;       /* twg_malloc calls with n > 0 */
+  int64_t bytes_pending;  /* freed, waiting for work on a recorded stream */
 } twg_mem_stats_t;
 int twg_mem_stats(twg_mem_stats_t *out);
 

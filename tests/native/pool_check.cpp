@@ -1,0 +1,137 @@
+// Drives the allocator's bookkeeping (csrc/hip/twg_pool.h) on the CPU with a backend that
+// hands out host memory and whose "events" complete when the test says so.
+#include <cstdio>
+#include <cstdlib>
+#include <set>
+
+#include "twg_pool.h"
+
+#define CHECK(cond)                                                        \
+  do {                                                                     \
+    if (!(cond)) {                                                         \
+      std::printf("FAILED line %d: %s\n", __LINE__, #cond);                \
+      return 1;                                                            \
+    }                                                                      \
+  } while (0)
+
+struct FakeBackend {
+  using Stream = int;
+  using Event = int;
+  static constexpr int kOutOfMemory = 2;
+  static size_t budget;             // bytes the "device" still has
+  static std::set<void *> device;   // live backend allocations
+  static std::set<int> completed;   // events that have finished
+  static std::set<int> destroyed;
+  static int next_event, syncs, capturing_stream;
+  static std::map<int, int> event_stream;
+  static int alloc(void **p, size_t n) {
+    if (n > budget) return kOutOfMemory;
+    budget -= n;
+    *p = std::malloc(n);
+    device.insert(*p);
+    sizes()[*p] = n;
+    return 0;
+  }
+  static int release(void *p) {
+    if (!device.erase(p)) return 99;
+    budget += sizes()[p];
+    std::free(p);
+    return 0;
+  }
+  static bool record(int s, int *e) {
+    if (s == capturing_stream) return false;
+    *e = next_event++;
+    event_stream[*e] = s;
+    return true;
+  }
+  static bool done(int e) { return completed.count(e) != 0; }
+  static void wait(int e) { completed.insert(e); }
+  static void destroy(int e) { destroyed.insert(e); }
+  static void sync_library_stream() { ++syncs; }
+  static std::map<void *, size_t> &sizes() {
+    static std::map<void *, size_t> m;
+    return m;
+  }
+};
+size_t FakeBackend::budget = size_t(64) << 20;
+std::set<void *> FakeBackend::device;
+std::set<int> FakeBackend::completed, FakeBackend::destroyed;
+int FakeBackend::next_event = 1, FakeBackend::syncs = 0, FakeBackend::capturing_stream = -1;
+std::map<int, int> FakeBackend::event_stream;
+
+int main() {
+  using twg::BlockPool;
+  BlockPool<FakeBackend> pool;
+  void *a = nullptr, *b = nullptr, *c = nullptr;
+
+  // zero bytes, unknown pointers
+  a = reinterpret_cast<void *>(1);
+  CHECK(pool.malloc(&a, 0) == 0 && a == nullptr);
+  CHECK(pool.free(nullptr) == 0);
+  CHECK(pool.free(reinterpret_cast<void *>(12345)) == -1);
+
+  // library-stream block: freed, it is reusable at once, without an event
+  CHECK(pool.malloc(&a, 3 << 20) == 0);
+  CHECK(pool.stats().bytes_in_use == (4 << 20));  // rounded to 2 MiB granules
+  CHECK(pool.free(a) == 0);
+  CHECK(pool.stats().bytes_cached == (4 << 20) && pool.stats().bytes_pending == 0);
+  CHECK(pool.malloc(&b, 3 << 20) == 0 && b == a && pool.stats().n_cache_hits == 1);
+  CHECK(FakeBackend::next_event == 1);
+
+  // the same block used on stream 7 (recorded through an interior address, twice) and on
+  // stream 9: freed, it waits for both events
+  CHECK(pool.record_stream(static_cast<char *>(b) + 100, 7) == 0);
+  CHECK(pool.record_stream(b, 7) == 0);
+  CHECK(pool.record_stream(b, 9) == 0);
+  CHECK(pool.record_stream(static_cast<char *>(b) + (4 << 20), 7) == -1);  // one past the end
+  CHECK(pool.free(b) == 0);
+  CHECK(FakeBackend::next_event == 3);
+  CHECK(FakeBackend::event_stream[1] == 7 && FakeBackend::event_stream[2] == 9);
+  CHECK(pool.stats().bytes_pending == (4 << 20) && pool.stats().bytes_cached == 0);
+  // a request of the same size must not get the pending block
+  CHECK(pool.malloc(&c, 3 << 20) == 0 && c != b);
+  CHECK(pool.stats().n_device_mallocs == 2);
+  FakeBackend::completed.insert(1);  // only one of the two streams is done
+  void *d = nullptr;
+  CHECK(pool.malloc(&d, 3 << 20) == 0 && d != b);
+  CHECK(pool.stats().bytes_pending == (4 << 20));
+  FakeBackend::completed.insert(2);  // now both
+  void *e = nullptr;
+  CHECK(pool.malloc(&e, 3 << 20) == 0 && e == b);
+  CHECK(pool.stats().bytes_pending == 0);
+  CHECK(FakeBackend::destroyed.count(1) && FakeBackend::destroyed.count(2));
+  // the reused block starts without recorded streams
+  CHECK(pool.free(e) == 0 && pool.stats().bytes_pending == 0);
+  CHECK(pool.free(c) == 0 && pool.free(d) == 0);
+
+  // a block freed while its stream is being captured is held until empty_cache
+  void *f = nullptr;
+  CHECK(pool.malloc(&f, 1000) == 0);
+  FakeBackend::capturing_stream = 5;
+  CHECK(pool.record_stream(f, 5) == 0);
+  CHECK(pool.free(f) == 0);
+  void *g = nullptr;
+  CHECK(pool.malloc(&g, 1000) == 0 && g != f);
+  CHECK(pool.stats().bytes_pending == 1024);
+  CHECK(pool.free(g) == 0);
+
+  // out of memory: pending and cached blocks are waited for, released, and the request retried
+  void *h = nullptr;
+  CHECK(pool.malloc(&h, 1 << 20) == 0);
+  CHECK(pool.record_stream(h, 3) == 0);
+  CHECK(pool.free(h) == 0);                       // pending on an event nobody completes
+  const int syncs = FakeBackend::syncs;
+  void *big = nullptr;
+  CHECK(pool.malloc(&big, size_t(60) << 20) == 0);  // only fits once everything else is released
+  CHECK(FakeBackend::syncs == syncs + 1);
+  CHECK(pool.stats().bytes_pending == 0 && pool.stats().bytes_cached == 0);
+  CHECK(FakeBackend::device.size() == 1);
+  CHECK(pool.malloc(&h, size_t(60) << 20) == FakeBackend::kOutOfMemory);
+  CHECK(pool.free(big) == 0);
+
+  CHECK(pool.empty_cache() == 0);
+  CHECK(FakeBackend::device.empty() && FakeBackend::budget == (size_t(64) << 20));
+  CHECK(pool.stats().bytes_in_use == 0);
+  std::printf("pool bookkeeping ok\n");
+  return 0;
+}

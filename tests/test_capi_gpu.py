@@ -950,3 +950,92 @@ def test_entry_points_capture_into_a_hip_graph(twg):
         hip.hipGraphDestroy(graph)
         hip.hipStreamDestroy(stream)
 
+
+
+def test_block_freed_while_a_caller_stream_still_uses_it(twg):
+    # Work queued on a stream of the caller's own; the output block of its first launch is
+    # recorded on that stream and freed at once, then a block of the same size is allocated and
+    # overwritten on the library's stream.  The allocator must keep the freed block aside until
+    # the caller's stream has passed the free (bytes_pending), so the second launch on that
+    # stream still reads the sum, bit for bit.
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = twg.load()
+    stream = ctypes.c_void_p()
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(stream), 1) == 0  # hipStreamNonBlocking
+    n = 1 << 24
+    g = torch.Generator().manual_seed(17)
+    a_h, b_h = torch.randn(n, generator=g), torch.randn(n, generator=g)
+    d_a, d_b = twg.to_device(a_h), twg.to_device(b_h)
+    d_res, d_busy = twg.DeviceBuffer(4 * n), twg.DeviceBuffer(4 * n)
+    it = twg.dense_iter(n)
+    twg.sync()
+    base = twg.mem_stats()
+    assert base["bytes_pending"] == 0
+    # keep the caller's stream busy for a few milliseconds first
+    for _ in range(40):
+        twg.check(L.twg_add_f32(d_busy.ptr, d_a.ptr, d_b.ptr, ctypes.c_float(1.0), ctypes.byref(it), stream))
+    d_sum = twg.DeviceBuffer(4 * n)
+    addr = d_sum.ptr
+    twg.check(L.twg_add_f32(d_sum.ptr, d_a.ptr, d_b.ptr, ctypes.c_float(1.0), ctypes.byref(it), stream))
+    twg.check(L.twg_unary_f32(twg.UNARY_GELU_ERF, d_res.ptr, d_sum.ptr, ctypes.byref(it), stream))
+    twg.check(L.twg_record_stream(ctypes.c_void_p(d_sum.ptr + 4096), stream))  # any address inside
+    d_sum.free()
+    assert twg.mem_stats()["bytes_pending"] == 4 * n
+    other = twg.DeviceBuffer(4 * n)   # same size class: must not be the block still in use
+    assert other.ptr != addr
+    twg.check(L.twg_fill_bytes(other.ptr, 0xAB, 4 * n, None))
+    assert hip.hipStreamSynchronize(stream) == 0
+    twg.sync()
+    # reference on the library's stream, into fresh buffers
+    d_s2, d_r2 = twg.DeviceBuffer(4 * n), twg.DeviceBuffer(4 * n)
+    assert twg.mem_stats()["bytes_pending"] == 0   # the caller's stream is done: reaped
+    twg.check(L.twg_add_f32(d_s2.ptr, d_a.ptr, d_b.ptr, ctypes.c_float(1.0), ctypes.byref(it), None))
+    twg.check(L.twg_unary_f32(twg.UNARY_GELU_ERF, d_r2.ptr, d_s2.ptr, ctypes.byref(it), None))
+    got, ref = d_res.download((n,), torch.float32), d_r2.download((n,), torch.float32)
+    assert bit_equal(got, ref)
+    assert bool((other.download((4 * n,), torch.uint8) == 0xAB).all())
+    # the library's own stream needs no record, and an unknown address is refused
+    assert L.twg_record_stream(ctypes.c_void_p(d_res.ptr), None) == 0
+    assert L.twg_record_stream(ctypes.c_void_p(12345), stream) == twg.E_INVALID_ARG
+    assert hip.hipStreamDestroy(stream) == 0
+
+
+def test_small_reads_from_several_threads(twg):
+    # each reader polls a mailbox of its own: 8 threads reading different scalars and counts
+    # at once must all get their own values
+    import threading
+    L = twg.load()
+    vals = torch.arange(64, dtype=torch.int64) * 1000 + 7
+    dev = twg.to_device(vals)
+    n = 50000
+    src = torch.arange(n, dtype=torch.float32)
+    d_src = twg.to_device(src)
+    errors = []
+
+    def reader(t):
+        try:
+            it = twg.dense_iter(n)
+            mask = (torch.arange(n) % (t + 2)) == 0
+            d_mask = twg.to_device(mask)
+            out = twg.DeviceBuffer(4 * n)
+            sb = L.twg_masked_select_scratch_bytes(n)
+            scr = twg.DeviceBuffer(sb)
+            for rep in range(50):
+                i = (t * 7 + rep) % 64
+                got = dev.download((1,), torch.int64, byte_offset=8 * i)
+                if int(got[0]) != int(vals[i]):
+                    errors.append(("scalar", t, rep, int(got[0])))
+                k = ctypes.c_int64(-1)
+                twg.check(L.twg_masked_select_count(out.ptr, ctypes.byref(k), d_src.ptr, 4, d_mask.ptr,
+                                                    ctypes.byref(it), scr.ptr, sb, None))
+                if k.value != int(mask.sum()):
+                    errors.append(("count", t, rep, k.value))
+        except Exception as exc:  # noqa: BLE001
+            errors.append(("exception", t, repr(exc)))
+
+    threads = [threading.Thread(target=reader, args=(t,)) for t in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors[:5]

@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "twg_internal.h"
+#include "twg_pool.h"
 
 namespace twg {
 namespace {
@@ -64,36 +65,44 @@ void do_init() {
 
 // ------------------------------------------------------------ allocator
 
-constexpr size_t kSmallGranule = 512;
-constexpr size_t kLargeGranule = size_t(2) << 20;
-constexpr size_t kLargeThreshold = size_t(1) << 20;
-
-size_t round_size(size_t n) {
-  if (n < kLargeThreshold) return (n + kSmallGranule - 1) / kSmallGranule * kSmallGranule;
-  return (n + kLargeGranule - 1) / kLargeGranule * kLargeGranule;
-}
-
-struct Pool {
-  std::mutex mu;
-  std::multimap<size_t, void *> free_blocks;     // rounded size -> block
-  std::unordered_map<void *, size_t> live;       // block -> rounded size
-  twg_mem_stats_t st{};
+// HIP side of the block pool (twg_pool.h holds the bookkeeping).
+struct HipPoolBackend {
+  using Stream = hipStream_t;
+  using Event = hipEvent_t;
+  static constexpr int kOutOfMemory = (int)hipErrorOutOfMemory;
+  static int alloc(void **p, size_t n) {
+    const hipError_t e = hipMalloc(p, n);
+    if (e != hipSuccess) (void)hipGetLastError();
+    return (int)e;
+  }
+  static int release(void *p) { return (int)hipFree(p); }
+  static bool record(hipStream_t s, hipEvent_t *e) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return false;  // a record would become a node of the graph, not a point in time
+    }
+    if (hipEventCreateWithFlags(e, hipEventDisableTiming) != hipSuccess) return false;
+    if (hipEventRecord(*e, s) != hipSuccess) {
+      (void)hipEventDestroy(*e);
+      return false;
+    }
+    return true;
+  }
+  static bool done(hipEvent_t e) {
+    const hipError_t r = hipEventQuery(e);
+    if (r != hipSuccess) (void)hipGetLastError();
+    return r == hipSuccess;
+  }
+  static void wait(hipEvent_t e) { (void)hipEventSynchronize(e); }
+  static void destroy(hipEvent_t e) { (void)hipEventDestroy(e); }
+  static void sync_library_stream() { (void)hipStreamSynchronize(rt().stream); }
 };
 
-Pool &pool() {
-  static Pool *p = new Pool;  // leaked on purpose: tensors may outlive static destructors
+BlockPool<HipPoolBackend> &pool() {
+  // leaked on purpose: tensors may outlive static destructors
+  static BlockPool<HipPoolBackend> *p = new BlockPool<HipPoolBackend>;
   return *p;
-}
-
-int release_cached_locked(Pool &p) {
-  int rc = 0;
-  for (auto &kv : p.free_blocks) {
-    hipError_t e = hipFree(kv.second);
-    if (e != hipSuccess) rc = (int)e;
-  }
-  p.free_blocks.clear();
-  p.st.bytes_cached = 0;
-  return rc;
 }
 
 // ------------------------------------------------------------ staging ring
@@ -102,7 +111,9 @@ constexpr int kStageSlots = 16;                    // events; a copy uses ring /
 constexpr size_t kStageRingBytes = size_t(64) << 20;
 constexpr size_t kStreamingDrainBytes = size_t(32) << 20;  // beyond what a last-level cache keeps
 constexpr size_t kHugePageHintBytes = size_t(8) << 20;      // D2H destinations from this size on
-constexpr size_t kMailboxBytes = 16384;                     // largest read served by the mailbox
+constexpr size_t kMailboxBytes = 16384;                     // largest read served by a mailbox
+constexpr int kMailboxSlots = 8;
+constexpr size_t kMailboxStride = kMailboxBytes + 64;       // payload, sequence word, padding
 constexpr size_t kFlowFlagBytes = 128 * sizeof(uint32_t);  // flags of a small download
 constexpr int kMailboxSpins = 200000;                      // then fall back to a stream sync
 
@@ -134,12 +145,18 @@ struct Staging {
   hipEvent_t ev[kStageSlots] = {};
   bool busy[kStageSlots] = {};  // an H2D DMA that reads the slot may still be in flight
   char *buf(int i) const { return base + (size_t)i * piece; }
-  // Mailbox for reads of a few bytes (a count, a scalar): coherent pinned memory a small
+  // Mailboxes for reads of a few bytes (a count, a scalar): coherent pinned memory a small
   // kernel writes and the host polls, which returns in ~3 us where waiting on the stream
-  // or on an event takes ~12 us.  [0, kMailboxBytes) payload, then the sequence word.
-  char *mailbox = nullptr;      // host address
+  // or on an event takes ~12 us.  Each is [0, kMailboxBytes) payload, then the sequence
+  // word.  A reader takes a mailbox under the lock and polls it with the lock released, so
+  // threads that wait for different kernels do not wait for each other.
+  char *mailbox = nullptr;      // host address of mailbox 0
   void *mailbox_dev = nullptr;  // the same memory as the device addresses it
-  uint32_t mailbox_seq = 0;
+  uint32_t mailbox_seq[kMailboxSlots] = {};
+  uint32_t mailbox_busy = 0;  // bit i: mailbox i is taken
+  std::condition_variable mailbox_cv;
+  char *box(int i) const { return mailbox + (size_t)i * kMailboxStride; }
+  char *box_dev(int i) const { return static_cast<char *>(mailbox_dev) + (size_t)i * kMailboxStride; }
   void *base_dev = nullptr;        // the ring as the device addresses it
   uint32_t *flow_flags = nullptr;  // coherent pinned: one word per 64 KiB piece of a small download
   void *flow_flags_dev = nullptr;
@@ -308,10 +325,10 @@ int staging_prepare_locked(Staging &s) {
   TWG_HIP_TRY(e);
   for (int i = 0; i < kStageSlots; ++i)
     TWG_HIP_TRY(hipEventCreateWithFlags(&s.ev[i], hipEventDisableTiming));
-  TWG_HIP_TRY(hipHostMalloc((void **)&s.mailbox, kMailboxBytes + 64,
+  TWG_HIP_TRY(hipHostMalloc((void **)&s.mailbox, kMailboxStride * kMailboxSlots,
                             hipHostMallocCoherent | hipHostMallocMapped));
   TWG_HIP_TRY(hipHostGetDevicePointer(&s.mailbox_dev, s.mailbox, 0));
-  std::memset(s.mailbox, 0, kMailboxBytes + 64);
+  std::memset(s.mailbox, 0, kMailboxStride * kMailboxSlots);
   TWG_HIP_TRY(hipHostGetDevicePointer(&s.base_dev, s.base, 0));
   TWG_HIP_TRY(hipHostMalloc((void **)&s.flow_flags, kFlowFlagBytes,
                             hipHostMallocCoherent | hipHostMallocMapped));
@@ -319,6 +336,22 @@ int staging_prepare_locked(Staging &s) {
   std::memset(s.flow_flags, 0, kFlowFlagBytes);
   s.ready = true;
   return 0;
+}
+
+// Take a free mailbox (waits for one if all are in use); call with the lock held.
+int mailbox_take(Staging &s, std::unique_lock<std::mutex> &lk) {
+  s.mailbox_cv.wait(lk, [&] { return s.mailbox_busy != (1u << kMailboxSlots) - 1u; });
+  int i = 0;
+  while (s.mailbox_busy & (1u << i)) ++i;
+  s.mailbox_busy |= 1u << i;
+  return i;
+}
+void mailbox_give_back(Staging &s, int i) {
+  {
+    std::lock_guard<std::mutex> lk(s.mu);
+    s.mailbox_busy &= ~(1u << i);
+  }
+  s.mailbox_cv.notify_one();
 }
 
 // Wait for every DMA that still reads a slot.
@@ -602,73 +635,34 @@ int twg_malloc(void **p, size_t n) {
   if (n == 0) return 0;
   int rc = ensure_init();
   if (rc) return rc;
-  const size_t want = round_size(n);
-  Pool &pl = pool();
-  std::lock_guard<std::mutex> lk(pl.mu);
-  pl.st.n_allocs++;
-  // Best fit: the smallest cached block that is large enough, as long as it
-  // wastes at most a quarter of itself (small blocks must match exactly).
-  auto it = pl.free_blocks.lower_bound(want);
-  if (it != pl.free_blocks.end()) {
-    size_t have = it->first;
-    bool ok = (have == want) || (want >= kLargeThreshold && have - want <= have / 4);
-    if (ok) {
-      *p = it->second;
-      pl.free_blocks.erase(it);
-      pl.live.emplace(*p, have);
-      pl.st.bytes_cached -= (int64_t)have;
-      pl.st.bytes_in_use += (int64_t)have;
-      pl.st.n_cache_hits++;
-      return 0;
-    }
-  }
-  void *d = nullptr;
-  hipError_t e = hipMalloc(&d, want);
-  if (e == hipErrorOutOfMemory) {
-    (void)hipGetLastError();
-    // Everything cached was freed by the caller; make sure queued work that
-    // still uses those blocks has drained before handing them to the driver.
-    (void)hipStreamSynchronize(rt().stream);
-    release_cached_locked(pl);
-    e = hipMalloc(&d, want);
-  }
-  if (e != hipSuccess) return (int)e;
-  pl.st.n_device_mallocs++;
-  pl.live.emplace(d, want);
-  pl.st.bytes_in_use += (int64_t)want;
-  *p = d;
-  return 0;
+  return pool().malloc(p, n);
 }
 
-int twg_free(void *p) {
-  if (!p) return 0;
-  Pool &pl = pool();
-  std::lock_guard<std::mutex> lk(pl.mu);
-  auto it = pl.live.find(p);
-  if (it == pl.live.end()) return TWG_E_INVALID_ARG;
-  size_t sz = it->second;
-  pl.live.erase(it);
-  pl.free_blocks.emplace(sz, p);
-  pl.st.bytes_in_use -= (int64_t)sz;
-  pl.st.bytes_cached += (int64_t)sz;
-  return 0;
+int twg_free(void *p) { return pool().free(p); }
+
+int twg_record_stream(const void *p, twg_stream_t stream) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  hipStream_t s = resolve_stream(stream);
+  if (s == rt().stream) return p ? 0 : TWG_E_INVALID_ARG;  // the owner: nothing to remember
+  return pool().record_stream(p, s);
 }
 
 int twg_empty_cache(void) {
   int rc = ensure_init();
   if (rc) return rc;
-  // Work queued before the matching twg_free calls may still touch the blocks.
-  TWG_HIP_TRY(hipStreamSynchronize(rt().stream));
-  Pool &pl = pool();
-  std::lock_guard<std::mutex> lk(pl.mu);
-  return release_cached_locked(pl);
+  return pool().empty_cache();
 }
 
 int twg_mem_stats(twg_mem_stats_t *out) {
   if (!out) return TWG_E_INVALID_ARG;
-  Pool &pl = pool();
-  std::lock_guard<std::mutex> lk(pl.mu);
-  *out = pl.st;
+  const PoolStats st = pool().stats();
+  out->bytes_in_use = st.bytes_in_use;
+  out->bytes_cached = st.bytes_cached;
+  out->n_device_mallocs = st.n_device_mallocs;
+  out->n_cache_hits = st.n_cache_hits;
+  out->n_allocs = st.n_allocs;
+  out->bytes_pending = st.bytes_pending;
   return 0;
 }
 
@@ -729,29 +723,35 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   if (rc) return rc;
   hipStream_t s = resolve_stream(stream);
   Staging &st = staging();
-  std::lock_guard<std::mutex> lk(st.mu);
-  if ((rc = staging_prepare_locked(st))) return rc;
-  if ((rc = staging_drain_locked(st))) return rc;  // uploads may still read the slots
   char *dst = static_cast<char *>(dst_host);
   const char *src = static_cast<const char *>(src_dev);
+  std::unique_lock<std::mutex> lk(st.mu);
+  if ((rc = staging_prepare_locked(st))) return rc;
   if (nbytes <= kMailboxBytes) {
-    const uint32_t seq = ++st.mailbox_seq;
-    mailbox_kernel<<<1, kMailboxLanes, 0, s>>>(reinterpret_cast<uint8_t *>(st.mailbox_dev),
+    // a mailbox of its own, polled with the lock released
+    const int mb = mailbox_take(st, lk);
+    const uint32_t seq = ++st.mailbox_seq[mb];
+    lk.unlock();
+    mailbox_kernel<<<1, kMailboxLanes, 0, s>>>(reinterpret_cast<uint8_t *>(st.box_dev(mb)),
                                     reinterpret_cast<const uint8_t *>(src), (uint32_t)nbytes, seq);
-    TWG_HIP_TRY(hipGetLastError());
-    const uint32_t *flag = reinterpret_cast<const uint32_t *>(st.mailbox + kMailboxBytes);
-    bool seen = false;
-    for (int i = 0; i < kMailboxSpins && !seen; ++i) {
-      seen = __atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq;
-      if (!seen) _mm_pause();
+    rc = (int)hipGetLastError();
+    if (rc == 0) {
+      const uint32_t *flag = reinterpret_cast<const uint32_t *>(st.box(mb) + kMailboxBytes);
+      bool seen = false;
+      for (int i = 0; i < kMailboxSpins && !seen; ++i) {
+        seen = __atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq;
+        if (!seen) _mm_pause();
+      }
+      if (!seen) {  // a long queue ahead of the kernel, or a failed launch: wait properly
+        rc = (int)hipStreamSynchronize(s);
+        if (rc == 0 && __atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) rc = (int)hipErrorUnknown;
+      }
+      if (rc == 0) std::memcpy(dst, st.box(mb), nbytes);
     }
-    if (!seen) {  // a long queue ahead of the kernel, or a failed launch: wait properly
-      TWG_HIP_TRY(hipStreamSynchronize(s));
-      if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) return (int)hipErrorUnknown;
-    }
-    std::memcpy(dst, st.mailbox, nbytes);
-    return 0;
+    mailbox_give_back(st, mb);
+    return rc;
   }
+  if ((rc = staging_drain_locked(st))) return rc;  // uploads may still read the ring's slots
   if (nbytes <= kFlowMaxBytes && nbytes <= st.ring_bytes) {
     const uint32_t seq = ++st.flow_seq;
     const uint32_t npieces = (uint32_t)((nbytes + kFlowPiece - 1) / kFlowPiece);
@@ -832,28 +832,31 @@ int twg_masked_select_count(void *out, int64_t *count_host, const void *src, int
   if (rc) return rc;
   hipStream_t s = resolve_stream(stream);
   Staging &st = staging();
-  std::lock_guard<std::mutex> lk(st.mu);
+  std::unique_lock<std::mutex> lk(st.mu);
   if ((rc = staging_prepare_locked(st))) return rc;
+  const int mb = mailbox_take(st, lk);
+  lk.unlock();
   // The first 8 bytes of the mailbox receive the count.  The sentinel is no valid
   // count; the kernel replaces it with one 8-byte store.
   constexpr int64_t kPending = INT64_MIN;
-  int64_t *slot = reinterpret_cast<int64_t *>(st.mailbox);
+  int64_t *slot = reinterpret_cast<int64_t *>(st.box(mb));
   __atomic_store_n(slot, kPending, __ATOMIC_RELEASE);
-  rc = masked_select_launch(out, static_cast<int64_t *>(st.mailbox_dev), src, elem_size, mask, it,
-                            scratch, scratch_bytes, stream);
-  if (rc) return rc;
+  rc = masked_select_launch(out, reinterpret_cast<int64_t *>(st.box_dev(mb)), src, elem_size, mask,
+                            it, scratch, scratch_bytes, stream);
   int64_t k = kPending;
-  if (it->numel != 0) {  // an empty input clears the count bytewise: wait for the stream instead
+  if (rc == 0 && it->numel != 0) {  // an empty input clears the count bytewise: wait for the stream
     for (int i = 0; i < kMailboxSpins && k == kPending; ++i) {
       k = __atomic_load_n(slot, __ATOMIC_ACQUIRE);
       if (k == kPending) _mm_pause();
     }
   }
-  if (k == kPending) {
-    TWG_HIP_TRY(hipStreamSynchronize(s));
+  if (rc == 0 && k == kPending) {
+    rc = (int)hipStreamSynchronize(s);
     k = __atomic_load_n(slot, __ATOMIC_ACQUIRE);
-    if (k == kPending) return (int)hipErrorUnknown;
+    if (rc == 0 && k == kPending) rc = (int)hipErrorUnknown;
   }
+  mailbox_give_back(st, mb);
+  if (rc) return rc;
   *count_host = k;
   return 0;
 }

@@ -55,4 +55,6 @@ def _install_repr():
 
 _install_repr()
 
-__all__ = ["webgpu"]
+from .compiler import webgpu_backend  # noqa: E402,F401  (python/torch_webgpu/__init__.py:15)
+
+__all__ = ["webgpu", "webgpu_backend"]

@@ -47,7 +47,8 @@ class Iter(ctypes.Structure):
 
 class MemStats(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in
-                ("bytes_in_use", "bytes_cached", "n_device_mallocs", "n_cache_hits", "n_allocs")]
+                ("bytes_in_use", "bytes_cached", "n_device_mallocs", "n_cache_hits", "n_allocs",
+                 "bytes_pending")]
 
 
 # Every symbol include/twg.h declares; tests check that the library exports them all.
@@ -56,7 +57,7 @@ SYMBOLS = [
     "twg_default_stream", "twg_stream_sync", "twg_device_sync",
     "twg_event_create", "twg_event_destroy", "twg_event_record", "twg_event_sync",
     "twg_event_elapsed_ms",
-    "twg_malloc", "twg_free", "twg_empty_cache", "twg_mem_stats",
+    "twg_malloc", "twg_free", "twg_record_stream", "twg_empty_cache", "twg_mem_stats",
     "twg_memcpy_h2d", "twg_memcpy_d2h", "twg_memcpy_d2d", "twg_fill_bytes",
     "twg_add_f32", "twg_add_scalar_f32", "twg_mul_f32", "twg_mul_scalar_f32",
     "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided", "twg_cast",
@@ -98,6 +99,7 @@ def load():
     L.twg_event_elapsed_ms.argtypes = [ctypes.POINTER(f32), vp, vp]
     L.twg_malloc.argtypes = [ctypes.POINTER(vp), sz]
     L.twg_free.argtypes = [vp]
+    L.twg_record_stream.argtypes = [vp, vp]
     L.twg_empty_cache.argtypes = []
     L.twg_mem_stats.argtypes = [ctypes.POINTER(MemStats)]
     L.twg_memcpy_h2d.argtypes = [vp, vp, sz, vp]
