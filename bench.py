@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--geometries", action="store_true",
                     help="instead of the benchmark: time add over families of broadcast and permuted "
                          "operands (~2^25 elements each) and print their spread as one JSON line")
+    ap.add_argument("--ablations", action="store_true",
+                    help="instead of the benchmark: time the launch shapes and kernel structures the hot "
+                         "kernels were chosen from (libtwg_ablate.so) and print them as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this op path is single-GPU (no collectives, nothing to shard in one "
@@ -71,6 +74,9 @@ def main():
     capi.init()
     if args.geometries:
         print(json.dumps(geometry_families(capi, L)), flush=True)
+        return
+    if args.ablations:
+        print(json.dumps(ablations(args.log2n)), flush=True)
         return
     dev_name, cus, mem = capi.device_info()
     log(f"device: {dev_name}  CUs={cus}  mem={mem / 2**30:.0f} GiB")
@@ -145,6 +151,12 @@ def main():
         return d
 
     f32 = ctypes.c_float
+
+    # Two transfers of known size that are none of the measured kernels: a 1 GiB device-to-device
+    # hipMemcpyAsync (the runtime's own blit kernel: 1 GiB read, 1 GiB written) and a 1 GiB fill
+    # (1 GiB written, nothing read).  A counter run of this script (rocprofv3 --pmc FETCH_SIZE /
+    # WRITE_SIZE) reads its scale factors off these two dispatches.
+    cal = calibration_transfers(capi, L)
 
     # ------------------------------------------------------------ headline inputs
     t0 = time.time()
@@ -282,8 +294,29 @@ def main():
         "dispatcher": disp,
         "ops": ops,
         "device": {"name": dev_name, "compute_units": cus},
+        "counter_calibration_transfers": cal,
     }
     print(json.dumps(out), flush=True)
+
+
+def calibration_transfers(capi, L):
+    gib = 1 << 30
+    a, b = capi.DeviceBuffer(gib), capi.DeviceBuffer(gib)
+    capi.check(L.twg_fill_bytes(a.ptr, 0x5A, gib, None))
+    capi.sync()
+    res = {}
+    for name, fn in (("hipMemcpyAsync_d2d_1GiB", lambda: capi.check(L.twg_memcpy_d2d(b.ptr, a.ptr, gib, None))),
+                     ("twg_fill_bytes_1GiB", lambda: capi.check(L.twg_fill_bytes(b.ptr, 0xA5, gib, None)))):
+        fn()
+        capi.sync()
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for _ in range(3):
+            fn()
+        e1.record()
+        capi.sync()
+        res[name] = {"ms": round(e0.elapsed_ms(e1) / 3, 4), "dispatches": 4}
+    return res
 
 
 def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, by_name,
@@ -338,6 +371,50 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
     del got
     line("masked_select_p0.50", lambda: torch.masked_select(src, m), W.masked_select_bytes(n, k50),
          c_abi("masked_select_p0.50", "op_ms_with_count_readback"))
+    return res
+
+
+def ablations(log2n):
+    """The experiments the kernel shapes rest on, from the ablation library (built by
+    `python torch-webgpu_amd/build.py ablate`; not part of the product): copies of 2^log2n floats
+    in every launch shape considered for the streaming kernels, and masked_select cut off phase
+    by phase and rebuilt in two other structures.  % of 8 TB/s on algorithmic bytes."""
+    path = os.path.join(ROOT, "torch-webgpu_amd", "torch_webgpu", "libtwg_ablate.so")
+    if not os.path.exists(path):
+        raise SystemExit(f"{path} is missing: build it with `python torch-webgpu_amd/build.py ablate`")
+    A = ctypes.CDLL(path)
+
+    class Result(ctypes.Structure):
+        _fields_ = [("name", ctypes.c_char * 96), ("ms", ctypes.c_float), ("bytes", ctypes.c_double),
+                    ("ok", ctypes.c_int32)]
+
+    cap = 64
+    buf = (Result * cap)()
+    A.twga_copy_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(Result), ctypes.c_int]
+    A.twga_masked_select.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.POINTER(Result), ctypes.c_int]
+
+    def rows(count, with_pct=True):
+        if count < 0:
+            raise RuntimeError(f"ablation library returned {count}")
+        out = []
+        for r in buf[:count]:
+            d = {"what": r.name.decode(), "ms": round(r.ms, 4),
+                 "verified": {1: True, 0: False}.get(r.ok)}
+            if with_pct:
+                d["pct_hbm_peak"] = round(r.bytes / r.ms / 1e6 / HBM_PEAK_GBS * 100, 1)
+            log(f"  {d['what']:84s} {d['ms']:8.4f} ms" + (f"  {d['pct_hbm_peak']:5.1f}%" if with_pct else "")
+                + ("" if d["verified"] is not False else "  OUTPUT DIFFERS"))
+            out.append(d)
+        return out
+
+    res = {"elements": 1 << log2n}
+    log(f"copy of 2^{log2n} floats (4 B read + 4 B written per element) by launch shape")
+    res["copy_shapes"] = rows(A.twga_copy_shapes(log2n, buf, cap))
+    res["masked_select"] = {}
+    for p in (0.5, 0.99, 0.01):
+        log(f"masked_select of 2^{log2n} floats, Bernoulli({p}) mask: ms of each form; % of peak on the "
+            "full op's algorithmic bytes (meaningful for the complete forms only)")
+        res["masked_select"][f"p{p}"] = rows(A.twga_masked_select(log2n, ctypes.c_float(p), buf, cap))
     return res
 
 

@@ -146,6 +146,13 @@ int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_strea
  * staging-buffer + MapAsync + WaitAny + memcpy sequence of cpu_copy_with_webgpu
  * (csrc/ops/copy.cpp:33-56). */
 int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_stream_t stream);
+/* Side effects of the two host copies worth knowing: destinations of 8 MiB and more get
+ * madvise(MADV_HUGEPAGE) on their 2 MiB-aligned interior (a freshly allocated destination
+ * otherwise faults 4 KiB at a time, 13 GB/s instead of 30-39; set TWG_NO_HUGEPAGE_HINT in
+ * the environment to leave the caller's mapping alone), and copies of 8 MiB and more are
+ * shared with three helper threads that the first such copy creates and that sleep
+ * otherwise.  A process forked after twg_init must not use the library (the helper threads
+ * and the locks do not come along). */
 /* Device -> device, contiguous.  Replaces CopyBufferToBuffer in copy_
  * (csrc/ops/copy.cpp:95-122).  Ranges must not overlap. */
 int twg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes, twg_stream_t stream);

@@ -1,0 +1,561 @@
+// Device side of masked_select: the compaction kernels and what they share (status words,
+// look-back, ballot offsets).  Included by twg_masked_select.hip, which launches them, and by
+// the benchmark's ablation library, which times cut-down and alternative forms of them.
+//
+// masked_select as a single-pass, order-preserving stream compaction.
+//
+// Replaces the boxed CPU fallback the reference registers for
+// aten::masked_select (csrc/bindings.cpp:42): two blocking device->host copies,
+// ATen's CPU kernel, one host->device copy.
+//
+// Shape of the algorithm (one kernel, mask and source each read once):
+//   * a tile is a contiguous run of elements owned by one workgroup; tiles are
+//     handed out in start order through one atomic ticket, so a tile only ever
+//     waits on tiles whose workgroups are already running (no deadlock whatever
+//     order the hardware starts workgroups in);
+//   * every lane turns 4 mask bytes into 4 selection bits; per-lane popcounts are
+//     reduced to wavefront totals, which meet in LDS;
+//   * the tile total is published at once as an AGGREGATE status word; wave 0
+//     then looks back over 256 predecessors per round (decoupled look-back) until
+//     it meets an INCLUSIVE word, and publishes its own inclusive prefix;
+//   * a source float4 is fetched from HBM only where the lane has a selection bit set;
+//     three 64-wide ballots of the lane counts plus mbcnt give each lane its offset, the
+//     values are compacted in LDS at the phase they will have in memory and written
+//     as aligned float4s.
+// A status word packs {flag:2, value:62} so one relaxed agent-scope 64-bit
+// load/store carries everything; no fences are needed because no other memory
+// is communicated between tiles.
+//
+// Three facts about MI355X shape the streaming variant (inputs from 2^21 elements).
+// Same-address agent-scope atomics retire at about one per 7 ns, so the ticket must not
+// be paid 32768 times for 2^28 elements: its tiles are 131072 elements (smaller for
+// smaller inputs, about one tile per CU).  A wavefront that mixes
+// loads and stores in a loop only keeps its loads in flight if the compiler can
+// count them, so its loads are unconditional (a lane with nothing selected reads
+// one shared dummy address).  And stores that leave partial 128-byte lines behind
+// cost HBM write efficiency, so each wavefront compacts through a small LDS ring
+// and writes whole aligned lines as soon as they are complete; only the first and
+// last line of a wavefront's run go out element by element.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "twg.h"
+
+namespace twg {
+namespace {
+
+constexpr int kSteps = 8;           // steps of 256 elements per wavefront (tile variants)
+constexpr int kWaveElems = 256 * kSteps;
+constexpr int kScalarWaves = 16;    // fallback variants: one element per lane,
+constexpr int kScalarSteps = 16;    //   16 wavefronts x 16 steps of 64 elements per tile
+constexpr int kScalarTile = 64 * kScalarWaves * kScalarSteps;
+constexpr int kMsMinTile = 256 * kSteps * 4;  // smallest tile of any variant (ms_compact_vec<4>)
+static_assert(kScalarTile >= kMsMinTile, "the scratch is sized for kMsMinTile-element tiles");
+constexpr size_t kMsHeaderBytes = 256;                  // tickets and carry, padded
+// Smallest tile of the streaming variant (8 wavefronts x 8 steps x 256 elements) and the
+// status words the scratch must hold: one per kMsMinTile elements for the small-tile
+// variants, or kStreamStatusStride per streaming tile plus the few tiles of its remainder
+// launch (less than one streaming tile, at most 16 small tiles).
+constexpr int64_t kStreamMinTile = 8 * 2048;
+constexpr size_t ms_scratch_bytes(int64_t numel) {
+  if (numel < 0) numel = 0;
+  const size_t small = (size_t)((numel + kMsMinTile - 1) / kMsMinTile);
+  const size_t big = (size_t)(numel / kStreamMinTile) * 4 + 16;  // 4 == kStreamStatusStride
+  return kMsHeaderBytes + sizeof(uint64_t) * (small > big ? small : big);
+}
+constexpr int kLookPerLane = 4;   // look-back window of the small-tile variants = 64 * 4 tiles
+// The streaming variant has few, large tiles: its wavefronts poll the status words of 64
+// predecessors per round instead of 256 and keep the words 32 bytes apart, so that the
+// store that publishes one tile's word does not contend with the polls of its neighbours'
+// words in the same 128-byte line (measured at 2^28 elements: +1.5 points at every density;
+// 16 or 64 bytes apart, or a 128-tile window, changed nothing more).
+constexpr int kStreamLookPerLane = 1;
+constexpr int kStreamStatusStride = 4;  // in 8-byte words (ms_scratch_bytes assumes 4)
+static_assert(kStreamStatusStride == 4, "ms_scratch_bytes sizes the scratch for a stride of 4");
+
+constexpr uint64_t kFlagShift = 62;
+constexpr uint64_t kFlagAggregate = 1ull << kFlagShift;
+constexpr uint64_t kFlagInclusive = 2ull << kFlagShift;
+constexpr uint64_t kValueMask = (1ull << kFlagShift) - 1;
+
+struct MsGeom {
+  int32_t ndim;
+  int64_t shape[TWG_MAX_DIMS];
+  int64_t sstride[TWG_MAX_DIMS];  // source
+  int64_t mstride[TWG_MAX_DIMS];  // mask
+};
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t lanes_below(uint64_t ballot) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(ballot >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((uint32_t)ballot, 0u));
+}
+
+__device__ __forceinline__ uint64_t status_load(const uint64_t *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void status_store(uint64_t *p, uint64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ int64_t wave_sum_i64(int64_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Four mask bytes -> four selection bits (bit j set if byte j is non-zero).
+__device__ __forceinline__ uint32_t select_bits(uint32_t w) {
+  const uint32_t high = (((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u;  // per byte: != 0
+  return (((high >> 7) * 0x01020408u) >> 24) & 0xFu;  // gather bits 0, 8, 16, 24
+}
+
+// From each lane's count c in 0..4: the lane's exclusive offset within the
+// wavefront and the wavefront total, by three ballots of the bits of c.
+__device__ __forceinline__ void wave_offsets(uint32_t c, uint32_t &below, uint32_t &total) {
+  const uint64_t b0 = __ballot(c & 1u), b1 = __ballot(c & 2u), b2 = __ballot(c & 4u);
+  below = lanes_below(b0) + 2u * lanes_below(b1) + 4u * lanes_below(b2);
+  total = (uint32_t)__popcll(b0) + 2u * (uint32_t)__popcll(b1) + 4u * (uint32_t)__popcll(b2);
+}
+
+// Exclusive prefix of tile `tile`: sum of the totals of all earlier tiles.  Run by
+// one full wavefront.  Each round inspects the 256 nearest unseen predecessors
+// (4 status words per lane, nearest first), waits until all of them have published
+// at least an aggregate, and stops at the nearest one that carries an inclusive
+// prefix.
+template <int LPL, int STRIDE>
+__device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t tile, int lane) {
+  int64_t exclusive = 0;
+  int64_t look = (int64_t)tile - 1 - lane;  // lane's nearest candidate
+  while (true) {
+    uint64_t st[LPL];
+    while (true) {
+      bool pending = false;
+#pragma unroll
+      for (int q = 0; q < LPL; ++q) {
+        const int64_t idx = look - 64 * q;
+        // slots before tile 0 behave like an inclusive prefix of 0
+        st[q] = (idx >= 0) ? status_load(status + idx * STRIDE) : kFlagInclusive;
+        pending |= (st[q] >> kFlagShift) == 0;
+      }
+      if (__ballot(pending) == 0) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    int64_t part = 0;
+    bool done = false;
+#pragma unroll
+    for (int q = 0; q < LPL; ++q) {
+      if (!done) {
+        const uint64_t incl = __ballot((st[q] >> kFlagShift) == 2);
+        const int64_t val = (int64_t)(st[q] & kValueMask);
+        if (incl) {
+          const int first = __builtin_ctzll(incl);  // nearest predecessor with a full prefix
+          part += (lane <= first) ? val : 0;
+          done = true;
+        } else {
+          part += val;
+        }
+      }
+    }
+    exclusive += wave_sum_i64(part);
+    if (done) return exclusive;
+    look -= 64 * LPL;
+  }
+}
+
+// Aggregate, look-back, inclusive prefix: the part every variant shares.  Call
+// with all threads; returns the tile's exclusive prefix to all of them.  s_slot is
+// one int64 of LDS.  The last tile also writes the grand total, plus *carry_in if a
+// previous launch compacted the elements before this one's.
+template <int LPL = kLookPerLane, int STRIDE = 1>
+__device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, uint32_t ntiles,
+                                               uint32_t tile_total, int64_t *d_count,
+                                               int64_t *s_slot, const int64_t *carry_in) {
+  const int lane = threadIdx.x & 63;
+  if (threadIdx.x < 64) {  // wave 0
+    uint64_t *mine = status + (size_t)tile * STRIDE;
+    if (lane == 0)
+      status_store(mine, (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
+    int64_t exclusive = 0;
+    if (tile != 0) {
+      exclusive = look_back<LPL, STRIDE>(status, tile, lane);
+      if (lane == 0) status_store(mine, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+    }
+    if (lane == 0) {
+      *s_slot = exclusive;
+      // One 8-byte store at system scope: the count may live in host memory that the
+      // host polls while the rest of the grid is still compacting.
+      if (tile == ntiles - 1)
+        __hip_atomic_store(d_count, exclusive + (int64_t)tile_total + (carry_in ? *carry_in : 0),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+  __syncthreads();
+  return *s_slot;
+}
+
+// ------------------------------------------------------------------ fast variants
+// Dense source and mask, 16-byte aligned source, 4-byte aligned mask.  Lane l of a
+// wavefront owns elements 4l..4l+3 of each 256-element step.
+
+// ---- streaming variant: full tiles only (the host launches it on a multiple of the
+// tile size, so it carries no bounds checks).  Wavefront w owns GROUPS * 8
+// consecutive steps of the tile.
+constexpr int kRingElems = 512;  // per wavefront; at most 31 + 256 values wait in it
+// Source steps in flight per wavefront.  4 measured best: 8 keeps more in flight than
+// the memory system rewards (dense masks lose 2-3%), and below ~64 VGPRs a second
+// 1024-lane workgroup becomes resident per CU, which costs dense masks 5-10%.
+constexpr int kDepth = 4;
+
+template <int WAVES, int GROUPS>
+struct MsStreamShared {
+  uint32_t tile;
+  uint32_t wave_total[WAVES];
+  int64_t base;
+  uint32_t bits[GROUPS][WAVES * 64];  // 4 selection bits per step, 8 steps per word
+  __attribute__((aligned(16))) float ring[WAVES][kRingElems];
+};
+
+// STAGES cuts the kernel short for timing experiments (the benchmark's ablation library
+// instantiates 1..4; the library itself only ever runs all 5): 1 = take the ticket, 2 = + mask
+// loads, selection bits and counts, 3 = + aggregate, look-back and the first source loads,
+// 4 = + every source load and the compaction in LDS, 5 = + the stores.
+template <int WAVES, int GROUPS, int STAGES = 5>
+__global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int64_t *d_count,
+                                                                const float *src,
+                                                                const uint8_t *mask,
+                                                                uint32_t ntiles, uint32_t *ticket,
+                                                                uint64_t *status) {
+  constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
+  constexpr int64_t kTileElems = (int64_t)kWaveSpan * WAVES;
+  __shared__ MsStreamShared<WAVES, GROUPS> sh;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0)
+    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const uint32_t tile = sh.tile;
+  if constexpr (STAGES < 2) return;
+  const int64_t start = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
+  const uint8_t *mask_w = mask + start + lane * 4;
+  const float *src_w = src + start + lane * 4;
+
+  // ---- 1. masks -> packed selection bits in LDS, wavefront totals
+  uint32_t cnt = 0;
+#pragma unroll 2
+  for (int g = 0; g < GROUPS; ++g) {
+    uint32_t w[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      w[k] = __builtin_nontemporal_load(
+          reinterpret_cast<const uint32_t *>(mask_w + (g * 8 + k) * 256));
+    uint32_t b = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) b |= select_bits(w[k]) << (4 * k);
+    sh.bits[g][threadIdx.x] = b;
+    cnt += __popc(b);
+  }
+  const uint32_t wt = wave_sum_u32(cnt);
+  if (lane == 0) sh.wave_total[wave] = wt;
+  __syncthreads();
+  uint32_t wbase = 0, tile_total = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const uint32_t t = sh.wave_total[w];
+    if ((uint32_t)w < wave) wbase += t;
+    tile_total += t;
+  }
+
+  if constexpr (STAGES < 3) {
+    if (tile_total == 0xFFFFFFFFu) *d_count = wbase;  // never true: keeps the counts alive
+    return;
+  }
+
+  // ---- 2. the first kDepth steps' values go in flight, then aggregate / look-back
+  const f32x4 *dummy = reinterpret_cast<const f32x4 *>(src + (int64_t)tile * kTileElems);
+  auto fetch = [&](uint32_t four_bits, int step) {
+    const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + step * 256);
+    return __builtin_nontemporal_load(four_bits ? p : dummy);
+  };
+  uint32_t b_cur = sh.bits[0][threadIdx.x];
+  f32x4 vals[kDepth];
+#pragma unroll
+  for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
+  const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(
+      status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
+  if constexpr (STAGES < 4) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kDepth; ++k) acc += vals[k][0];
+    if (acc == 1.2345e38f) out[base + wbase] = acc;  // practically never: keeps the loads alive
+    return;
+  }
+
+  // ---- 3. stream: compact a step into the ring, refill its register for kDepth steps
+  //         later, write out the lines the step completed.  Position p of this
+  //         wavefront's run is obase[p] in memory and ring[p % kRingElems] in LDS.
+  float *ring = sh.ring[wave];
+  float *wout = out + (base + wbase);
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 31u);
+  float *obase = wout - shift;         // 128-byte aligned
+  uint32_t run = shift;                // next free position
+  uint32_t flushed = shift ? 8u : 0u;  // float4 slots written; a shifted first line is not ours alone
+#pragma unroll 1
+  for (int g = 0; g < GROUPS; ++g) {
+    const int gn = (g + 1 < GROUPS) ? g + 1 : g;  // past the end: all lanes read the dummy
+    const uint32_t b_next = (g + 1 < GROUPS) ? sh.bits[gn][threadIdx.x] : 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t f = (b_cur >> (4 * k)) & 0xFu;
+      uint32_t below, total;
+      wave_offsets(__popc(f), below, total);
+      const f32x4 x4 = vals[k % kDepth];
+      {
+        const int ahead = k + kDepth;  // the step to prefetch, counted from this group's first
+        vals[k % kDepth] = ahead < 8 ? fetch((b_cur >> (4 * ahead)) & 0xFu, g * 8 + ahead)
+                                     : fetch((b_next >> (4 * (ahead - 8))) & 0xFu, gn * 8 + ahead - 8);
+      }
+      if (f) {
+        uint32_t pos = run + below;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (f & (1u << j)) {
+            const float x = x4[j];
+            ring[pos & (kRingElems - 1)] = x;
+            if constexpr (STAGES >= 5)
+              if (pos < 32u && shift) obase[pos] = x;  // shared first line: element by element
+            ++pos;
+          }
+        }
+      }
+      run += total;
+      const uint32_t end4 = (run >> 5) << 3;  // whole 128-byte lines only
+      if (end4 > flushed) {                   // wavefront-uniform
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t idx = flushed + lane; idx < end4; idx += 64) {
+          const f32x4 x =
+              *reinterpret_cast<const f32x4 *>(ring + ((4 * idx) & (kRingElems - 1)));
+          if constexpr (STAGES >= 5) {
+            __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * (size_t)idx));
+          } else if (x[0] == 1.2345e38f && x[3] == -1.2345e38f) {  // practically never
+            obase[4 * (size_t)idx] = x[1];
+          }
+        }
+        flushed = end4;
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+    b_cur = b_next;
+  }
+  // the last, incomplete line (its other elements belong to the next wavefront)
+  const uint32_t p = 4 * flushed + lane;
+  if constexpr (STAGES >= 5)
+    if (lane < 32 && p < run) obase[p] = ring[p & (kRingElems - 1)];
+}
+
+// ---- tile variant: any length.  One pass of 8 steps per wavefront, compacted in LDS at
+// the 16-byte phase the values will have in memory and written as aligned float4s.
+template <int WAVES>
+struct MsShared {
+  uint32_t tile;
+  uint32_t wave_total[WAVES];
+  int64_t base;
+  __attribute__((aligned(16))) float stage[WAVES][kWaveElems + 4];
+};
+
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t *d_count,
+                                                             const float *src,
+                                                             const uint8_t *mask, int64_t n,
+                                                             uint32_t ntiles, uint32_t *ticket,
+                                                             uint64_t *status,
+                                                             const int64_t *carry_in) {
+  constexpr int64_t kTileElems = (int64_t)kWaveElems * WAVES;
+  __shared__ MsShared<WAVES> sh;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  // A launch of a single tile needs no ticket (and no cleared scratch: nothing is looked back at).
+  if (threadIdx.x == 0)
+    sh.tile = ntiles == 1
+                  ? 0u
+                  : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const uint32_t tile = sh.tile;
+  // tile bases are wavefront-uniform; everything per lane is a 32-bit offset
+  const int64_t start = (int64_t)tile * kTileElems;
+  const uint8_t *mask_tile = mask + start;
+  const float *src_tile = src + start;
+  const uint32_t lane_off = wave * kWaveElems + lane * 4;
+  const int64_t left = n - start;
+  const uint32_t remaining = left < kTileElems ? (uint32_t)left : (uint32_t)kTileElems;
+  if (carry_in) out += *carry_in;
+
+  // ---- 1. mask -> packed selection bits (bit 4k+j <=> element j of step k) and totals
+  uint32_t w[kSteps];
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) {  // all 8 loads in flight before any is used
+    const uint32_t e = lane_off + k * 256;
+    if (e + 4 <= remaining) {
+      w[k] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(mask_tile + e));
+    } else {
+      w[k] = 0;
+      for (uint32_t j = 0; j < 4; ++j)
+        if (e + j < remaining && mask_tile[e + j]) w[k] |= 1u << (8 * j);
+    }
+  }
+  uint32_t bits = 0;
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) bits |= select_bits(w[k]) << (4 * k);
+  const uint32_t wt = wave_sum_u32(__popc(bits));
+  if (lane == 0) sh.wave_total[wave] = wt;
+  __syncthreads();
+  uint32_t wbase = 0, tile_total = 0;
+#pragma unroll
+  for (int v = 0; v < WAVES; ++v) {
+    const uint32_t t = sh.wave_total[v];
+    if ((uint32_t)v < wave) wbase += t;
+    tile_total += t;
+  }
+
+  // ---- 2. source values go in flight, then aggregate / look-back
+  f32x4 vals[kSteps];
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) {
+    if ((bits >> (4 * k)) & 0xFu) {
+      const uint32_t e = lane_off + k * 256;
+      if (e + 4 <= remaining) {
+        vals[k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src_tile + e));
+      } else {
+        for (uint32_t j = 0; j < 4; ++j) vals[k][j] = (e + j < remaining) ? src_tile[e + j] : 0.0f;
+      }
+    }
+  }
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, carry_in);
+
+  // ---- 3. compact in LDS, write aligned float4s; the ragged ends go out element by
+  //         element: their neighbours belong to other wavefronts.
+  float *stage = sh.stage[wave];
+  float *wout = out + (base + wbase);  // this wavefront's first output value
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 3u);
+  uint32_t run = shift;
+#pragma unroll
+  for (int k = 0; k < kSteps; ++k) {
+    const uint32_t f = (bits >> (4 * k)) & 0xFu;
+    uint32_t below, total;
+    wave_offsets(__popc(f), below, total);
+    if (f) {
+      uint32_t pos = run + below;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (f & (1u << j)) stage[pos++] = vals[k][j];
+      }
+    }
+    run += total;
+  }
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t span_end = shift + wt;
+  float *obase = wout - shift;  // 16-byte aligned
+  if (wt != 0) {
+    for (uint32_t v = lane; 4 * v < span_end; v += 64) {
+      const f32x4 x = *reinterpret_cast<const f32x4 *>(stage + 4 * v);
+      if (4 * v >= shift && 4 * v + 4 <= span_end) {
+        __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * v));
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t i = 4 * v + c;
+          if (i >= shift && i < span_end) obase[i] = x[c];
+        }
+      }
+    }
+  }
+}
+
+// -------------------------------------------------------------- fallback variants
+// One element per lane: misaligned pointers (STRIDED = false) or broadcast /
+// strided source and mask addressed through div/mod index math (STRIDED = true).
+// The values are moved as T without being looked at, so T is an unsigned integer of
+// the element's size.
+
+template <bool STRIDED, typename T>
+__global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
+    T *out, int64_t *d_count, const T *src, const uint8_t *mask, int64_t n,
+    uint32_t ntiles, uint32_t *ticket, uint64_t *status, MsGeom g) {
+  constexpr int kWaveSpan = 64 * kScalarSteps;
+  constexpr int kTileElems = kWaveSpan * kScalarWaves;
+
+  __shared__ uint32_t s_tile;
+  __shared__ uint32_t s_wave_total[kScalarWaves];
+  __shared__ int64_t s_base;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0)
+    s_tile = ntiles == 1
+                 ? 0u
+                 : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const uint32_t tile = s_tile;
+  const int64_t wstart = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
+
+  bool sel[kScalarSteps];
+  uint32_t loff[kScalarSteps];
+  int64_t soff[kScalarSteps];
+  uint32_t wtotal = 0;
+#pragma unroll
+  for (int k = 0; k < kScalarSteps; ++k) {
+    const int64_t e = wstart + k * 64 + lane;
+    bool f = false;
+    soff[k] = e;
+    if (e < n) {
+      if constexpr (STRIDED) {
+        int64_t rem = e, om = 0, os = 0;
+        for (int d = 0; d < g.ndim; ++d) {  // dimension 0 is the fastest-moving one
+          const int64_t q = rem / g.shape[d];
+          const int64_t c = rem - q * g.shape[d];
+          rem = q;
+          om += c * g.mstride[d];
+          os += c * g.sstride[d];
+        }
+        soff[k] = os;
+        f = mask[om] != 0;
+      } else {
+        f = mask[e] != 0;
+      }
+    }
+    const uint64_t b = __ballot(f);
+    loff[k] = wtotal + lanes_below(b);
+    wtotal += (uint32_t)__popcll(b);
+    sel[k] = f;
+  }
+  if (lane == 0) s_wave_total[wave] = wtotal;
+  __syncthreads();
+  uint32_t wave_base = 0, tile_total = 0;
+#pragma unroll
+  for (int w = 0; w < kScalarWaves; ++w) {
+    const uint32_t t = s_wave_total[w];
+    if (w < wave) wave_base += t;
+    tile_total += t;
+  }
+  T vals[kScalarSteps];
+#pragma unroll
+  for (int k = 0; k < kScalarSteps; ++k)
+    if (sel[k]) vals[k] = src[soff[k]];
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &s_base, nullptr);
+  const int64_t wpos = base + wave_base;
+#pragma unroll
+  for (int k = 0; k < kScalarSteps; ++k)
+    if (sel[k]) out[wpos + loff[k]] = vals[k];
+}
+
+}  // namespace
+}  // namespace twg

@@ -243,9 +243,17 @@ class CopyTeam {
   // Claim parts of job `id` until none is left or another job has begun.  The ticket holds
   // the job number next to the part counter, so a helper that arrives late for a finished
   // job claims nothing of the next one with the old description in hand.  Parts are split
-  // at multiples of 64 bytes: streaming stores of neighbouring parts must not share a line.
+  // at 64-byte lines of the destination: streaming stores of neighbouring parts must not
+  // share a line.
   void work(const CopyJob &j, uint32_t id) {
     const size_t per = ((j.n / kTeamParts) + 63) & ~size_t(63);
+    // part boundaries fall on 64-byte lines of the destination, whatever its alignment
+    const size_t head = (64 - (reinterpret_cast<uintptr_t>(j.dst) & 63)) & 63;
+    auto bound = [&](uint32_t k) {
+      if (k == 0) return size_t(0);
+      const size_t b = head + per * k;
+      return b < j.n ? b : j.n;
+    };
     for (;;) {
       uint64_t t = ticket_.load(std::memory_order_acquire);
       uint32_t part;
@@ -254,8 +262,8 @@ class CopyTeam {
         if ((uint32_t)(t >> 32) != id || part >= (uint32_t)kTeamParts) return;
       } while (!ticket_.compare_exchange_weak(t, t + 1, std::memory_order_acq_rel,
                                               std::memory_order_acquire));
-      const size_t lo = per * part < j.n ? per * part : j.n;
-      const size_t hi = (part == kTeamParts - 1) ? j.n : (lo + per < j.n ? lo + per : j.n);
+      const size_t lo = bound(part);
+      const size_t hi = (part == kTeamParts - 1) ? j.n : bound(part + 1);
       if (hi > lo) drain_slot(j.dst + lo, j.src + lo, hi - lo, j.streaming);
       done_.fetch_add(1, std::memory_order_release);
     }
@@ -801,7 +809,8 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
     const uintptr_t two_mib = uintptr_t(2) << 20;
     const uintptr_t lo = (reinterpret_cast<uintptr_t>(dst) + two_mib - 1) & ~(two_mib - 1);
     const uintptr_t hi = (reinterpret_cast<uintptr_t>(dst) + nbytes) & ~(two_mib - 1);
-    if (hi > lo) (void)madvise(reinterpret_cast<void *>(lo), hi - lo, MADV_HUGEPAGE);
+    static const bool hint = getenv("TWG_NO_HUGEPAGE_HINT") == nullptr;
+    if (hint && hi > lo) (void)madvise(reinterpret_cast<void *>(lo), hi - lo, MADV_HUGEPAGE);
   }
   // The DMA engine runs up to a ring (less one slot) ahead of the CPU draining the slots:
   // while chunk c is drained, the DMA that refills the slot drained before it is issued.
