@@ -147,6 +147,8 @@ def main():
             d.update(extra)
         on_traffic = (f"  ({d['pct_hbm_peak_on_traffic']:6.2f}% on measured traffic)"
                       if moved else "")
+        if "pct_hbm_peak_rotating_outputs" in d:
+            on_traffic += f"  ({d['pct_hbm_peak_rotating_outputs']:6.2f}% with rotating outputs)"
         log(f"  {name:28s} {d['avg_ms']:9.4f} ms  {d['GBps']:8.1f} GB/s  {d['pct_hbm_peak']:6.2f}% of peak{on_traffic}")
         return d
 
@@ -549,12 +551,41 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         d_p, d_q, d_z = capi.to_device(p_h), capi.to_device(q_h), capi.to_device(z_h)
         del p_h, q_h, z_h
         d_m1, d_m2, d_m3 = capi.DeviceBuffer(n), capi.DeviceBuffer(n), capi.DeviceBuffer(n)
-        ms = time_launches(lambda: capi.check(L.twg_eq_f32(d_m1.ptr, d_p.ptr, d_q.ptr, ctypes.byref(it), None)), Wm, K)
-        res.append(summarize("eq", "ew_contig<EqOp>", by["eq"] * n, ms, n))
-        ms = time_launches(lambda: capi.check(L.twg_ne_scalar_f32(d_m2.ptr, d_z.ptr, f32(0.0), ctypes.byref(it), None)), Wm, K)
-        res.append(summarize("ne_scalar", "ew_contig<NeScalarOp>", by["ne_scalar"] * n, ms, n))
-        ms = time_launches(lambda: capi.check(L.twg_and_u8(d_m3.ptr, d_m1.ptr, d_m2.ptr, ctypes.byref(it), None)), Wm, K)
-        res.append(summarize("bitwise_and", "ew_contig<AndOp>", by["bitwise_and"] * n, ms, n))
+        # A bool output of 2^28 elements is 256 MiB, the size of the last-level (Infinity)
+        # cache: launched again and again into the same buffer, the kernel writes lines that
+        # are still resident.  Each of these three is therefore also timed with its output
+        # rotating over three buffers (`pct_hbm_peak_rotating_outputs`), which is what a call
+        # whose result lands in memory not touched recently sees.
+        spare = [capi.DeviceBuffer(n), capi.DeviceBuffer(n)]
+
+        def rotating(call, first):
+            outs = [first] + spare
+            state = {"i": 0}
+
+            def fn():
+                o = outs[state["i"] % 3]
+                state["i"] += 1
+                call(o)
+            ms_r = time_launches(fn, Wm + 3, K)
+            return ms_r.batch_avg
+
+        def mask_line(name, kernel, nbytes, call, first):
+            ms = time_launches(lambda: call(first), Wm, K)
+            t_rot = rotating(call, first)
+            res.append(summarize(name, kernel, nbytes, ms, n, {
+                "avg_ms_rotating_outputs": round(t_rot, 5),
+                "pct_hbm_peak_rotating_outputs": round(nbytes / t_rot / 1e6 / HBM_PEAK_GBS * 100, 2)}))
+
+        mask_line("eq", "ew_contig<EqOp>", by["eq"] * n,
+                  lambda o: capi.check(L.twg_eq_f32(o.ptr, d_p.ptr, d_q.ptr, ctypes.byref(it), None)), d_m1)
+        mask_line("ne_scalar", "ew_contig<NeScalarOp>", by["ne_scalar"] * n,
+                  lambda o: capi.check(L.twg_ne_scalar_f32(o.ptr, d_z.ptr, f32(0.0), ctypes.byref(it), None)), d_m2)
+        # leave the masks of the parity configuration in d_m1 / d_m2 for bitwise_and
+        capi.check(L.twg_eq_f32(d_m1.ptr, d_p.ptr, d_q.ptr, ctypes.byref(it), None))
+        capi.check(L.twg_ne_scalar_f32(d_m2.ptr, d_z.ptr, f32(0.0), ctypes.byref(it), None))
+        mask_line("bitwise_and", "ew_contig<AndOp>", by["bitwise_and"] * n,
+                  lambda o: capi.check(L.twg_and_u8(o.ptr, d_m1.ptr, d_m2.ptr, ctypes.byref(it), None)), d_m3)
+        del spare
         # dtype conversion of a mask (mask.float()) and of fp32 data (x.half()): 5 and 6 B/element
         if want("cast_bool_f32"):
             ms = time_launches(lambda: capi.check(L.twg_cast(d_out.ptr, capi.DTYPES[torch.float32], d_m1.ptr,

@@ -104,6 +104,17 @@ int main() {
   CHECK(pool.free(e) == 0 && pool.stats().bytes_pending == 0);
   CHECK(pool.free(c) == 0 && pool.free(d) == 0);
 
+  // among cached blocks of one size the one freed last comes back first
+  {
+    void *x = nullptr, *y = nullptr, *z = nullptr;
+    CHECK(pool.malloc(&x, 5 << 20) == 0 && pool.malloc(&y, 5 << 20) == 0);
+    CHECK(pool.free(x) == 0 && pool.free(y) == 0);
+    CHECK(pool.malloc(&z, 5 << 20) == 0 && z == y);
+    CHECK(pool.free(z) == 0);
+    CHECK(pool.malloc(&z, 5 << 20) == 0 && z == y);   // and again: no alternation
+    CHECK(pool.free(z) == 0);
+  }
+
   // a block freed while its stream is being captured is held until empty_cache
   void *f = nullptr;
   CHECK(pool.malloc(&f, 1000) == 0);

@@ -125,7 +125,7 @@ __device__ __forceinline__ TO apply(const Op &op, TA a, TB b) {
 // elements (packs per lane x lanes):
 //   same width in and out (add, activations, and): 1 x 64 (add 83% of peak; 80% with
 //     2 x 64 or 1 x 256, 77% with 4 x 64);
-//   two float4 in, one dword of bools out (eq): 1 x 64 (89%; 84% with 2 x 64);
+//   two float4 in, one dword of bools out (eq): 1 x 64 (86.5%; 84% with 2 x 64);
 //   8 bytes out per lane (float32 -> half): 1 x 64 (87%; 84% with 2 x 64);
 //   one pack in, at most a dword out (ne.Scalar, float32 -> bool): 2 x 64 (90%; 88% with
 //     4 x 64, 80% with 1 x 1024; 1 x 64 moves too little per block, 73%: the grid then
@@ -171,10 +171,12 @@ __global__ __launch_bounds__(THREADS) void ew_contig(TO *out, const TA *a, const
 #pragma unroll
       for (int e = 0; e < VEC; ++e)
         r.v[e] = apply<NIN, Op, TO, TA, TB>(op, va[k].v[e], NIN == 2 ? vb[k].v[e] : TB());
-      // the nontemporal hint pays for stores of 8 and 16 bytes per lane (float32 -> half:
-      // 87% vs 84% of peak); one dword of bools per lane streams faster with a plain store
-      // (ne: 83% vs 79%)
-      store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+      // Streamed outputs are stored with the nontemporal hint whatever their width.  A plain
+      // store of one dword of bools per lane looks faster when the same 256 MiB output is
+      // written again and again, because the last-level cache (256 MB) still holds it (eq 89%
+      // of peak, ne 89%), and is slower when the output lands in memory not touched lately
+      // (82% / 81%); with the hint both cases run at 86.5% / 84.8%.
+      store_pack<STREAM>(reinterpret_cast<PO *>(out) + i, r);
     }
   }
   if constexpr (VEC > 1) {  // the last numel % VEC elements
@@ -241,7 +243,7 @@ __global__ __launch_bounds__(64) void ew_flat_bc(TO *out, const TA *a, const TB 
     PO r;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) r.v[k] = op(va.v[k], vb.v[k]);
-    store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+    store_pack<STREAM>(reinterpret_cast<PO *>(out) + i, r);
   } else if (e0 < numel) {  // the last numel % VEC elements (never with EXACT)
     for (uint32_t e = e0; e < numel; ++e) {
       const uint32_t row = e / len, col = e - row * len;
@@ -370,7 +372,7 @@ __global__ __launch_bounds__(64) void ew_flat_nd(TO *out, const TA *a, const TB 
     PO r;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) r.v[k] = op(va.v[k], vb.v[k]);
-    store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out) + i, r);
+    store_pack<STREAM>(reinterpret_cast<PO *>(out) + i, r);
   } else {  // the last numel % VEC elements
     for (uint32_t e = e0; e < g.numel; ++e) {
       const TS x = small[off];
