@@ -1501,7 +1501,9 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
         } else if (b_pair) {
           pd = pb; qd = qb;
         }
-        if (pd >= 1 && g.shape[pd] < 128 && g.shape[pd] * g.shape[qd] >= 32) {
+        // (an inner extent that is a multiple of 64 fills the tiles of (iii) by itself)
+        if (pd >= 1 && g.shape[pd] < 128 && g.shape[pd] % 64 != 0 &&
+            g.shape[pd] * g.shape[qd] >= 32) {
           int r = launch_tile<NIN, Op, TO, TA, TB>(out, a, b, g, qd, a_x, b_x, op, s, pd);
           if (r != TWG_E_UNSUPPORTED) return r;
         }
