@@ -565,3 +565,12 @@ def test_masked_select_out_is_validated():
     out = torch.empty(3, device="webgpu")
     torch.masked_select(src, m, out=out)
     assert bit_equal(out.to("cpu"), torch.masked_select(src_h, m_h))
+    # an out= with room for every element receives the values in place (no temporary, no copy)
+    big = torch.empty(6000, device="webgpu")
+    where = big.data_ptr()
+    torch.masked_select(src, m, out=big)
+    assert big.data_ptr() == where and big.shape == (int(m_h.sum()),)
+    assert bit_equal(big.to("cpu"), torch.masked_select(src_h, m_h))
+    none = torch.empty(10, device="webgpu")
+    torch.masked_select(src, dev(torch.zeros(5000, dtype=torch.bool)), out=none)
+    assert none.shape == (0,)

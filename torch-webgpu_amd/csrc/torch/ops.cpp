@@ -314,7 +314,10 @@ at::Tensor bitwise_and(const at::Tensor &self, const at::Tensor &other) {
 
 // -------------------------------------------------------------- masked_select
 
-at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
+// `into`: a dense device tensor of self's dtype with room for every element of the broadcast
+// shape, or undefined.  With it the selected values are compacted straight into its storage
+// and it is shrunk to the count; without it a result tensor is allocated.
+at::Tensor masked_select_impl(const at::Tensor &self, const at::Tensor &mask, at::Tensor into) {
   // Error text and semantics of ATen's CPU kernel, which is what the reference runs
   // (csrc/bindings.cpp:42).
   TORCH_CHECK(mask.scalar_type() == at::kBool, "masked_select: expected BoolTensor for mask");
@@ -329,7 +332,13 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   at::Tensor me = *std::get<0>(expanded);
   at::Tensor se = *std::get<1>(expanded);
   const int64_t n = se.numel();
-  if (n == 0) return at::empty({0}, self.options());
+  if (n == 0) {
+    if (into.defined()) {
+      into.resize_({0});
+      return into;
+    }
+    return at::empty({0}, self.options());
+  }
   // The compaction kernels stream dense operands 3-5x faster than they gather strided or
   // broadcast ones element by element (2^26 elements: 0.09 ms against 0.31-0.47 ms), and a
   // strided copy runs near the dense rate, so from 2^16 elements on anything that is not
@@ -343,7 +352,8 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   fill_iter_logical(se, me, &it);
   const size_t scratch_bytes = twg_masked_select_scratch_bytes(n);
   at::Tensor work = at::empty({(int64_t)scratch_bytes}, self.options().dtype(at::kByte));
-  at::Tensor out = at::empty({n}, self.options());
+  const bool direct = into.defined() && into.is_contiguous() && into.numel() >= n;
+  at::Tensor out = direct ? into : at::empty({n}, self.options());
   // The output shape depends on the data: waiting for the count is the op's one sync
   // point.  The kernel hands it over through pinned memory as soon as it is known.
   int64_t k = 0;
@@ -351,6 +361,10 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
                                     static_cast<const uint8_t *>(me.const_data_ptr()), &it,
                                     work.data_ptr(), scratch_bytes, nullptr));
   TORCH_CHECK(k >= 0 && k <= n, "webgpu masked_select: implausible count ", k);
+  if (direct) {
+    out.resize_({k});  // shrinking keeps the storage
+    return out;
+  }
   // Do not pin a source-sized block under a small result, unless the block is small
   // anyway (then the extra copy kernel would cost more than the memory is worth).
   if (k * 4 <= n && n * esize > (int64_t(1) << 20)) {
@@ -363,6 +377,10 @@ at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
   return out;
 }
 
+at::Tensor masked_select(const at::Tensor &self, const at::Tensor &mask) {
+  return masked_select_impl(self, mask, at::Tensor());
+}
+
 at::Tensor &masked_select_out(const at::Tensor &self, const at::Tensor &mask, at::Tensor &out) {
   // ATen's checks for the out= form (aten/src/ATen/native/TensorAdvancedIndexing.cpp,
   // masked_select_out_impl): same dtype, same device, no overlap with the inputs.
@@ -372,9 +390,12 @@ at::Tensor &masked_select_out(const at::Tensor &self, const at::Tensor &mask, at
   at::assert_no_internal_overlap(out);
   at::assert_no_overlap(out, self);
   at::assert_no_overlap(out, mask);
-  at::Tensor r = ops::masked_select(self, mask);
-  out.resize_(r.sizes());
-  out.copy_(r);
+  // an out= tensor with room for the whole broadcast shape receives the values directly
+  at::Tensor r = masked_select_impl(self, mask, out);
+  if (!r.is_same(out)) {
+    out.resize_(r.sizes());
+    out.copy_(r);
+  }
   return out;
 }
 
