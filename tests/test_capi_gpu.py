@@ -808,6 +808,13 @@ def test_masked_select_streaming_edge_patterns(twg):
             "around tile edges": ((idx + 2) % 16384) < 4,
             "second half": idx >= n // 2,
             "one wavefront's span": (idx >= 70000) & (idx < 70000 + 2048),
+            # around the density (1 in 16 per wavefront) below which a wavefront gathers
+            # its elements one by one instead of streaming
+            "every 16th": idx % 16 == 5,
+            "every 16th and one more": (idx % 16 == 5) | (idx % 2048 == 0),
+            "128 in a row per 8192": (idx % 8192 >= 384) & (idx < 512 + idx // 8192 * 8192),
+            "3 percent": W.bernoulli_mask(n, 0.03, seed=21),
+            "6 percent": W.bernoulli_mask(n, 0.06, seed=22),
         }
         for name, m in patterns.items():
             ref = torch.masked_select(x, m)
