@@ -367,6 +367,212 @@ __global__ __launch_bounds__(WAVES * 64) void small_tiles_known_bases(float *out
   }
 }
 
+// One-shot workgroups like the streaming kernel's, but SWAVES wavefronts stream and one more,
+// the last, owns no elements: it publishes the tile's aggregate, looks back and hands the
+// tile's base to the others through LDS.  The streaming wavefronts do not wait for it:
+// they compact into their rings at ring-local positions and only need the base once a
+// ring is full (or at the end), so the look-back of a tile overlaps its own streaming.
+// Until then nothing is written to memory; the position of a value in memory (and with it
+// the 128-byte line phase of the flushes) is applied when the ring is read back.
+// WAIT_FIRST: the streaming wavefronts wait for the base before their first step instead
+// (what the layout alone costs).
+constexpr int kAheadRing = 2048;  // floats per streaming wavefront
+
+template <int SWAVES, int GROUPS>
+struct MsAheadShared {
+  uint32_t tile;
+  uint32_t base_ready;
+  uint32_t wave_total[SWAVES];
+  int64_t base;
+  uint32_t bits[GROUPS][SWAVES * 64];
+  __attribute__((aligned(16))) float ring[SWAVES][kAheadRing];
+};
+
+template <int SWAVES, int GROUPS, bool WAIT_FIRST>
+__global__ __launch_bounds__((SWAVES + 1) * 64) void one_shot_run_ahead(float *out, int64_t *d_count,
+                                                                      const float *src,
+                                                                      const uint8_t *mask,
+                                                                      uint32_t ntiles,
+                                                                      uint32_t *ticket,
+                                                                      uint64_t *status) {
+  constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
+  constexpr int64_t kTileElems = (int64_t)kWaveSpan * SWAVES;
+  constexpr uint32_t kMask = kAheadRing - 1;
+  __shared__ MsAheadShared<SWAVES, GROUPS> sh;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) {
+    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh.base_ready = 0u;
+  }
+  __syncthreads();
+  const uint32_t tile = sh.tile;
+  const bool front = wave == SWAVES;  // wavefront-uniform
+  const uint32_t swave = front ? 0u : wave;
+  const int64_t start = (int64_t)tile * kTileElems + (int64_t)swave * kWaveSpan;
+  const uint8_t *mask_w = mask + start + lane * 4;
+  const float *src_w = src + start + lane * 4;
+
+  // ---- 1. masks -> packed selection bits in LDS, wavefront totals
+  uint32_t wt = 0;
+  if (!front) {
+    uint32_t cnt = 0;
+#pragma unroll 2
+    for (int g = 0; g < GROUPS; ++g) {
+      uint32_t w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        w[k] = __builtin_nontemporal_load(
+            reinterpret_cast<const uint32_t *>(mask_w + (g * 8 + k) * 256));
+      uint32_t b = 0;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) b |= select_bits(w[k]) << (4 * k);
+      sh.bits[g][threadIdx.x] = b;
+      cnt += __popc(b);
+    }
+    wt = wave_sum_u32(cnt);
+    if (lane == 0) sh.wave_total[wave] = wt;
+  }
+  __syncthreads();
+  uint32_t wbase = 0, tile_total = 0;
+#pragma unroll
+  for (int w = 0; w < SWAVES; ++w) {
+    const uint32_t t = sh.wave_total[w];
+    if ((uint32_t)w < wave) wbase += t;
+    tile_total += t;
+  }
+
+  // ---- 2. the front wavefront: aggregate, look-back, inclusive prefix, base into LDS
+  if (front) {
+    uint64_t *mine = status + (size_t)tile * kStreamStatusStride;
+    if (lane == 0)
+      status_store(mine, (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
+    int64_t exclusive = 0;
+    if (tile != 0) {
+      exclusive = look_back<kStreamLookPerLane, kStreamStatusStride>(status, tile, (int)lane);
+      if (lane == 0) status_store(mine, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+    }
+    if (lane == 0) {
+      if (tile == ntiles - 1)
+        __hip_atomic_store(d_count, exclusive + (int64_t)tile_total, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+      sh.base = exclusive;
+      __hip_atomic_store(&sh.base_ready, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    return;
+  }
+  if (wt == 0) return;
+
+  auto base_is_ready = [&]() {
+    return __hip_atomic_load(&sh.base_ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != 0u;
+  };
+  auto wait_for_base = [&]() {
+    while (!base_is_ready()) __builtin_amdgcn_s_sleep(1);
+  };
+
+  // ---- 3. streaming
+  const f32x4 *dummy = reinterpret_cast<const f32x4 *>(src + (int64_t)tile * kTileElems);
+  auto fetch = [&](uint32_t four_bits, int step) {
+    const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + step * 256);
+    return __builtin_nontemporal_load(four_bits ? p : dummy);
+  };
+  uint32_t b_cur = sh.bits[0][threadIdx.x];
+  f32x4 vals[kDepth];
+#pragma unroll
+  for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
+
+  float *ring = sh.ring[wave];
+  bool have = false;
+  uint32_t shift = 0;    // elements of the wavefront's first 128-byte line that belong to others
+  float *obase = out;    // 128-byte aligned; memory position q = shift + ring-local position
+  uint32_t flushed = 0;  // float4 slots of obase written
+  uint32_t run = 0;      // ring-local: elements compacted so far
+  auto adopt = [&]() {
+    float *wout = out + (sh.base + (int64_t)wbase);
+    shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 31u);
+    obase = wout - shift;
+    if (shift) {  // a shared first line goes out element by element
+      const uint32_t head = run < 32u - shift ? run : 32u - shift;
+      __builtin_amdgcn_wave_barrier();
+      if (lane < head) obase[shift + lane] = ring[lane];
+      flushed = 8u;
+    }
+    have = true;
+  };
+  auto flush_lines = [&]() {
+    const uint32_t end4 = ((shift + run) >> 5) << 3;  // whole 128-byte lines only
+    if (end4 > flushed) {                             // wavefront-uniform
+      __builtin_amdgcn_wave_barrier();
+      for (uint32_t idx = flushed + lane; idx < end4; idx += 64) {
+        const uint32_t l = 4u * idx - shift;  // ring-local position of the slot's first element
+        f32x4 x;
+        x[0] = ring[l & kMask];
+        x[1] = ring[(l + 1u) & kMask];
+        x[2] = ring[(l + 2u) & kMask];
+        x[3] = ring[(l + 3u) & kMask];
+        __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * (size_t)idx));
+      }
+      flushed = end4;
+      __builtin_amdgcn_wave_barrier();
+    }
+  };
+  if constexpr (WAIT_FIRST) {
+    wait_for_base();
+    adopt();
+  }
+#pragma unroll 1
+  for (int g = 0; g < GROUPS; ++g) {
+    const int gn = (g + 1 < GROUPS) ? g + 1 : g;  // past the end: all lanes read the dummy
+    const uint32_t b_next = (g + 1 < GROUPS) ? sh.bits[gn][threadIdx.x] : 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t f = (b_cur >> (4 * k)) & 0xFu;
+      uint32_t below, total;
+      wave_offsets(__popc(f), below, total);
+      const f32x4 x4 = vals[k % kDepth];
+      {
+        const int ahead = k + kDepth;  // the step to prefetch, counted from this group's first
+        vals[k % kDepth] = ahead < 8 ? fetch((b_cur >> (4 * ahead)) & 0xFu, g * 8 + ahead)
+                                     : fetch((b_next >> (4 * (ahead - 8))) & 0xFu, gn * 8 + ahead - 8);
+      }
+      if (!have) {  // wavefront-uniform
+        bool ready = base_is_ready();
+        if (!ready && run + total > (uint32_t)kAheadRing) {  // no room to run further ahead
+          wait_for_base();
+          ready = true;
+        }
+        if (ready) {
+          adopt();
+          flush_lines();
+        }
+      }
+      if (f) {
+        uint32_t pos = run + below;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (f & (1u << j)) {
+            const float x = x4[j];
+            ring[pos & kMask] = x;
+            if (have && shift && pos + shift < 32u) obase[pos + shift] = x;
+            ++pos;
+          }
+        }
+      }
+      run += total;
+      if (have) flush_lines();
+    }
+    b_cur = b_next;
+  }
+  if (!have) {
+    wait_for_base();
+    adopt();
+    flush_lines();
+  }
+  // the last, incomplete line (its other elements belong to the next wavefront)
+  const uint32_t p = 4 * flushed + lane;
+  if (lane < 32 && p >= shift && p < shift + run) obase[p] = ring[(p - shift) & kMask];
+}
+
 // Persistent workgroups: S stream wavefronts compact tile i while one front wavefront takes the
 // ticket of tile i + 1, turns its masks into selection nibbles in the other LDS buffer,
 // publishes the aggregate, looks back and leaves the base.  The hand-over goes through LDS
@@ -668,6 +874,63 @@ struct SelectStudy {
     return 0;
   }
 
+  template <int S, bool WAIT_FIRST>
+  int run_ahead() {
+    constexpr int64_t kTile = 256 * 8 * 4 * S;
+    const int64_t nb = n / kTile;  // whole tiles only: compared on the prefix they cover
+    const int64_t covered = nb * kTile;
+    if (nb < 1) return 0;
+    uint32_t *ticket = static_cast<uint32_t *>(scratch);
+    uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+    const size_t clear = kMsHeaderBytes + 8 * (size_t)nb * kStreamStatusStride;
+    if (clear > scratch_bytes) return -1;
+    TWGA_TRY(hipMemsetAsync(out, 0, (size_t)n * 4, tm.s));
+    float ms = 0;
+    int rc = tm.run([&] {
+      (void)hipMemsetAsync(scratch, 0, clear, tm.s);
+      one_shot_run_ahead<S, 4, WAIT_FIRST><<<(unsigned)nb, (S + 1) * 64, 0, tm.s>>>(
+          out, cnt, src, mask, (uint32_t)nb, ticket, status);
+    }, &ms);
+    if (rc) return rc;
+    int64_t k = -1;
+    TWGA_TRY(hipMemcpyAsync(&k, cnt, 8, hipMemcpyDeviceToHost, tm.s));
+    TWGA_TRY(hipStreamSynchronize(tm.s));
+    int ok = 0;
+    if ((rc = check_prefix(covered, k, &ok))) return rc;
+    char name[112];
+    std::snprintf(name, sizeof(name),
+                  WAIT_FIRST ? "one-shot: %d stream wavefronts wait for 1 front wavefront's base"
+                             : "one-shot: %d stream wavefronts run ahead of 1 front wavefront's look-back",
+                  S);
+    put(res, name, ms, bytes_of(covered, k), ok);
+    return 0;
+  }
+
+  // Is out[0..k) the compaction of the first `covered` elements?  Compared with the streaming
+  // kernel's output over the whole input, whose first outputs are exactly that.
+  int check_prefix(int64_t covered, int64_t k, int *ok) {
+    uint32_t *ticket = static_cast<uint32_t *>(scratch);
+    uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+    const int64_t pieces = covered / 1024;
+    tile_counts<<<(unsigned)pieces, 256, 0, tm.s>>>(mask, 1024, counts);
+    std::vector<uint32_t> c((size_t)pieces);
+    TWGA_TRY(hipMemcpyAsync(c.data(), counts, 4 * (size_t)pieces, hipMemcpyDeviceToHost, tm.s));
+    TWGA_TRY(hipStreamSynchronize(tm.s));
+    int64_t want = 0;
+    for (uint32_t x : c) want += x;
+    unsigned long long h = 0, href = 0;
+    int rc = checksum(k, &h);
+    if (rc) return rc;
+    constexpr int64_t kFull = 256 * 8 * 4 * 16;
+    const int64_t nbf = n / kFull;
+    (void)hipMemsetAsync(scratch, 0, kMsHeaderBytes + 8 * (size_t)nbf * kStreamStatusStride, tm.s);
+    ms_compact_stream<16, 4, 5><<<(unsigned)nbf, 1024, 0, tm.s>>>(out, cnt, src, mask, (uint32_t)nbf, ticket,
+                                                                 status);
+    if ((rc = checksum(want, &href))) return rc;
+    *ok = (k == want && h == href) ? 1 : 0;
+    return 0;
+  }
+
   template <int S, int DEPTH, int RB>
   int front_wave() {
     constexpr int64_t kTile = 256 * 8 * 4 * S;
@@ -824,6 +1087,8 @@ int twga_masked_select(int log2n, float p, twga_result_t *out, int cap) {
   TWGA_STEP((st.small_tiles<4, 8>()));
   TWGA_STEP((st.small_tiles<4, 2>()));
   TWGA_STEP((st.small_tiles<16, 4>()));
+  TWGA_STEP((st.run_ahead<15, true>()));
+  TWGA_STEP((st.run_ahead<15, false>()));
   TWGA_STEP((st.front_wave<15, 4, 3>()));
   TWGA_STEP((st.front_wave<12, 4, 3>()));
 done:
