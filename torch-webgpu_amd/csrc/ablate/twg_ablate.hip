@@ -113,6 +113,22 @@ __global__ __launch_bounds__(WAVES * 64) void copy_tiles(float *__restrict__ out
     __builtin_nontemporal_store(v[k], reinterpret_cast<f32x4 *>(out + base + (int64_t)(s + k) * stride));
 }
 
+// One-shot single-wavefront blocks of 1 KiB, as in the fastest shape, but consecutive blocks
+// (which run at the same time) are dealt round-robin to `regions` equal parts of the array:
+// block b copies KiB number (b % regions) * (blocks / regions) + b / regions.  Every part is
+// still walked front to back over the launch; only the set of addresses in flight at one
+// moment changes, from one window of a few MiB to `regions` windows of a few KiB.
+__global__ __launch_bounds__(64) void copy_oneshot_regions(float *__restrict__ out,
+                                                           const float *__restrict__ src,
+                                                           uint32_t regions, uint32_t per_region) {
+  const uint32_t b = blockIdx.x;
+  // blocks past regions * per_region (when the count does not divide) keep their own KiB
+  const int64_t kib = b / regions < per_region ? (int64_t)(b % regions) * per_region + b / regions : (int64_t)b;
+  const int64_t at = kib * 256 + threadIdx.x * 4;
+  const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src + at));
+  __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(out + at));
+}
+
 // Persistent grid-stride loop: gridDim.x blocks, each round covers gridDim.x * WAVES KiB.
 template <int WAVES, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void copy_grid_stride(float *__restrict__ out,
@@ -224,6 +240,22 @@ struct CopyStudy {
     char name[96];
     std::snprintf(name, sizeof(name), "%s: %d wavefronts x %d KiB each, %d loads in flight", what, WAVES,
                   steps, DEPTH);
+    put(res, name, ms, 8.0 * (double)n, ok);
+    return 0;
+  }
+  int regions(uint32_t r) {
+    const int64_t blocks = n / 256;
+    if (blocks * 256 != n || blocks > 0x7FFFFFFF) return 0;
+    TWGA_TRY(hipMemsetAsync(out, 0, (size_t)n * 4, tm.s));
+    float ms = 0;
+    int rc = tm.run([&] {
+      copy_oneshot_regions<<<(unsigned)blocks, 64, 0, tm.s>>>(out, src, r, (uint32_t)(blocks / r));
+    }, &ms);
+    if (rc) return rc;
+    int ok = 0;
+    if ((rc = verify(&ok))) return rc;
+    char name[96];
+    std::snprintf(name, sizeof(name), "one-shot: 1 wavefront x 1 KiB, blocks dealt round-robin to %u regions", r);
     put(res, name, ms, 8.0 * (double)n, ok);
     return 0;
   }
@@ -1024,6 +1056,13 @@ int twga_copy_shapes(int log2n, twga_result_t *out, int cap) {
   } while (0)
   // one-shot blocks
   TWGA_STEP((st.tiles<1, 1, true>("one-shot", 256)));
+  TWGA_STEP(st.regions(16));
+  TWGA_STEP(st.regions(15));
+  TWGA_STEP(st.regions(256));
+  TWGA_STEP(st.regions(255));
+  TWGA_STEP(st.regions(4096));
+  TWGA_STEP(st.regions(4095));
+  TWGA_STEP(st.regions(65536));
   TWGA_STEP((st.tiles<1, 2, true>("one-shot", 512)));
   TWGA_STEP((st.tiles<1, 4, true>("one-shot", 1024)));
   TWGA_STEP((st.tiles<4, 1, true>("one-shot", 1024)));
