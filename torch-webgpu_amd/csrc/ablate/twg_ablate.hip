@@ -399,6 +399,185 @@ __global__ __launch_bounds__(WAVES * 64) void small_tiles_known_bases(float *out
   }
 }
 
+// Counters ahead of movers, in one launch of 256-lane one-shot blocks.  A counter block reads
+// the masks of 16 consecutive 2048-element chunks, chains its total to the earlier counter
+// blocks by decoupled look-back and publishes the 16 chunks' output offsets; a mover block is
+// small_tiles_known_bases<4, 2> for one chunk, taking its offset from that table.  Counter
+// block t sits LEAD blocks-of-17 before the movers of its chunks, so an offset is normally
+// there long before its mover starts, and the movers walk masks, source and output as one
+// narrow front.  The masks are read twice, the second time by another CU: whether that read
+// is served by a cache decides what this form costs.  Block index stands for start order
+// here; every wait is bounded (on overrun *err is set and the block carries on with what it has).
+constexpr int kAheadSpinCap = 1 << 14;
+constexpr int kChunksPerCounter = 16;
+
+__device__ __forceinline__ int64_t look_back_bounded(const uint64_t *status, uint32_t tile, int lane,
+                                                     uint32_t *err) {
+  int64_t exclusive = 0;
+  int64_t look = (int64_t)tile - 1 - lane;
+  while (true) {
+    uint64_t st = 0;
+    int spins = 0;
+    while (true) {
+      st = look >= 0 ? status_load(status + look) : kFlagInclusive;
+      if (__ballot((st >> kFlagShift) == 0) == 0) break;
+      if (++spins > kAheadSpinCap) {
+        if (lane == 0) *err = 1u;
+        return exclusive;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    const uint64_t incl = __ballot((st >> kFlagShift) == 2);
+    const int64_t val = (int64_t)(st & kValueMask);
+    if (incl) {
+      const int first = __builtin_ctzll(incl);
+      return exclusive + wave_sum_i64(lane <= first ? val : 0);
+    }
+    exclusive += wave_sum_i64(val);
+    look -= 64;
+  }
+}
+
+struct AheadShared {
+  uint32_t wave_total[4];
+  uint32_t chunk_count[kChunksPerCounter];
+  int64_t base;
+  __attribute__((aligned(16))) float stage[4][256 * 2 + 4];
+};
+
+template <int LEAD>
+__global__ __launch_bounds__(256) void counters_ahead_of_movers(float *out, int64_t *d_count,
+                                                                const float *src,
+                                                                const uint8_t *mask, uint32_t nchunks,
+                                                                uint64_t *status, uint64_t *offsets,
+                                                                uint32_t *err) {
+  constexpr int kPer = kChunksPerCounter + 1;
+  __shared__ AheadShared sh;
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t ncounters = nchunks / kChunksPerCounter;
+  const uint32_t b = blockIdx.x;
+  bool counter;
+  uint32_t index;
+  if (b < (uint32_t)LEAD) {
+    counter = true;
+    index = b;
+  } else {
+    const uint32_t q = b - LEAD, g = q / kPer, r = q % kPer;
+    counter = r == 0;
+    index = counter ? g + LEAD : g * kChunksPerCounter + (r - 1);
+  }
+  if (counter) {
+    if (index >= ncounters) return;
+    // wavefront w counts chunks 4w .. 4w+3 of the block's 16: 8 steps of 256 masks each
+    const uint8_t *m = mask + (int64_t)index * (kChunksPerCounter * 2048) + wave * 8192 + lane * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      uint32_t w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) w[k] = *reinterpret_cast<const uint32_t *>(m + c * 2048 + k * 256);
+      uint32_t cnt = 0;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) cnt += __popc(select_bits(w[k]));
+      cnt = wave_sum_u32(cnt);
+      if (lane == 0) sh.chunk_count[wave * 4 + c] = cnt;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const uint32_t mine = lane < (uint32_t)kChunksPerCounter ? sh.chunk_count[lane] : 0u;
+    uint32_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < kChunksPerCounter; d *= 2) {
+      const uint32_t t = __shfl_up(incl, d);
+      if (lane >= (uint32_t)d) incl += t;
+    }
+    const uint32_t total = __shfl(incl, kChunksPerCounter - 1);
+    if (lane == 0)
+      status_store(status + index, (index == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)total);
+    int64_t exclusive = 0;
+    if (index != 0) {
+      exclusive = look_back_bounded(status, index, (int)lane, err);
+      if (lane == 0) status_store(status + index, kFlagInclusive | (uint64_t)(exclusive + total));
+    }
+    if (lane < (uint32_t)kChunksPerCounter)
+      status_store(offsets + (size_t)index * kChunksPerCounter + lane,
+                   kFlagInclusive | (uint64_t)(exclusive + (int64_t)(incl - mine)));
+    if (lane == 0 && index == ncounters - 1)
+      __hip_atomic_store(d_count, exclusive + (int64_t)total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    return;
+  }
+
+  // ---- mover: one 2048-element chunk, 4 wavefronts x 2 steps
+  if (index >= nchunks) return;
+  const int64_t start = (int64_t)index * 2048;
+  const uint32_t lane_off = wave * 512 + lane * 4;
+  uint32_t w[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k)
+    w[k] = *reinterpret_cast<const uint32_t *>(mask + start + lane_off + k * 256);
+  uint32_t bits = 0;
+#pragma unroll
+  for (int k = 0; k < 2; ++k) bits |= select_bits(w[k]) << (4 * k);
+  const uint32_t wt = wave_sum_u32(__popc(bits));
+  if (lane == 0) sh.wave_total[wave] = wt;
+  f32x4 vals[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k)
+    if ((bits >> (4 * k)) & 0xFu)
+      vals[k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src + start + lane_off + k * 256));
+  if (threadIdx.x == 0) {
+    uint64_t o = 0;
+    int spins = 0;
+    while (((o = status_load(offsets + index)) >> kFlagShift) == 0) {
+      if (++spins > kAheadSpinCap) {
+        *err = 2u;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    sh.base = (int64_t)(o & kValueMask);
+  }
+  __syncthreads();
+  uint32_t wbase = 0;
+#pragma unroll
+  for (int v = 0; v < 4; ++v)
+    if ((uint32_t)v < wave) wbase += sh.wave_total[v];
+  float *stage = sh.stage[wave];
+  float *wout = out + (sh.base + wbase);
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 3u);
+  uint32_t run = shift;
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const uint32_t f = (bits >> (4 * k)) & 0xFu;
+    uint32_t below, total;
+    wave_offsets(__popc(f), below, total);
+    if (f) {
+      uint32_t pos = run + below;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (f & (1u << j)) stage[pos++] = vals[k][j];
+    }
+    run += total;
+  }
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t span_end = shift + wt;
+  float *obase = wout - shift;
+  if (wt != 0) {
+    for (uint32_t v = lane; 4 * v < span_end; v += 64) {
+      const f32x4 x = *reinterpret_cast<const f32x4 *>(stage + 4 * v);
+      if (4 * v >= shift && 4 * v + 4 <= span_end) {
+        __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * v));
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t i = 4 * v + c;
+          if (i >= shift && i < span_end) obase[i] = x[c];
+        }
+      }
+    }
+  }
+}
+
+
 // One-shot workgroups like the streaming kernel's, but SWAVES wavefronts stream and one more,
 // the last, owns no elements: it publishes the tile's aggregate, looks back and hands the
 // tile's base to the others through LDS.  The streaming wavefronts do not wait for it:
@@ -874,6 +1053,37 @@ struct SelectStudy {
     return 0;
   }
 
+  // counters ahead of movers: needs a table of one word per 2048-element chunk
+  template <int LEAD>
+  int counters_ahead(uint64_t *offsets) {
+    if (n % (2048 * kChunksPerCounter) != 0) return 0;
+    const uint32_t nchunks = (uint32_t)(n / 2048);
+    const uint32_t ncounters = nchunks / kChunksPerCounter;
+    uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+    if (kMsHeaderBytes + 8 * (size_t)ncounters > scratch_bytes) return -1;
+    const unsigned grid = (unsigned)LEAD + ncounters * (kChunksPerCounter + 1);
+    TWGA_TRY(hipMemsetAsync(err, 0, 4, tm.s));
+    TWGA_TRY(hipMemsetAsync(out, 0, (size_t)n * 4, tm.s));
+    float ms = 0;
+    int rc = tm.run([&] {
+      (void)hipMemsetAsync(scratch, 0, kMsHeaderBytes + 8 * (size_t)ncounters, tm.s);
+      (void)hipMemsetAsync(offsets, 0, 8 * (size_t)nchunks, tm.s);
+      counters_ahead_of_movers<LEAD><<<grid, 256, 0, tm.s>>>(out, cnt, src, mask, nchunks, status, offsets, err);
+    }, &ms);
+    if (rc) return rc;
+    int64_t k = -1;
+    uint32_t e = 0;
+    TWGA_TRY(hipMemcpyAsync(&k, cnt, 8, hipMemcpyDeviceToHost, tm.s));
+    TWGA_TRY(hipMemcpyAsync(&e, err, 4, hipMemcpyDeviceToHost, tm.s));
+    TWGA_TRY(hipStreamSynchronize(tm.s));
+    unsigned long long h = 0;
+    if ((rc = checksum(k, &h))) return rc;
+    char name[96];
+    std::snprintf(name, sizeof(name), "one-shot 2048-element movers, counter blocks %d x 16 chunks ahead", LEAD);
+    put(res, name, ms, bytes_of(n, k), (e == 0 && k == k_ref && h == sum_ref) ? 1 : 0);
+    return 0;
+  }
+
   template <int WAVES, int STEPS>
   int small_tiles() {
     constexpr int kTile = 256 * STEPS * WAVES;
@@ -1126,6 +1336,8 @@ int twga_masked_select(int log2n, float p, twga_result_t *out, int cap) {
   TWGA_STEP((st.small_tiles<4, 8>()));
   TWGA_STEP((st.small_tiles<4, 2>()));
   TWGA_STEP((st.small_tiles<16, 4>()));
+  TWGA_STEP((st.counters_ahead<512>(reinterpret_cast<uint64_t *>(st.bases))));
+  TWGA_STEP((st.counters_ahead<8192>(reinterpret_cast<uint64_t *>(st.bases))));
   TWGA_STEP((st.run_ahead<15, true>()));
   TWGA_STEP((st.run_ahead<15, false>()));
   TWGA_STEP((st.front_wave<15, 4, 3>()));
