@@ -307,7 +307,21 @@ def calibration_transfers(capi, L):
     capi.check(L.twg_fill_bytes(a.ptr, 0x5A, gib, None))
     capi.sync()
     res = {}
-    for name, fn in (("hipMemcpyAsync_d2d_1GiB", lambda: capi.check(L.twg_memcpy_d2d(b.ptr, a.ptr, gib, None))),
+    # the runtime's own device-to-device copy, called directly: an anchor that is none of the
+    # library's kernels (twg_memcpy_d2d uses the library's copy kernel at this size)
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                                   ctypes.c_void_p]
+    hip.hipMemcpyAsync.restype = ctypes.c_int
+    L.twg_default_stream.restype = ctypes.c_void_p
+    stream = L.twg_default_stream()
+
+    def runtime_copy():
+        rc = hip.hipMemcpyAsync(b.ptr, a.ptr, gib, 3, stream)  # 3 = hipMemcpyDeviceToDevice
+        if rc:
+            raise RuntimeError(f"hipMemcpyAsync failed: {rc}")
+
+    for name, fn in (("hipMemcpyAsync_d2d_1GiB", runtime_copy),
                      ("twg_fill_bytes_1GiB", lambda: capi.check(L.twg_fill_bytes(b.ptr, 0xA5, gib, None)))):
         fn()
         capi.sync()

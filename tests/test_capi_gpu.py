@@ -102,6 +102,24 @@ def test_copy_round_trip_fp32_and_bool(twg):
     assert bit_equal(raw[8:-8].view(torch.float32), t)
 
 
+def test_large_device_to_device_copies(twg):
+    # from 128 MiB on, aligned copies run the library's own streaming copy kernel and hand a
+    # tail of 1-3 bytes to the runtime; misaligned ones stay with the runtime
+    L = twg.load()
+    nb = (1 << 27) + 4096 + 3
+    g = torch.Generator().manual_seed(5)
+    host = torch.randint(0, 256, (nb + 64,), dtype=torch.uint8, generator=g)
+    src = twg.to_device(host)
+    dst = twg.DeviceBuffer(nb + 128)
+    for d_off, s_off in ((16, 0), (16, 16), (17, 0), (16, 1), (32, 48)):
+        _say(f"d2d {nb} bytes, offsets {d_off}/{s_off}")
+        twg.check(L.twg_fill_bytes(dst.ptr, 0xCD, dst.nbytes, None))
+        twg.check(L.twg_memcpy_d2d(dst.ptr + d_off, src.ptr + s_off, nb, None))
+        raw = dst.download((dst.nbytes,), torch.uint8)
+        assert torch.equal(raw[d_off:d_off + nb], host[s_off:s_off + nb]), (d_off, s_off)
+        assert bool((raw[:d_off] == 0xCD).all()) and bool((raw[d_off + nb:] == 0xCD).all())
+
+
 def test_copy_sizes_around_every_staging_boundary(twg):
     # The pinned ring is divided differently for each copy size and large copies are split
     # over helper threads; sizes just below, at and above each switch, with ragged tails, in

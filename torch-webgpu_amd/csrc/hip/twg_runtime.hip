@@ -892,6 +892,26 @@ int twg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes, twg_stream
   if (!dst_dev || !src_dev) return TWG_E_INVALID_ARG;
   int rc = ensure_init();
   if (rc) return rc;
+  // From 128 MiB on, the library's own streaming copy is the faster one (1 GiB: 0.32 ms
+  // against 0.41 ms for hipMemcpyAsync); below, the runtime's copy is as fast or faster
+  // (64 MiB: 19.5 against 23 us).
+  constexpr size_t kOwnCopyMin = size_t(1) << 27;
+  if (nbytes >= kOwnCopyMin && reinterpret_cast<uintptr_t>(dst_dev) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(src_dev) % 16 == 0) {
+    twg_iter_t it{};
+    it.ndim = 1;
+    it.numel = (int64_t)(nbytes / 4);
+    it.shape[0] = it.numel;
+    it.stride[TWG_OUT][0] = it.stride[TWG_A][0] = it.stride[TWG_B][0] = 1;
+    rc = twg_unary_f32(TWG_UNARY_COPY, static_cast<float *>(dst_dev),
+                       static_cast<const float *>(src_dev), &it, stream);
+    if (rc) return rc;
+    const size_t done = (size_t)it.numel * 4;
+    if (done == nbytes) return 0;
+    dst_dev = static_cast<char *>(dst_dev) + done;
+    src_dev = static_cast<const char *>(src_dev) + done;
+    nbytes -= done;
+  }
   TWG_HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, nbytes, hipMemcpyDeviceToDevice,
                              resolve_stream(stream)));
   return 0;
