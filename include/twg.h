@@ -282,8 +282,10 @@ int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
  * pinned host memory the moment the last tile knows it and the host polls that word,
  * which saves the separate read-back of twg_masked_select_f32 + twg_memcpy_d2h (one
  * launch and one wait per call).  This is what the masked_select registration calls:
- * it needs K to shape the result.  `out` and `src` must be aligned to elem_size;
- * 4-byte elements take the same kernels as twg_masked_select_f32. */
+ * it needs K to shape the result.  `out` and `src` must be aligned to elem_size; every
+ * element size takes the kernels of twg_masked_select_f32, instantiated for it (dense
+ * operands with `src` aligned to four elements, 16 bytes for 8-byte elements; anything
+ * else runs the one-element-per-lane variant). */
 int twg_masked_select_count(void *out, int64_t *count_host, const void *src,
                             int32_t elem_size, const uint8_t *mask, const twg_iter_t *it,
                             void *scratch, size_t scratch_bytes, twg_stream_t stream);

@@ -645,6 +645,36 @@ def test_masked_select_every_element_size(twg, dtype):
     assert bit_equal(vals, torch.masked_select(xt, m[:100]))
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int64, torch.float64])
+def test_masked_select_fast_kernels_every_element_size(twg, dtype):
+    # the streaming kernel (all three tile sizes, with a remainder launch) and the tile variant
+    # for 1-, 2- and 8-byte elements: dense and sparse masks, runs, shifted output pointers
+    g = torch.Generator().manual_seed(35)
+    es = torch.empty(0, dtype=dtype).element_size()
+    for n in (8192 * 3 + 17, (1 << 21) + 8192 + 5, (1 << 23) + 70001, (1 << 25) + 131072 + 4099):
+        if dtype.is_floating_point:
+            x = torch.randn(n, generator=g, dtype=dtype)
+        else:
+            info = torch.iinfo(dtype)
+            x = torch.randint(max(info.min, -(1 << 62)), min(info.max, 1 << 62), (n,), generator=g,
+                              dtype=dtype)
+        idx = torch.arange(n)
+        masks = {
+            "p=0.5": torch.rand(n, generator=g) < 0.5,
+            "p=0.99": torch.rand(n, generator=g) < 0.99,
+            "p=0.02": torch.rand(n, generator=g) < 0.02,
+            "every 16th": idx % 16 == 5,
+            "runs": (idx % 5003) < 2500,
+            "last only": idx == n - 1,
+        }
+        for name, m in masks.items():
+            ref = torch.masked_select(x, m)
+            for off in (0, 1, 128 // es - 1):
+                _say(f"masked_select {dtype} n={n} {name} out_offset={off}")
+                vals, k = H.masked_select(x, m, out_offset=off, check_guard=True)
+                assert k == ref.numel() and bit_equal(vals, ref), (dtype, n, name, off)
+
+
 # ------------------------------------------------------------- activations
 
 def _unary(op, x, **kw):

@@ -21,10 +21,11 @@ constexpr int kSmallWaves = 4;
 constexpr int64_t kSmallTile = (int64_t)kWaveElems * kSmallWaves;
 constexpr int64_t kStreamMinElems = int64_t(1) << 21;
 
+template <typename T>
 struct MsLaunch {
-  float *out;
+  T *out;
   int64_t *d_count;
-  const float *src;
+  const T *src;
   const uint8_t *mask;
   int64_t numel;
   uint32_t *ticket;  // [0] streaming launch, [1] remainder launch
@@ -37,8 +38,8 @@ struct MsLaunch {
 // Full tiles go through the streaming kernel; what is left (less than one of its tiles)
 // is compacted by a second launch of the tile variant that starts from the first
 // launch's total.
-template <int WAVES, int GROUPS>
-int launch_stream(const MsLaunch &m) {
+template <int WAVES, int GROUPS, typename T>
+int launch_stream(const MsLaunch<T> &m) {
   constexpr int64_t kTile = (int64_t)256 * 8 * GROUPS * WAVES;
   const int64_t nbig = m.numel / kTile;
   const int64_t rem = m.numel - nbig * kTile;
@@ -50,12 +51,42 @@ int launch_stream(const MsLaunch &m) {
                           m.stream);
   if (rc) return rc;
   hipStream_t s = resolve_stream(m.stream);
-  ms_compact_stream<WAVES, GROUPS><<<(unsigned)nbig, WAVES * 64, 0, s>>>(
+  ms_compact_stream<WAVES, GROUPS, 5, T><<<(unsigned)nbig, WAVES * 64, 0, s>>>(
       m.out, rem ? m.carry : m.d_count, m.src, m.mask, (uint32_t)nbig, m.ticket, m.status);
   if (rem)
-    ms_compact_vec<kSmallWaves><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
+    ms_compact_vec<kSmallWaves, T><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
         m.out, m.d_count, m.src + nbig * kTile, m.mask + nbig * kTile, rem, (uint32_t)nrem,
         m.ticket + 1, m.status + big_words, m.carry);
+  return (int)hipGetLastError();
+}
+
+// The fast variants for one element type: streaming tiles for large inputs, the tile
+// variant below that.
+template <typename T>
+int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t *mask, int64_t numel,
+                void *scratch, twg_stream_t stream) {
+  // scratch: [0] ticket, [4] ticket of the remainder launch, [8] carry between the
+  // two launches, [256...] one status word per tile
+  uint32_t *ticket = static_cast<uint32_t *>(scratch);
+  int64_t *carry = reinterpret_cast<int64_t *>(static_cast<char *>(scratch) + 8);
+  uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+  T *out = static_cast<T *>(out_v);
+  const T *src = static_cast<const T *>(src_v);
+  if (numel >= kStreamMinElems) {
+    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, carry, status, scratch, stream};
+    if (numel >= (int64_t(1) << 25)) return launch_stream<16, 4>(m);
+    if (numel >= (int64_t(1) << 23)) return launch_stream<16, 2>(m);
+    return launch_stream<8, 1>(m);
+  }
+  const int64_t ntiles64 = (numel + kSmallTile - 1) / kSmallTile;
+  const uint32_t ntiles = (uint32_t)ntiles64;
+  int rc = 0;
+  // one tile takes no ticket and looks back at nothing: the scratch may hold anything
+  if (ntiles > 1 &&
+      (rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
+    return rc;
+  ms_compact_vec<kSmallWaves, T><<<ntiles, kSmallWaves * 64, 0, resolve_stream(stream)>>>(
+      out, d_count, src, mask, numel, ntiles, ticket, status, nullptr);
   return (int)hipGetLastError();
 }
 
@@ -98,28 +129,25 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
   hipStream_t s = resolve_stream(stream);
   const bool dense =
       g.ndim == 0 || (g.ndim == 1 && g.stride[TWG_A][0] == 1 && g.stride[TWG_B][0] == 1);
-  float *out = static_cast<float *>(out_v);  // the fast variants move 4-byte elements
-  const float *src = static_cast<const float *>(src_v);
-  const bool vec4 = elem_size == 4 && dense && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
-                    reinterpret_cast<uintptr_t>(mask) % 4 == 0 &&
-                    reinterpret_cast<uintptr_t>(out) % 4 == 0;
-
-  // scratch: [0] ticket, [4] ticket of the remainder launch, [8] carry between the
-  // two launches, [256...] one status word per tile
-  uint32_t *ticket = static_cast<uint32_t *>(scratch);
-  int64_t *carry = reinterpret_cast<int64_t *>(static_cast<char *>(scratch) + 8);
-  uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
-  auto tiles_of = [](int64_t n, int64_t tile) { return (n + tile - 1) / tile; };
-
-  if (vec4 && g.numel >= kStreamMinElems) {
-    const MsLaunch m{out, d_count, src, mask, g.numel, ticket, carry, status, scratch, stream};
-    if (g.numel >= (int64_t(1) << 25)) return launch_stream<16, 4>(m);
-    if (g.numel >= (int64_t(1) << 23)) return launch_stream<16, 2>(m);
-    return launch_stream<8, 1>(m);
+  // The fast variants want the source aligned to four of its elements (one lane's share of
+  // a step; 16 bytes are enough for 8-byte elements, which take two loads) and the mask to
+  // a dword.  They move 4-byte elements as floats, the others as unsigned integers.
+  const uintptr_t src_align = elem_size == 8 ? 16 : (uintptr_t)(4 * elem_size);
+  const bool fast = dense && reinterpret_cast<uintptr_t>(src_v) % src_align == 0 &&
+                    reinterpret_cast<uintptr_t>(mask) % 4 == 0;
+  if (fast) {
+    switch (elem_size) {
+      case 1: return launch_fast<uint8_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
+      case 2: return launch_fast<uint16_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
+      case 4: return launch_fast<float>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
+      default: return launch_fast<uint64_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
+    }
   }
 
-  const int64_t tile = vec4 ? kSmallTile : (int64_t)kScalarTile;
-  const int64_t ntiles64 = tiles_of(g.numel, tile);
+  // scratch: [0] ticket, [256...] one status word per tile
+  uint32_t *ticket = static_cast<uint32_t *>(scratch);
+  uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+  const int64_t ntiles64 = (g.numel + kScalarTile - 1) / kScalarTile;
   if (ntiles64 > INT32_MAX) return TWG_E_UNSUPPORTED;
   const uint32_t ntiles = (uint32_t)ntiles64;
   // one tile takes no ticket and looks back at nothing: the scratch may hold anything
@@ -127,10 +155,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
       (rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
     return rc;
 
-  if (vec4) {
-    ms_compact_vec<kSmallWaves><<<ntiles, kSmallWaves * 64, 0, s>>>(
-        out, d_count, src, mask, g.numel, ntiles, ticket, status, nullptr);
-  } else {
+  {
     MsGeom mg{};
     mg.ndim = g.ndim;
     for (int d = 0; d < TWG_MAX_DIMS; ++d) {

@@ -205,45 +205,105 @@ __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, 
 }
 
 // ------------------------------------------------------------------ fast variants
-// Dense source and mask, 16-byte aligned source, 4-byte aligned mask.  Lane l of a
-// wavefront owns elements 4l..4l+3 of each 256-element step.
+// Dense source and mask; the source aligned to four of its elements (16 bytes at most), the
+// mask to 4 bytes.  Lane l of a wavefront owns elements 4l..4l+3 of each 256-element step.
+// The values are moved without being looked at: T is float for 4-byte elements and an
+// unsigned integer of the element's size otherwise.
+
+typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+
+// Four consecutive elements, loaded with the widest loads they allow.
+template <typename T>
+struct Quad;
+template <>
+struct Quad<float> {
+  f32x4 v;
+  __device__ __forceinline__ float get(int j) const { return v[j]; }
+  __device__ __forceinline__ void set(int j, float x) { v[j] = x; }
+  static __device__ __forceinline__ Quad load(const float *p) {
+    return {__builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p))};
+  }
+};
+template <>
+struct Quad<uint64_t> {
+  u64x2 a, b;
+  __device__ __forceinline__ uint64_t get(int j) const { return j < 2 ? a[j] : b[j - 2]; }
+  __device__ __forceinline__ void set(int j, uint64_t x) {
+    if (j < 2) a[j] = x; else b[j - 2] = x;
+  }
+  static __device__ __forceinline__ Quad load(const uint64_t *p) {
+    return {__builtin_nontemporal_load(reinterpret_cast<const u64x2 *>(p)),
+            __builtin_nontemporal_load(reinterpret_cast<const u64x2 *>(p) + 1)};
+  }
+};
+template <>
+struct Quad<uint16_t> {
+  u16x4 v;
+  __device__ __forceinline__ uint16_t get(int j) const { return v[j]; }
+  __device__ __forceinline__ void set(int j, uint16_t x) { v[j] = x; }
+  static __device__ __forceinline__ Quad load(const uint16_t *p) {
+    return {__builtin_nontemporal_load(reinterpret_cast<const u16x4 *>(p))};
+  }
+};
+template <>
+struct Quad<uint8_t> {
+  uint32_t v;
+  __device__ __forceinline__ uint8_t get(int j) const { return (uint8_t)(v >> (8 * j)); }
+  __device__ __forceinline__ void set(int j, uint8_t x) {
+    v = (v & ~(0xFFu << (8 * j))) | ((uint32_t)x << (8 * j));
+  }
+  static __device__ __forceinline__ Quad load(const uint8_t *p) {
+    return {__builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p))};
+  }
+};
 
 // ---- streaming variant: full tiles only (the host launches it on a multiple of the
 // tile size, so it carries no bounds checks).  Wavefront w owns GROUPS * 8
 // consecutive steps of the tile.
-constexpr int kRingElems = 512;  // per wavefront; at most 31 + 256 values wait in it
+constexpr int kRingElems = 512;  // per wavefront; at most a line less one element + 256 values wait in it
 // Source steps in flight per wavefront.  4 measured best: 8 keeps more in flight than
 // the memory system rewards (dense masks lose 2-3%), and below ~64 VGPRs a second
 // 1024-lane workgroup becomes resident per CU, which costs dense masks 5-10%.
 constexpr int kDepth = 4;
 // A wavefront of the streaming kernel with at most one selected element in 16 gathers
-// them individually instead of streaming its steps (measured at 2^28 elements, 8192 per
-// wavefront: 0.121 ms against 0.164 ms at 1% selected, 0.185 against 0.205 ms at 3%, even
-// at 5%; above that the streaming loop wins).
+// them individually instead of streaming its steps (measured at 2^28 float elements, 8192
+// per wavefront: 0.121 ms against 0.164 ms at 1% selected, 0.185 against 0.205 ms at 3%,
+// even at 5%; above that the streaming loop wins).
 constexpr uint32_t kSparseDivisor = 16;
+// The ring also holds the gather path's element-order bitmap (256 words) and position
+// list (at most 512 words).
+template <typename T>
+constexpr int ring_bytes() {
+  return kRingElems * (int)sizeof(T) > 2048 ? kRingElems * (int)sizeof(T) : 2048;
+}
 
-template <int WAVES, int GROUPS>
+template <int WAVES, int GROUPS, typename T>
 struct MsStreamShared {
   uint32_t tile;
   uint32_t wave_total[WAVES];
   int64_t base;
   uint32_t bits[GROUPS][WAVES * 64];  // 4 selection bits per step, 8 steps per word
-  __attribute__((aligned(16))) float ring[WAVES][kRingElems];
+  __attribute__((aligned(16))) unsigned char ring[WAVES][ring_bytes<T>()];
 };
 
 // STAGES cuts the kernel short for timing experiments (the benchmark's ablation library
 // instantiates 1..4; the library itself only ever runs all 5): 1 = take the ticket, 2 = + mask
 // loads, selection bits and counts, 3 = + aggregate, look-back and the first source loads,
 // 4 = + every source load and the compaction in LDS, 5 = + the stores.
-template <int WAVES, int GROUPS, int STAGES = 5>
-__global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int64_t *d_count,
-                                                                const float *src,
+template <int WAVES, int GROUPS, int STAGES = 5, typename T = float>
+__global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t *d_count,
+                                                                const T *src,
                                                                 const uint8_t *mask,
                                                                 uint32_t ntiles, uint32_t *ticket,
                                                                 uint64_t *status) {
   constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
   constexpr int64_t kTileElems = (int64_t)kWaveSpan * WAVES;
-  __shared__ MsStreamShared<WAVES, GROUPS> sh;
+  constexpr uint32_t kLine = 128u / sizeof(T);  // elements per 128-byte line
+  constexpr uint32_t kSlot = 16u / sizeof(T);   // elements per 16-byte store
+  constexpr uint32_t kLineShift = sizeof(T) == 1 ? 7 : sizeof(T) == 2 ? 6 : sizeof(T) == 4 ? 5 : 4;
+  static_assert(kLine - 1 + 256 <= (uint32_t)kRingElems, "a step must fit the ring behind a partial line");
+  __shared__ MsStreamShared<WAVES, GROUPS, T> sh;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
   if (threadIdx.x == 0)
@@ -253,7 +313,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
   if constexpr (STAGES < 2) return;
   const int64_t start = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
   const uint8_t *mask_w = mask + start + lane * 4;
-  const float *src_w = src + start + lane * 4;
+  const T *src_w = src + start + lane * 4;
 
   // ---- 1. masks -> packed selection bits in LDS, wavefront totals
   uint32_t cnt = 0;
@@ -287,17 +347,16 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
   }
 
   // ---- 2. the first kDepth steps' values go in flight, then aggregate / look-back
-  const f32x4 *dummy = reinterpret_cast<const f32x4 *>(src + (int64_t)tile * kTileElems);
+  const T *dummy = src + (int64_t)tile * kTileElems;
   auto fetch = [&](uint32_t four_bits, int step) {
-    const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + step * 256);
-    return __builtin_nontemporal_load(four_bits ? p : dummy);
+    return Quad<T>::load(four_bits ? src_w + step * 256 : dummy);
   };
   uint32_t b_cur = sh.bits[0][threadIdx.x];
   constexpr uint32_t kSparseMax = kWaveSpan / kSparseDivisor;
-  static_assert(kSparseMax <= (uint32_t)kRingElems && kWaveSpan <= 8192u,
+  static_assert(kSparseMax <= 512u && kWaveSpan <= 8192u,
                 "the bitmap and the position list live in the wavefront's ring");
   const bool sparse = wt <= kSparseMax;  // wavefront-uniform
-  f32x4 vals[kDepth] = {};
+  Quad<T> vals[kDepth] = {};
   if (!sparse) {
 #pragma unroll
     for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
@@ -305,10 +364,10 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
   const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(
       status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
   if constexpr (STAGES < 4) {
-    float acc = 0.0f;
+    uint32_t acc = 0;
 #pragma unroll
-    for (int k = 0; k < kDepth; ++k) acc += vals[k][0];
-    if (acc == 1.2345e38f) out[base + wbase] = acc;  // practically never: keeps the loads alive
+    for (int k = 0; k < kDepth; ++k) acc += (uint32_t)vals[k].get(0);
+    if (acc == 0x7E39A4C5u) out[base + wbase] = vals[0].get(0);  // practically never: keeps the loads alive
     return;
   }
 
@@ -355,13 +414,13 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
       }
     }
     __builtin_amdgcn_wave_barrier();
-    const float *src_wave = src + start;
-    float *wout = out + (base + wbase);
+    const T *src_wave = src + start;
+    T *wout = out + (base + wbase);
     for (uint32_t i = lane; i < wt; i += 64) {
-      const float x = __builtin_nontemporal_load(src_wave + lds[i]);
+      const T x = __builtin_nontemporal_load(src_wave + lds[i]);
       if constexpr (STAGES >= 5) {
         wout[i] = x;
-      } else if (x == 1.2345e38f) {  // practically never
+      } else if ((uint32_t)x == 0x7E39A4C5u) {  // practically never
         wout[i] = x;
       }
     }
@@ -371,12 +430,12 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
   // ---- 3. stream: compact a step into the ring, refill its register for kDepth steps
   //         later, write out the lines the step completed.  Position p of this
   //         wavefront's run is obase[p] in memory and ring[p % kRingElems] in LDS.
-  float *ring = sh.ring[wave];
-  float *wout = out + (base + wbase);
-  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 31u);
-  float *obase = wout - shift;         // 128-byte aligned
+  T *ring = reinterpret_cast<T *>(sh.ring[wave]);
+  T *wout = out + (base + wbase);
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) / sizeof(T)) & (kLine - 1));
+  T *obase = wout - shift;             // 128-byte aligned
   uint32_t run = shift;                // next free position
-  uint32_t flushed = shift ? 8u : 0u;  // float4 slots written; a shifted first line is not ours alone
+  uint32_t flushed = shift ? 8u : 0u;  // 16-byte slots written; a shifted first line is not ours alone
 #pragma unroll 1
   for (int g = 0; g < GROUPS; ++g) {
     const int gn = (g + 1 < GROUPS) ? g + 1 : g;  // past the end: all lanes read the dummy
@@ -386,7 +445,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
       const uint32_t f = (b_cur >> (4 * k)) & 0xFu;
       uint32_t below, total;
       wave_offsets(__popc(f), below, total);
-      const f32x4 x4 = vals[k % kDepth];
+      const Quad<T> x4 = vals[k % kDepth];
       {
         const int ahead = k + kDepth;  // the step to prefetch, counted from this group's first
         vals[k % kDepth] = ahead < 8 ? fetch((b_cur >> (4 * ahead)) & 0xFu, g * 8 + ahead)
@@ -397,25 +456,26 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if (f & (1u << j)) {
-            const float x = x4[j];
+            const T x = x4.get(j);
             ring[pos & (kRingElems - 1)] = x;
             if constexpr (STAGES >= 5)
-              if (pos < 32u && shift) obase[pos] = x;  // shared first line: element by element
+              if (pos < kLine && shift) obase[pos] = x;  // shared first line: element by element
             ++pos;
           }
         }
       }
       run += total;
-      const uint32_t end4 = (run >> 5) << 3;  // whole 128-byte lines only
-      if (end4 > flushed) {                   // wavefront-uniform
+      const uint32_t end4 = (run >> kLineShift) << 3;  // whole 128-byte lines only
+      if (end4 > flushed) {                            // wavefront-uniform
         __builtin_amdgcn_wave_barrier();
         for (uint32_t idx = flushed + lane; idx < end4; idx += 64) {
-          const f32x4 x =
-              *reinterpret_cast<const f32x4 *>(ring + ((4 * idx) & (kRingElems - 1)));
+          const u32x4 x = *reinterpret_cast<const u32x4 *>(
+              sh.ring[wave] + ((16u * idx) & (uint32_t)(kRingElems * sizeof(T) - 1)));
           if constexpr (STAGES >= 5) {
-            __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * (size_t)idx));
-          } else if (x[0] == 1.2345e38f && x[3] == -1.2345e38f) {  // practically never
-            obase[4 * (size_t)idx] = x[1];
+            __builtin_nontemporal_store(
+                x, reinterpret_cast<u32x4 *>(reinterpret_cast<unsigned char *>(obase) + 16 * (size_t)idx));
+          } else if (x[0] == 0x7E39A4C5u && x[3] == 0xFE39A4C5u) {  // practically never
+            obase[kSlot * (size_t)idx] = ring[(kSlot * idx) & (kRingElems - 1)];
           }
         }
         flushed = end4;
@@ -425,30 +485,30 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(float *out, int6
     b_cur = b_next;
   }
   // the last, incomplete line (its other elements belong to the next wavefront)
-  const uint32_t p = 4 * flushed + lane;
   if constexpr (STAGES >= 5)
-    if (lane < 32 && p < run) obase[p] = ring[p & (kRingElems - 1)];
+    for (uint32_t p = kSlot * flushed + lane; p < run; p += 64) obase[p] = ring[p & (kRingElems - 1)];
 }
 
 // ---- tile variant: any length.  One pass of 8 steps per wavefront, compacted in LDS at
-// the 16-byte phase the values will have in memory and written as aligned float4s.
-template <int WAVES>
+// the 16-byte phase the values will have in memory and written as aligned 16-byte packs.
+template <int WAVES, typename T>
 struct MsShared {
   uint32_t tile;
   uint32_t wave_total[WAVES];
   int64_t base;
-  __attribute__((aligned(16))) float stage[WAVES][kWaveElems + 4];
+  __attribute__((aligned(16))) T stage[WAVES][kWaveElems + 16 / sizeof(T)];
 };
 
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t *d_count,
-                                                             const float *src,
+template <int WAVES, typename T = float>
+__global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_count,
+                                                             const T *src,
                                                              const uint8_t *mask, int64_t n,
                                                              uint32_t ntiles, uint32_t *ticket,
                                                              uint64_t *status,
                                                              const int64_t *carry_in) {
   constexpr int64_t kTileElems = (int64_t)kWaveElems * WAVES;
-  __shared__ MsShared<WAVES> sh;
+  constexpr uint32_t kSlot = 16u / sizeof(T);  // elements per 16-byte store
+  __shared__ MsShared<WAVES, T> sh;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
   // A launch of a single tile needs no ticket (and no cleared scratch: nothing is looked back at).
@@ -461,7 +521,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t
   // tile bases are wavefront-uniform; everything per lane is a 32-bit offset
   const int64_t start = (int64_t)tile * kTileElems;
   const uint8_t *mask_tile = mask + start;
-  const float *src_tile = src + start;
+  const T *src_tile = src + start;
   const uint32_t lane_off = wave * kWaveElems + lane * 4;
   const int64_t left = n - start;
   const uint32_t remaining = left < kTileElems ? (uint32_t)left : (uint32_t)kTileElems;
@@ -495,25 +555,25 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t
   }
 
   // ---- 2. source values go in flight, then aggregate / look-back
-  f32x4 vals[kSteps];
+  Quad<T> vals[kSteps];
 #pragma unroll
   for (int k = 0; k < kSteps; ++k) {
     if ((bits >> (4 * k)) & 0xFu) {
       const uint32_t e = lane_off + k * 256;
       if (e + 4 <= remaining) {
-        vals[k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src_tile + e));
+        vals[k] = Quad<T>::load(src_tile + e);
       } else {
-        for (uint32_t j = 0; j < 4; ++j) vals[k][j] = (e + j < remaining) ? src_tile[e + j] : 0.0f;
+        for (uint32_t j = 0; j < 4; ++j) vals[k].set((int)j, (e + j < remaining) ? src_tile[e + j] : T(0));
       }
     }
   }
   const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, carry_in);
 
-  // ---- 3. compact in LDS, write aligned float4s; the ragged ends go out element by
+  // ---- 3. compact in LDS, write aligned 16-byte packs; the ragged ends go out element by
   //         element: their neighbours belong to other wavefronts.
-  float *stage = sh.stage[wave];
-  float *wout = out + (base + wbase);  // this wavefront's first output value
-  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 3u);
+  T *stage = sh.stage[wave];
+  T *wout = out + (base + wbase);  // this wavefront's first output value
+  const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) / sizeof(T)) & (kSlot - 1));
   uint32_t run = shift;
 #pragma unroll
   for (int k = 0; k < kSteps; ++k) {
@@ -524,24 +584,24 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(float *out, int64_t
       uint32_t pos = run + below;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (f & (1u << j)) stage[pos++] = vals[k][j];
+        if (f & (1u << j)) stage[pos++] = vals[k].get(j);
       }
     }
     run += total;
   }
   __builtin_amdgcn_wave_barrier();
   const uint32_t span_end = shift + wt;
-  float *obase = wout - shift;  // 16-byte aligned
+  T *obase = wout - shift;  // 16-byte aligned
   if (wt != 0) {
-    for (uint32_t v = lane; 4 * v < span_end; v += 64) {
-      const f32x4 x = *reinterpret_cast<const f32x4 *>(stage + 4 * v);
-      if (4 * v >= shift && 4 * v + 4 <= span_end) {
-        __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * v));
+    for (uint32_t v = lane; kSlot * v < span_end; v += 64) {
+      if (kSlot * v >= shift && kSlot * v + kSlot <= span_end) {
+        const u32x4 x = *reinterpret_cast<const u32x4 *>(stage + kSlot * v);
+        __builtin_nontemporal_store(x, reinterpret_cast<u32x4 *>(obase + kSlot * v));
       } else {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const uint32_t i = 4 * v + c;
-          if (i >= shift && i < span_end) obase[i] = x[c];
+        for (uint32_t c = 0; c < kSlot; ++c) {
+          const uint32_t i = kSlot * v + c;
+          if (i >= shift && i < span_end) obase[i] = stage[i];
         }
       }
     }
