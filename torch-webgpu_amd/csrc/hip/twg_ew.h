@@ -880,7 +880,7 @@ constexpr int kDeintLds = 8192;  // elements of one strip at most
 
 template <int NIN, bool A_D, bool B_D, typename Op, typename TO, typename TA, typename TB>
 __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const TB *b, TileGeom g,
-                                                     uint32_t tx_elems, Op op) {
+                                                     uint32_t tx_elems, uint32_t rows, Op op) {
   static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
   using PO = Pack<TO, 4>;
   using PA = Pack<TA, 4>;
@@ -892,7 +892,21 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   const uint32_t t0i = bid % g.tiles0;
   int64_t r = bid / g.tiles0;
   int64_t off_o = 0, off_a = 0, off_b = 0;
-  for (int d = 0; d < g.nbatch; ++d) {
+  // rows > 1 (dimension 0 is short): the block takes `rows` consecutive indices of the first
+  // batch dimension, one strip each
+  uint32_t nrows = 1;
+  int d_first = 0;
+  if (rows > 1) {
+    const int64_t q = r / g.tilest;
+    const int64_t row0 = (r - q * g.tilest) * rows;
+    r = q;
+    nrows = (uint32_t)(g.bshape[0] - row0 < (int64_t)rows ? g.bshape[0] - row0 : (int64_t)rows);
+    off_o = row0 * g.bstride[0][0];
+    off_a = row0 * g.bstride[1][0];
+    if constexpr (NIN == 2) off_b = row0 * g.bstride[2][0];
+    d_first = 1;
+  }
+  for (int d = d_first; d < g.nbatch; ++d) {
     const int64_t q = r / g.bshape[d];
     const int64_t c = r - q * g.bshape[d];
     r = q;
@@ -904,43 +918,54 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   const int64_t x0 = (int64_t)t0i * tx_elems;
   const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)tx_elems ? g.n0 - x0 : (int64_t)tx_elems);
   const uint32_t strip = nx * P;  // consecutive elements of a deinterleaved operand
+  const uint32_t pitch = (strip + 3u) & ~3u;  // of a strip in LDS
   if constexpr (A_D) {
     const TA *src = a + off_a + x0 * (int64_t)P;
-    for (uint32_t i = 4 * threadIdx.x; i < strip; i += 4 * kThreads)
-      *reinterpret_cast<PA *>(&sa[i]) = load4_edge(src + i, (int64_t)strip - i);
+    for (uint32_t i = 4 * threadIdx.x; i < nrows * pitch; i += 4 * kThreads) {
+      const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
+      if (j < strip)
+        *reinterpret_cast<PA *>(&sa[i]) = load4_edge(src + row * g.bstride[1][0] + j, (int64_t)strip - j);
+    }
   }
   if constexpr (NIN == 2 && B_D) {
     const TB *src = b + off_b + x0 * (int64_t)P;
-    for (uint32_t i = 4 * threadIdx.x; i < strip; i += 4 * kThreads)
-      *reinterpret_cast<PB *>(&sb[i]) = load4_edge(src + i, (int64_t)strip - i);
+    for (uint32_t i = 4 * threadIdx.x; i < nrows * pitch; i += 4 * kThreads) {
+      const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
+      if (j < strip)
+        *reinterpret_cast<PB *>(&sb[i]) = load4_edge(src + row * g.bstride[2][0] + j, (int64_t)strip - j);
+    }
   }
   __syncthreads();
   const uint32_t packs = (nx + 3) / 4;  // per channel
-  for (uint32_t idx = threadIdx.x; idx < packs * P; idx += kThreads) {
-    const uint32_t c = idx / packs, j = idx - c * packs;
+  const uint32_t per_row = packs * P;
+  for (uint32_t idx = threadIdx.x; idx < nrows * per_row; idx += kThreads) {
+    const uint32_t row = rows > 1 ? idx / per_row : 0u, rem = idx - row * per_row;
+    const uint32_t c = rem / packs, j = rem - c * packs;
     const uint32_t x = 4 * j;
     const int64_t left = (int64_t)nx - x;
     PA va;
     PB vb;
     if constexpr (A_D) {
+      const TA *l = sa + row * pitch;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) va.v[k] = k < left ? sa[(x + k) * P + c] : TA();
+      for (int k = 0; k < 4; ++k) va.v[k] = k < left ? l[(x + k) * P + c] : TA();
     } else {
-      va = load4_edge(a + off_a + x0 + x + (int64_t)c * g.st[1], left);
+      va = load4_edge(a + off_a + row * g.bstride[1][0] + x0 + x + (int64_t)c * g.st[1], left);
     }
     if constexpr (NIN == 2) {
       if constexpr (B_D) {
+        const TB *l = sb + row * pitch;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) vb.v[k] = k < left ? sb[(x + k) * P + c] : TB();
+        for (int k = 0; k < 4; ++k) vb.v[k] = k < left ? l[(x + k) * P + c] : TB();
       } else {
-        vb = load4_edge(b + off_b + x0 + x + (int64_t)c * g.st[2], left);
+        vb = load4_edge(b + off_b + row * g.bstride[2][0] + x0 + x + (int64_t)c * g.st[2], left);
       }
     }
     PO o;
 #pragma unroll
     for (int k = 0; k < 4; ++k)
       o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
-    TO *dst = out + off_o + x0 + x + (int64_t)c * g.st[0];
+    TO *dst = out + off_o + row * g.bstride[0][0] + x0 + x + (int64_t)c * g.st[0];
     if (left >= 4) {
       store4_any(dst, o);
     } else {
@@ -1369,18 +1394,35 @@ int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool 
     uint32_t tx = 1024;
     while ((int64_t)tx * P > kDeintLds) tx /= 2;
     const int64_t tiles0 = (tg.n0 + tx - 1) / tx;
+    // a short dimension 0 (one strip, a fraction of a block's lanes): a block takes several
+    // indices of the first batch dimension, as many strips as fit the LDS array and add up
+    // to about 1024 output elements per channel
+    uint32_t rows = 1;
+    int64_t row_tiles = 1;
+    if (tg.n0 < 512 && tg.nbatch >= 1) {
+      const int64_t pitch = (tg.n0 * P + 3) / 4 * 4;
+      int64_t fit = kDeintLds / pitch, want = (2048 + tg.n0 - 1) / tg.n0;
+      int64_t k = fit < want ? fit : want;
+      if (k > tg.bshape[0]) k = tg.bshape[0];
+      if (k >= 2) {
+        rows = (uint32_t)k;
+        row_tiles = (tg.bshape[0] + k - 1) / k;
+        batch = batch / tg.bshape[0] * row_tiles;
+      }
+    }
+    if (tg.n0 < 256 && rows < 2) return TWG_E_UNSUPPORTED;  // the gather kernel is as fast
     if (tiles0 > INT32_MAX || tiles0 * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
     tg.tiles0 = (uint32_t)tiles0;
-    tg.tilest = 1;
+    tg.tilest = (uint32_t)row_tiles;
     const unsigned grid = (unsigned)(tiles0 * batch);
     if (a_d && b_d) {
       if constexpr (NIN == 2)
-        ew_deint<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, op);
+        ew_deint<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, rows, op);
     } else if (a_d) {
-      ew_deint<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, op);
+      ew_deint<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, rows, op);
     } else {
       if constexpr (NIN == 2)
-        ew_deint<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, op);
+        ew_deint<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, rows, op);
     }
     return (int)hipGetLastError();
   }
@@ -1437,6 +1479,29 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
       const int r = launch_generic_vec<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
       if (r != TWG_E_UNSUPPORTED) return r;
     }
+    // An input stored [.., x, c] with a short c against an output stored [.., c, x]: strips
+    // through LDS (a single strip of fewer than 256 output elements per channel runs no
+    // faster than a gather; with another dimension to take several strips from, 32 are enough).
+    auto try_deint = [&]() -> int {
+      if (!(g.ndim >= 2 && g.stride[0][0] == 1 &&
+            (g.shape[0] >= 256 || (g.ndim >= 3 && g.shape[0] >= 32))))
+        return TWG_E_UNSUPPORTED;
+      const int64_t sa0 = g.stride[1][0];
+      const int64_t sb0 = (NIN == 2) ? g.stride[2][0] : 1;
+      const bool a_x = sa0 != 0 && sa0 != 1, b_x = NIN == 2 && sb0 != 0 && sb0 != 1;
+      if (!a_x && !b_x) return TWG_E_UNSUPPORTED;
+      const int o = a_x ? 1 : 2;
+      int pd = -1;
+      for (int d = 1; d < g.ndim; ++d)
+        if (g.stride[o][d] == 1 && g.shape[d] == g.stride[o][0]) pd = d;
+      if (pd < 1) return TWG_E_UNSUPPORTED;
+      return launch_deint<NIN, Op, TO, TA, TB>(out, a, b, g, pd, a_x, b_x, op, s);
+    };
+    // short rows of that layout would otherwise be taken by (i-c)
+    if (g.shape[0] < 256) {
+      const int r = try_deint();
+      if (r != TWG_E_UNSUPPORTED) return r;
+    }
     // (i-c) rows too short or too ragged for one block per 256-element row chunk: if the
     // output and one input are dense, walk them flat and gather the other input
     if constexpr (NIN == 2) {
@@ -1462,19 +1527,9 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
         if (r != TWG_E_UNSUPPORTED) return r;
       }
       // (iii-00) an input stored [.., x, c] with a short c against an output stored [.., c, x]
-      // (strips of fewer than 256 output elements per channel run no faster than the gather)
-      if (g.ndim >= 2 && g.shape[0] >= 256) {
-        const bool a_x = sa0 != 0 && sa0 != 1, b_x = NIN == 2 && sb0 != 0 && sb0 != 1;
-        if (a_x || b_x) {
-          const int o = a_x ? 1 : 2;
-          int pd = -1;
-          for (int d = 1; d < g.ndim; ++d)
-            if (g.stride[o][d] == 1 && g.shape[d] == g.stride[o][0]) pd = d;
-          if (pd >= 1) {
-            int r = launch_deint<NIN, Op, TO, TA, TB>(out, a, b, g, pd, a_x, b_x, op, s);
-            if (r != TWG_E_UNSUPPORTED) return r;
-          }
-        }
+      {
+        const int r = try_deint();
+        if (r != TWG_E_UNSUPPORTED) return r;
       }
       // (iii-0) an input whose two innermost memory dimensions are both other dimensions than
       // dimension 0, the inner one short (3 channels, a head size): walked as one transposed
