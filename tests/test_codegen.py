@@ -56,14 +56,21 @@ def test_streaming_masked_select_counts_its_loads():
     asm = _device_asm(os.path.join(ROOT, "torch-webgpu_amd", "csrc", "hip", "twg_masked_select.hip"),
                       "/tmp")
     parts = re.split(r"\n(_ZN3twg[^\n:]*):", asm)
+    # the instantiation for each element type (mangled: f = float, m / t / h = 8-, 2-, 1-byte
+    # unsigned) and the width of its source loads
+    wanted = {"f": "dwordx4", "m": "dwordx4", "t": "dwordx2", "h": "dword"}
+    seen = set()
     for i in range(1, len(parts), 2):
         name, body = parts[i], parts[i + 1].split("s_endpgm")[0]
-        if "ms_compact_streamILi16ELi4E" not in name:
+        m = re.search(r"ms_compact_streamILi16ELi4ELi5E([fmth])E", name)
+        if not m:
             continue
         waits = re.findall(r"s_waitcnt vmcnt\((\d+)\)", body)
         partial = [w for w in waits if int(w) > 0]
-        assert len(partial) >= 3 * len([w for w in waits if int(w) == 0]), (len(partial), len(waits))
-        src_loads = [l for l in body.split("\n") if "global_load_dwordx4" in l]
-        assert src_loads and all(" nt" in l for l in src_loads)
-        return
-    raise AssertionError("streaming kernel not found in the assembly")
+        assert len(partial) >= 3 * len([w for w in waits if int(w) == 0]), (name, len(partial), len(waits))
+        # (the look-back's status words are 8-byte loads too: agent scope, marked sc1)
+        src_loads = [l for l in body.split("\n")
+                     if f"global_load_{wanted[m.group(1)]} " in l and " sc1" not in l]
+        assert src_loads and all(" nt" in l for l in src_loads), name
+        seen.add(m.group(1))
+    assert seen == set(wanted), f"streaming kernel instantiations found: {sorted(seen)}"
