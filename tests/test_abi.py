@@ -61,6 +61,30 @@ def test_error_strings_without_gpu():
     assert lib.twg_masked_select_scratch_bytes(1 << 28) >= 8 * ((1 << 28) // 8192)
 
 
+def test_masked_select_scratch_covers_every_launch_variant():
+    # what the host side clears before a launch (twg_masked_select.hip): a 256-byte header and
+    # one 8-byte status word per 8192-element tile of the tile variant, or, from 2^21 elements,
+    # four words per streaming tile (16384 / 65536 / 131072 elements) plus one per 8192-element
+    # tile of the remainder launch; the one-element-per-lane variant has 16384-element tiles
+    import random
+    import twg_capi
+    lib = twg_capi.load()
+    rng = random.Random(7)
+    lengths = [0, 1, 8191, 8192, 8193, (1 << 21) - 1, 1 << 21, (1 << 23) - 1, 1 << 23, (1 << 25) - 1,
+               1 << 25, (1 << 25) + 131071, 1 << 28, (1 << 30), (1 << 31) + 4099]
+    lengths += [rng.randrange(1, 1 << 32) for _ in range(2000)]
+    for n in lengths:
+        have = lib.twg_masked_select_scratch_bytes(n)
+        small = -(-n // 8192)
+        scalar = -(-n // 16384)
+        need = max(small, scalar)
+        if n >= 1 << 21:
+            tile = 131072 if n >= 1 << 25 else 65536 if n >= 1 << 23 else 16384
+            need = max(need, (n // tile) * 4 + -(-(n % tile) // 8192))
+        assert have >= 256 + 8 * need, (n, have, need)
+        assert have % 8 == 0
+
+
 HOT_PATH_OPS = [
     "empty.memory_format", "empty_strided", "as_strided", "resize_", "view", "_reshape_alias",
     "copy_", "_copy_from", "_copy_from_and_resize",
