@@ -64,8 +64,8 @@ def test_error_strings_without_gpu():
 def test_masked_select_scratch_covers_every_launch_variant():
     # what the host side clears before a launch (twg_masked_select.hip): a 256-byte header and
     # one 8-byte status word per 8192-element tile of the tile variant, or, from 2^21 elements,
-    # four words per streaming tile (16384 / 65536 / 131072 elements) plus one per 8192-element
-    # tile of the remainder launch; the one-element-per-lane variant has 16384-element tiles
+    # four words per streaming tile (16384 / 65536 / 131072 elements, the last one possibly
+    # incomplete); the one-element-per-lane variant has 16384-element tiles
     import random
     import twg_capi
     lib = twg_capi.load()
@@ -80,7 +80,7 @@ def test_masked_select_scratch_covers_every_launch_variant():
         need = max(small, scalar)
         if n >= 1 << 21:
             tile = 131072 if n >= 1 << 25 else 65536 if n >= 1 << 23 else 16384
-            need = max(need, (n // tile) * 4 + -(-(n % tile) // 8192))
+            need = max(need, -(-n // tile) * 4)
         assert have >= 256 + 8 * need, (n, have, need)
         assert have % 8 == 0
 

@@ -651,7 +651,7 @@ def test_masked_select_every_element_size(twg, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int64, torch.float64])
 def test_masked_select_fast_kernels_every_element_size(twg, dtype):
-    # the streaming kernel (all three tile sizes, with a remainder launch) and the tile variant
+    # the streaming kernel (all three tile sizes, with an incomplete last tile) and the tile variant
     # for 1-, 2- and 8-byte elements: dense and sparse masks, runs, shifted output pointers
     g = torch.Generator().manual_seed(35)
     es = torch.empty(0, dtype=dtype).element_size()
@@ -828,9 +828,8 @@ def test_masked_select_bernoulli(twg, n, p):
     (1 << 21, 0.5, 1)])
 def test_masked_select_large_tiles(twg, n, p, out_offset):
     # From 2^21 elements the streaming kernel runs (16384-, 65536- and, from 2^25,
-    # 131072-element tiles); a remainder below one of its tiles goes to a second launch
-    # that continues from the first one's count.  A shifted output pointer moves every
-    # wavefront's first and last line.
+    # 131072-element tiles), its last tile bounds-checked.  A shifted output pointer moves
+    # every wavefront's first and last line.
     _say(f"masked_select large n={n} p={p} out_offset={out_offset}")
     x = W.select_source(n, seed=4)
     if p < 0:

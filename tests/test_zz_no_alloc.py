@@ -47,7 +47,7 @@ def _both(twg, L, n, p, seed):
 def test_static_scratch_matches_allocated_scratch(twg):
     L = twg.load()
     print("static masked_select: 2^22+12345 elements, then 70001", flush=True)
-    # streaming kernel plus remainder launch (tickets, carry and thousands of status words
+    # streaming kernel with an incomplete last tile (the ticket and thousands of status words
     # are left behind) ...
     _both(twg, L, (1 << 22) + 12345, 0.5, 1)
     # ... then a smaller input that reuses the front of the same array

@@ -1038,7 +1038,7 @@ struct SelectStudy {
     float ms = 0;
     int rc = tm.run([&] {
       (void)hipMemsetAsync(scratch, 0, clear, tm.s);
-      ms_compact_stream<16, 4, STAGES><<<(unsigned)nb, 1024, 0, tm.s>>>(out, cnt, src, mask, (uint32_t)nb,
+      ms_compact_stream<16, 4, STAGES><<<(unsigned)nb, 1024, 0, tm.s>>>(out, cnt, src, mask, n, (uint32_t)nb,
                                                                         ticket, status);
     }, &ms);
     if (rc) return rc;
@@ -1166,7 +1166,7 @@ struct SelectStudy {
     constexpr int64_t kFull = 256 * 8 * 4 * 16;
     const int64_t nbf = n / kFull;
     (void)hipMemsetAsync(scratch, 0, kMsHeaderBytes + 8 * (size_t)nbf * kStreamStatusStride, tm.s);
-    ms_compact_stream<16, 4, 5><<<(unsigned)nbf, 1024, 0, tm.s>>>(out, cnt, src, mask, (uint32_t)nbf, ticket,
+    ms_compact_stream<16, 4, 5><<<(unsigned)nbf, 1024, 0, tm.s>>>(out, cnt, src, mask, n, (uint32_t)nbf, ticket,
                                                                  status);
     if ((rc = checksum(want, &href))) return rc;
     *ok = (k == want && h == href) ? 1 : 0;
@@ -1223,7 +1223,7 @@ struct SelectStudy {
         constexpr int64_t kFull = 256 * 8 * 4 * 16;
         const int64_t nbf = n / kFull;
         (void)hipMemsetAsync(scratch, 0, kMsHeaderBytes + 8 * (size_t)nbf * kStreamStatusStride, tm.s);
-        ms_compact_stream<16, 4, 5><<<(unsigned)nbf, 1024, 0, tm.s>>>(out, cnt, src, mask, (uint32_t)nbf, ticket,
+        ms_compact_stream<16, 4, 5><<<(unsigned)nbf, 1024, 0, tm.s>>>(out, cnt, src, mask, n, (uint32_t)nbf, ticket,
                                                                      status);
         if ((rc = checksum(want, &href))) return rc;
       }

@@ -15,8 +15,7 @@ namespace {
 // Tile shapes of the fast variants.  The streaming kernel wants about one tile per CU
 // or more and as few tickets as that allows: 131072-element tiles from 2^25 elements,
 // 65536 from 2^23, 16384 from 2^21 (measured: each is 1.2-1.8x faster in its range than
-// its neighbours); 8192-element tiles of the stage-then-write variant below that and
-// for what the big tiles leave over.
+// its neighbours); 8192-element tiles of the stage-then-write variant below that.
 constexpr int kSmallWaves = 4;
 constexpr int64_t kSmallTile = (int64_t)kWaveElems * kSmallWaves;
 constexpr int64_t kStreamMinElems = int64_t(1) << 21;
@@ -28,35 +27,24 @@ struct MsLaunch {
   const T *src;
   const uint8_t *mask;
   int64_t numel;
-  uint32_t *ticket;  // [0] streaming launch, [1] remainder launch
-  int64_t *carry;    // count handed from the first launch to the second
+  uint32_t *ticket;
   uint64_t *status;
   void *scratch;
   twg_stream_t stream;
 };
 
-// Full tiles go through the streaming kernel; what is left (less than one of its tiles)
-// is compacted by a second launch of the tile variant that starts from the first
-// launch's total.
+// One launch of the streaming kernel; its last tile may be incomplete.
 template <int WAVES, int GROUPS, typename T>
 int launch_stream(const MsLaunch<T> &m) {
   constexpr int64_t kTile = (int64_t)256 * 8 * GROUPS * WAVES;
-  const int64_t nbig = m.numel / kTile;
-  const int64_t rem = m.numel - nbig * kTile;
-  const int64_t nrem = (rem + kSmallTile - 1) / kSmallTile;
-  if (nbig > INT32_MAX) return TWG_E_UNSUPPORTED;
-  // status words: the big tiles' first, kStreamStatusStride apart, then the remainder's
-  const size_t big_words = (size_t)nbig * kStreamStatusStride;
-  int rc = twg_fill_bytes(m.scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * (big_words + (size_t)nrem),
-                          m.stream);
+  const int64_t ntiles = (m.numel + kTile - 1) / kTile;
+  if (ntiles > INT32_MAX) return TWG_E_UNSUPPORTED;
+  // status words kStreamStatusStride apart
+  const size_t words = (size_t)ntiles * kStreamStatusStride;
+  int rc = twg_fill_bytes(m.scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * words, m.stream);
   if (rc) return rc;
-  hipStream_t s = resolve_stream(m.stream);
-  ms_compact_stream<WAVES, GROUPS, 5, T><<<(unsigned)nbig, WAVES * 64, 0, s>>>(
-      m.out, rem ? m.carry : m.d_count, m.src, m.mask, (uint32_t)nbig, m.ticket, m.status);
-  if (rem)
-    ms_compact_vec<kSmallWaves, T><<<(unsigned)nrem, kSmallWaves * 64, 0, s>>>(
-        m.out, m.d_count, m.src + nbig * kTile, m.mask + nbig * kTile, rem, (uint32_t)nrem,
-        m.ticket + 1, m.status + big_words, m.carry);
+  ms_compact_stream<WAVES, GROUPS, 5, T><<<(unsigned)ntiles, WAVES * 64, 0, resolve_stream(m.stream)>>>(
+      m.out, m.d_count, m.src, m.mask, m.numel, (uint32_t)ntiles, m.ticket, m.status);
   return (int)hipGetLastError();
 }
 
@@ -65,15 +53,13 @@ int launch_stream(const MsLaunch<T> &m) {
 template <typename T>
 int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t *mask, int64_t numel,
                 void *scratch, twg_stream_t stream) {
-  // scratch: [0] ticket, [4] ticket of the remainder launch, [8] carry between the
-  // two launches, [256...] one status word per tile
+  // scratch: [0] ticket, [256...] the tiles' status words
   uint32_t *ticket = static_cast<uint32_t *>(scratch);
-  int64_t *carry = reinterpret_cast<int64_t *>(static_cast<char *>(scratch) + 8);
   uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
   T *out = static_cast<T *>(out_v);
   const T *src = static_cast<const T *>(src_v);
   if (numel >= kStreamMinElems) {
-    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, carry, status, scratch, stream};
+    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, status, scratch, stream};
     if (numel >= (int64_t(1) << 25)) return launch_stream<16, 4>(m);
     if (numel >= (int64_t(1) << 23)) return launch_stream<16, 2>(m);
     return launch_stream<8, 1>(m);
@@ -86,7 +72,7 @@ int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t 
       (rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
     return rc;
   ms_compact_vec<kSmallWaves, T><<<ntiles, kSmallWaves * 64, 0, resolve_stream(stream)>>>(
-      out, d_count, src, mask, numel, ntiles, ticket, status, nullptr);
+      out, d_count, src, mask, numel, ntiles, ticket, status);
   return (int)hipGetLastError();
 }
 
@@ -187,7 +173,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
 }  // namespace twg
 
 // ------------------------------------------------- scratch that is never allocated
-// Tickets, carry and status words of twg_masked_select_f32_static live in this array
+// Tickets and status words of twg_masked_select_f32_static live in this array
 // instead of a buffer the caller allocates.  The name below is a host-side handle, not a
 // device address: the address each device gives its copy is looked up once per device
 // (static_scratch_setup, run by the library's init) and only that pointer is ever handed

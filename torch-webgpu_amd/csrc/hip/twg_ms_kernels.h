@@ -53,11 +53,10 @@ constexpr int kScalarSteps = 16;    //   16 wavefronts x 16 steps of 64 elements
 constexpr int kScalarTile = 64 * kScalarWaves * kScalarSteps;
 constexpr int kMsMinTile = 256 * kSteps * 4;  // smallest tile of any variant (ms_compact_vec<4>)
 static_assert(kScalarTile >= kMsMinTile, "the scratch is sized for kMsMinTile-element tiles");
-constexpr size_t kMsHeaderBytes = 256;                  // tickets and carry, padded
+constexpr size_t kMsHeaderBytes = 256;                  // the ticket, padded
 // Smallest tile of the streaming variant (8 wavefronts x 8 steps x 256 elements) and the
 // status words the scratch must hold: one per kMsMinTile elements for the small-tile
-// variants, or kStreamStatusStride per streaming tile plus the few tiles of its remainder
-// launch (less than one streaming tile, at most 16 small tiles).
+// variants, or kStreamStatusStride per streaming tile, the incomplete last one included.
 constexpr int64_t kStreamMinTile = 8 * 2048;
 constexpr size_t ms_scratch_bytes(int64_t numel) {
   if (numel < 0) numel = 0;
@@ -175,12 +174,11 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
 
 // Aggregate, look-back, inclusive prefix: the part every variant shares.  Call
 // with all threads; returns the tile's exclusive prefix to all of them.  s_slot is
-// one int64 of LDS.  The last tile also writes the grand total, plus *carry_in if a
-// previous launch compacted the elements before this one's.
+// one int64 of LDS.  The last tile also writes the grand total.
 template <int LPL = kLookPerLane, int STRIDE = 1>
 __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, uint32_t ntiles,
                                                uint32_t tile_total, int64_t *d_count,
-                                               int64_t *s_slot, const int64_t *carry_in) {
+                                               int64_t *s_slot) {
   const int lane = threadIdx.x & 63;
   if (threadIdx.x < 64) {  // wave 0
     uint64_t *mine = status + (size_t)tile * STRIDE;
@@ -196,7 +194,7 @@ __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, 
       // One 8-byte store at system scope: the count may live in host memory that the
       // host polls while the rest of the grid is still compacting.
       if (tile == ntiles - 1)
-        __hip_atomic_store(d_count, exclusive + (int64_t)tile_total + (carry_in ? *carry_in : 0),
+        __hip_atomic_store(d_count, exclusive + (int64_t)tile_total,
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
@@ -258,9 +256,9 @@ struct Quad<uint8_t> {
   }
 };
 
-// ---- streaming variant: full tiles only (the host launches it on a multiple of the
-// tile size, so it carries no bounds checks).  Wavefront w owns GROUPS * 8
-// consecutive steps of the tile.
+// ---- streaming variant.  Wavefront w owns GROUPS * 8 consecutive steps of the tile.  Only
+// the last tile may be incomplete: its mask loads are bounds-checked, and since a lane
+// without a selected element never touches the source nothing else needs to know.
 constexpr int kRingElems = 512;  // per wavefront; at most a line less one element + 256 values wait in it
 // Source steps in flight per wavefront.  4 measured best: 8 keeps more in flight than
 // the memory system rewards (dense masks lose 2-3%), and below ~64 VGPRs a second
@@ -294,7 +292,7 @@ struct MsStreamShared {
 template <int WAVES, int GROUPS, int STAGES = 5, typename T = float>
 __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t *d_count,
                                                                 const T *src,
-                                                                const uint8_t *mask,
+                                                                const uint8_t *mask, int64_t n,
                                                                 uint32_t ntiles, uint32_t *ticket,
                                                                 uint64_t *status) {
   constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
@@ -317,18 +315,42 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
 
   // ---- 1. masks -> packed selection bits in LDS, wavefront totals
   uint32_t cnt = 0;
+  const bool whole = (int64_t)(tile + 1) * kTileElems <= n;  // workgroup-uniform
+  if (whole) {
 #pragma unroll 2
-  for (int g = 0; g < GROUPS; ++g) {
-    uint32_t w[8];
+    for (int g = 0; g < GROUPS; ++g) {
+      uint32_t w[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
-      w[k] = __builtin_nontemporal_load(
-          reinterpret_cast<const uint32_t *>(mask_w + (g * 8 + k) * 256));
-    uint32_t b = 0;
+      for (int k = 0; k < 8; ++k)
+        w[k] = __builtin_nontemporal_load(
+            reinterpret_cast<const uint32_t *>(mask_w + (g * 8 + k) * 256));
+      uint32_t b = 0;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) b |= select_bits(w[k]) << (4 * k);
-    sh.bits[g][threadIdx.x] = b;
-    cnt += __popc(b);
+      for (int k = 0; k < 8; ++k) b |= select_bits(w[k]) << (4 * k);
+      sh.bits[g][threadIdx.x] = b;
+      cnt += __popc(b);
+    }
+  } else {  // the last tile: elements from n on count as not selected
+    const int64_t left = n - (start + lane * 4);  // elements from this lane's first one on
+#pragma unroll 1
+    for (int g = 0; g < GROUPS; ++g) {
+      uint32_t b = 0;
+#pragma unroll 1
+      for (int k = 0; k < 8; ++k) {
+        const int64_t have = left - (int64_t)(g * 8 + k) * 256;
+        const uint8_t *m = mask_w + (g * 8 + k) * 256;
+        uint32_t w = 0;
+        if (have >= 4) {
+          w = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(m));
+        } else {
+          for (int j = 0; j < 4; ++j)
+            if (j < have && m[j]) w |= 1u << (8 * j);
+        }
+        b |= select_bits(w) << (4 * k);
+      }
+      sh.bits[g][threadIdx.x] = b;
+      cnt += __popc(b);
+    }
   }
   const uint32_t wt = wave_sum_u32(cnt);
   if (lane == 0) sh.wave_total[wave] = wt;
@@ -347,7 +369,9 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
   }
 
   // ---- 2. the first kDepth steps' values go in flight, then aggregate / look-back
-  const T *dummy = src + (int64_t)tile * kTileElems;
+  // (a lane with nothing selected reads the tile's first four elements; in an incomplete
+  // last tile those may not all exist, so there it reads the array's first four)
+  const T *dummy = whole ? src + (int64_t)tile * kTileElems : src;
   auto fetch = [&](uint32_t four_bits, int step) {
     return Quad<T>::load(four_bits ? src_w + step * 256 : dummy);
   };
@@ -362,7 +386,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
   }
   const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(
-      status, tile, ntiles, tile_total, d_count, &sh.base, nullptr);
+      status, tile, ntiles, tile_total, d_count, &sh.base);
   if constexpr (STAGES < 4) {
     uint32_t acc = 0;
 #pragma unroll
@@ -504,8 +528,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
                                                              const T *src,
                                                              const uint8_t *mask, int64_t n,
                                                              uint32_t ntiles, uint32_t *ticket,
-                                                             uint64_t *status,
-                                                             const int64_t *carry_in) {
+                                                             uint64_t *status) {
   constexpr int64_t kTileElems = (int64_t)kWaveElems * WAVES;
   constexpr uint32_t kSlot = 16u / sizeof(T);  // elements per 16-byte store
   __shared__ MsShared<WAVES, T> sh;
@@ -525,7 +548,6 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
   const uint32_t lane_off = wave * kWaveElems + lane * 4;
   const int64_t left = n - start;
   const uint32_t remaining = left < kTileElems ? (uint32_t)left : (uint32_t)kTileElems;
-  if (carry_in) out += *carry_in;
 
   // ---- 1. mask -> packed selection bits (bit 4k+j <=> element j of step k) and totals
   uint32_t w[kSteps];
@@ -567,7 +589,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
       }
     }
   }
-  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base, carry_in);
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base);
 
   // ---- 3. compact in LDS, write aligned 16-byte packs; the ragged ends go out element by
   //         element: their neighbours belong to other wavefronts.
@@ -678,7 +700,7 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
 #pragma unroll
   for (int k = 0; k < kScalarSteps; ++k)
     if (sel[k]) vals[k] = src[soff[k]];
-  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &s_base, nullptr);
+  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &s_base);
   const int64_t wpos = base + wave_base;
 #pragma unroll
   for (int k = 0; k < kScalarSteps; ++k)
