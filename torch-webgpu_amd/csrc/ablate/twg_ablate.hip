@@ -578,6 +578,112 @@ __global__ __launch_bounds__(256) void counters_ahead_of_movers(float *out, int6
 }
 
 
+// The streaming kernel's tile body in a persistent grid with a static tile order: `grid`
+// co-resident workgroups, workgroup w compacts tiles w, w + grid, w + 2 grid, ...  No ticket:
+// a tile only waits on lower tiles, which belong to workgroups that are resident too and at
+// the same round or an earlier one.  Dense path only (no gather path for sparse wavefronts).
+template <int WAVES, int GROUPS>
+__global__ __launch_bounds__(WAVES * 64) void static_order_persistent(float *out, int64_t *d_count,
+                                                                      const float *src,
+                                                                      const uint8_t *mask,
+                                                                      uint32_t ntiles,
+                                                                      uint64_t *status) {
+  constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
+  constexpr int64_t kTileElems = (int64_t)kWaveSpan * WAVES;
+  __shared__ MsStreamShared<WAVES, GROUPS, float> sh;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const int64_t start = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
+    const uint8_t *mask_w = mask + start + lane * 4;
+    const float *src_w = src + start + lane * 4;
+    uint32_t cnt = 0;
+#pragma unroll 2
+    for (int g = 0; g < GROUPS; ++g) {
+      uint32_t w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        w[k] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(mask_w + (g * 8 + k) * 256));
+      uint32_t b = 0;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) b |= select_bits(w[k]) << (4 * k);
+      sh.bits[g][threadIdx.x] = b;
+      cnt += __popc(b);
+    }
+    const uint32_t wt = wave_sum_u32(cnt);
+    if (lane == 0) sh.wave_total[wave] = wt;
+    __syncthreads();
+    uint32_t wbase = 0, tile_total = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const uint32_t t = sh.wave_total[w];
+      if ((uint32_t)w < wave) wbase += t;
+      tile_total += t;
+    }
+    const f32x4 *dummy = reinterpret_cast<const f32x4 *>(src + (int64_t)tile * kTileElems);
+    auto fetch = [&](uint32_t four_bits, int step) {
+      const f32x4 *p = reinterpret_cast<const f32x4 *>(src_w + step * 256);
+      return __builtin_nontemporal_load(four_bits ? p : dummy);
+    };
+    uint32_t b_cur = sh.bits[0][threadIdx.x];
+    f32x4 vals[kDepth];
+#pragma unroll
+    for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
+    const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(status, tile, ntiles, tile_total,
+                                                                             d_count, &sh.base);
+    float *ring = reinterpret_cast<float *>(sh.ring[wave]);
+    float *wout = out + (base + wbase);
+    const uint32_t shift = (uint32_t)((reinterpret_cast<uintptr_t>(wout) >> 2) & 31u);
+    float *obase = wout - shift;
+    uint32_t run = shift;
+    uint32_t flushed = shift ? 8u : 0u;
+#pragma unroll 1
+    for (int g = 0; g < GROUPS; ++g) {
+      const int gn = (g + 1 < GROUPS) ? g + 1 : g;
+      const uint32_t b_next = (g + 1 < GROUPS) ? sh.bits[gn][threadIdx.x] : 0u;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t f = (b_cur >> (4 * k)) & 0xFu;
+        uint32_t below, total;
+        wave_offsets(__popc(f), below, total);
+        const f32x4 x4 = vals[k % kDepth];
+        {
+          const int ahead = k + kDepth;
+          vals[k % kDepth] = ahead < 8 ? fetch((b_cur >> (4 * ahead)) & 0xFu, g * 8 + ahead)
+                                       : fetch((b_next >> (4 * (ahead - 8))) & 0xFu, gn * 8 + ahead - 8);
+        }
+        if (f) {
+          uint32_t pos = run + below;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (f & (1u << j)) {
+              const float x = x4[j];
+              ring[pos & (kRingElems - 1)] = x;
+              if (pos < 32u && shift) obase[pos] = x;
+              ++pos;
+            }
+          }
+        }
+        run += total;
+        const uint32_t end4 = (run >> 5) << 3;
+        if (end4 > flushed) {
+          __builtin_amdgcn_wave_barrier();
+          for (uint32_t idx = flushed + lane; idx < end4; idx += 64) {
+            const f32x4 x = *reinterpret_cast<const f32x4 *>(ring + ((4 * idx) & (kRingElems - 1)));
+            __builtin_nontemporal_store(x, reinterpret_cast<f32x4 *>(obase + 4 * (size_t)idx));
+          }
+          flushed = end4;
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+      b_cur = b_next;
+    }
+    for (uint32_t p = 4 * flushed + lane; p < run; p += 64) obase[p] = ring[p & (kRingElems - 1)];
+    __syncthreads();  // the selection bits, totals and base in LDS are rewritten by the next round
+  }
+}
+
+
 // One-shot workgroups like the streaming kernel's, but SWAVES wavefronts stream and one more,
 // the last, owns no elements: it publishes the tile's aggregate, looks back and hands the
 // tile's base to the others through LDS.  The streaming wavefronts do not wait for it:
@@ -1116,6 +1222,41 @@ struct SelectStudy {
     return 0;
   }
 
+  // the streaming tile body in a persistent grid of `per_cu` workgroups per CU, static order
+  int static_order(int per_cu) {
+    constexpr int64_t kTile = 256 * 8 * 4 * 16;
+    const int64_t nb = n / kTile;
+    if (nb * kTile != n) return 0;
+    uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
+    const size_t clear = kMsHeaderBytes + 8 * (size_t)nb * kStreamStatusStride;
+    if (clear > scratch_bytes) return -1;
+    auto kern = static_order_persistent<16, 4>;
+    int occ = 0;
+    TWGA_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, 1024, 0));
+    if (occ < per_cu) return 0;  // would not be co-resident: the static order could deadlock
+    hipDeviceProp_t prop;
+    TWGA_TRY(hipGetDeviceProperties(&prop, 0));
+    int64_t grid = (int64_t)per_cu * prop.multiProcessorCount;
+    if (grid > nb) grid = nb;
+    TWGA_TRY(hipMemsetAsync(out, 0, (size_t)n * 4, tm.s));
+    float ms = 0;
+    int rc = tm.run([&] {
+      (void)hipMemsetAsync(scratch, 0, clear, tm.s);
+      kern<<<(unsigned)grid, 1024, 0, tm.s>>>(out, cnt, src, mask, (uint32_t)nb, status);
+    }, &ms);
+    if (rc) return rc;
+    int64_t k = -1;
+    TWGA_TRY(hipMemcpyAsync(&k, cnt, 8, hipMemcpyDeviceToHost, tm.s));
+    TWGA_TRY(hipStreamSynchronize(tm.s));
+    unsigned long long h = 0;
+    if ((rc = checksum(k, &h))) return rc;
+    char name[96];
+    std::snprintf(name, sizeof(name), "persistent, static tile order: %ld workgroups of 16 wavefronts, no ticket",
+                  (long)grid);
+    put(res, name, ms, bytes_of(n, k), (k == k_ref && h == sum_ref) ? 1 : 0);
+    return 0;
+  }
+
   template <int S, bool WAIT_FIRST>
   int run_ahead() {
     constexpr int64_t kTile = 256 * 8 * 4 * S;
@@ -1338,6 +1479,7 @@ int twga_masked_select(int log2n, float p, twga_result_t *out, int cap) {
   TWGA_STEP((st.small_tiles<16, 4>()));
   TWGA_STEP((st.counters_ahead<512>(reinterpret_cast<uint64_t *>(st.bases))));
   TWGA_STEP((st.counters_ahead<8192>(reinterpret_cast<uint64_t *>(st.bases))));
+  TWGA_STEP(st.static_order(1));
   TWGA_STEP((st.run_ahead<15, true>()));
   TWGA_STEP((st.run_ahead<15, false>()));
   TWGA_STEP((st.front_wave<15, 4, 3>()));
