@@ -393,8 +393,9 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
 def ablations(log2n):
     """The experiments the kernel shapes rest on, from the ablation library (built by
     `python torch-webgpu_amd/build.py ablate`; not part of the product): copies of 2^log2n floats
-    in every launch shape considered for the streaming kernels, and masked_select cut off phase
-    by phase and rebuilt in two other structures.  % of 8 TB/s on algorithmic bytes."""
+    in every launch shape considered for the streaming kernels, the transposed add in other tile
+    shapes, and masked_select cut off phase by phase and rebuilt in other structures.  % of
+    8 TB/s on algorithmic bytes."""
     path = os.path.join(ROOT, "torch-webgpu_amd", "torch_webgpu", "libtwg_ablate.so")
     if not os.path.exists(path):
         raise SystemExit(f"{path} is missing: build it with `python torch-webgpu_amd/build.py ablate`")
@@ -426,6 +427,9 @@ def ablations(log2n):
     res = {"elements": 1 << log2n}
     log(f"copy of 2^{log2n} floats (4 B read + 4 B written per element) by launch shape")
     res["copy_shapes"] = rows(A.twga_copy_shapes(log2n, buf, cap))
+    A.twga_transposed_add.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(Result), ctypes.c_int]
+    log("transposed add, out[8192][32768] = a + c^T with c stored [32768][8192] (12 B per element), by tile shape")
+    res["transposed_add"] = rows(A.twga_transposed_add(8192, 32768, buf, cap))
     res["masked_select"] = {}
     for p in (0.5, 0.99, 0.01):
         log(f"masked_select of 2^{log2n} floats, Bernoulli({p}) mask: ms of each form; % of peak on the "

@@ -13,6 +13,10 @@
 //                         and persistent workgroups with a front wavefront that prepares the
 //                         next tile while the others stream the current one
 //
+//   twga_transposed_add   out[i][j] = a[i][j] + c[j][i] (the transposed operand read along its
+//                         own rows) with the library's tile kernel in other tile shapes
+//                         and block sizes than the one the library launches
+//
 // Every kernel touches [0, n) of its buffers only; tile sizes divide what they are run on
 // (the host checks) and every wait inside a kernel is bounded.
 #include <hip/hip_runtime.h>
@@ -22,6 +26,7 @@
 #include <cstring>
 #include <vector>
 
+#include "../hip/twg_ew.h"
 #include "../hip/twg_ms_kernels.h"
 
 extern "C" {
@@ -1378,6 +1383,63 @@ struct SelectStudy {
   }
 };
 
+// ------------------------------------------------------------- transposed add
+
+struct AblAdd {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+
+struct TransposeStudy {
+  float *a = nullptr, *c = nullptr, *out = nullptr, *ref = nullptr;
+  uint32_t *bad = nullptr;
+  int64_t rows = 0, cols = 0;  // out and a are [rows][cols]; c is stored [cols][rows]
+  Timer tm;
+  std::vector<twga_result_t> res;
+
+  template <int TD0, int TT, int THREADS>
+  int shape(bool baseline) {
+    if (cols % TD0 != 0 || rows % TT != 0) return 0;
+    TileGeom g{};
+    g.n0 = cols;
+    g.nt = rows;
+    g.s0[0] = 1;
+    g.st[0] = cols;  // out
+    g.s0[1] = 1;
+    g.st[1] = cols;  // a
+    g.s0[2] = rows;
+    g.st[2] = 1;     // c: unit stride along t
+    g.psplit = 1;
+    g.tiles0 = (uint32_t)(cols / TD0);
+    g.tilest = (uint32_t)(rows / TT);
+    g.nbatch = 0;
+    const int64_t blocks = (int64_t)g.tiles0 * g.tilest;
+    if (blocks > 0x7FFFFFFF) return 0;
+    float *dst = baseline ? ref : out;
+    TWGA_TRY(hipMemsetAsync(dst, 0, (size_t)rows * cols * 4, tm.s));
+    float ms = 0;
+    int rc = tm.run([&] {
+      ew_tile_vec<2, false, true, TD0, TT, AblAdd, float, float, float, THREADS>
+          <<<(unsigned)blocks, THREADS, 0, tm.s>>>(dst, a, c, g, AblAdd{});
+    }, &ms);
+    if (rc) return rc;
+    int ok = 1;
+    if (!baseline) {
+      const int64_t n = rows * cols;
+      TWGA_TRY(hipMemsetAsync(bad, 0, 4, tm.s));
+      count_differences<<<(unsigned)((n + 255) / 256), 256, 0, tm.s>>>(out, ref, n, bad);
+      uint32_t h = 1;
+      TWGA_TRY(hipMemcpyAsync(&h, bad, 4, hipMemcpyDeviceToHost, tm.s));
+      TWGA_TRY(hipStreamSynchronize(tm.s));
+      ok = h == 0;
+    }
+    char name[96];
+    std::snprintf(name, sizeof(name), "tiles of %d (output rows) x %d (operand rows), %d lanes%s", TD0, TT,
+                  THREADS, baseline ? " - what the library launches" : "");
+    put(res, name, ms, 12.0 * (double)rows * (double)cols, ok);
+    return 0;
+  }
+};
+
 int copy_out(const std::vector<twga_result_t> &v, twga_result_t *out, int cap) {
   const int m = (int)v.size() < cap ? (int)v.size() : cap;
   for (int i = 0; i < m; ++i) out[i] = v[(size_t)i];
@@ -1495,6 +1557,48 @@ done:
   (void)hipFree(st.scratch);
   (void)hipFree(st.counts);
   (void)hipFree(st.bases);
+  (void)hipStreamDestroy(st.tm.s);
+  if (rc) return rc;
+  return copy_out(st.res, out, cap);
+}
+
+// out[rows][cols] = a + c^T with c stored [cols][rows], fp32: the library's tile kernel in
+// the shape it launches for this geometry and in others.
+int twga_transposed_add(int rows, int cols, twga_result_t *out, int cap) {
+  if (!out || rows < 1024 || cols < 1024 || rows % 1024 || cols % 1024 || (int64_t)rows * cols > (int64_t(1) << 30))
+    return -1;
+  TransposeStudy st;
+  st.rows = rows;
+  st.cols = cols;
+  const int64_t n = (int64_t)rows * cols;
+  int rc = st.tm.init();
+  if (rc) return rc;
+  TWGA_TRY(hipStreamCreateWithFlags(&st.tm.s, hipStreamNonBlocking));
+  TWGA_TRY(hipMalloc(&st.a, (size_t)n * 4));
+  TWGA_TRY(hipMalloc(&st.c, (size_t)n * 4));
+  TWGA_TRY(hipMalloc(&st.out, (size_t)n * 4));
+  TWGA_TRY(hipMalloc(&st.ref, (size_t)n * 4));
+  TWGA_TRY(hipMalloc(&st.bad, 4));
+  fill_pattern<<<(unsigned)((n + 255) / 256), 256, 0, st.tm.s>>>(st.a, n);
+  fill_pattern<<<(unsigned)((n + 255) / 256), 256, 0, st.tm.s>>>(st.c, n);
+  TWGA_STEP((st.shape<256, 32, 1024>(true)));
+  TWGA_STEP((st.shape<256, 32, 512>(false)));
+  TWGA_STEP((st.shape<256, 32, 256>(false)));
+  TWGA_STEP((st.shape<128, 32, 256>(false)));
+  TWGA_STEP((st.shape<64, 64, 256>(false)));
+  TWGA_STEP((st.shape<128, 64, 1024>(false)));
+  TWGA_STEP((st.shape<256, 64, 1024>(false)));
+  TWGA_STEP((st.shape<128, 128, 1024>(false)));
+  TWGA_STEP((st.shape<512, 32, 1024>(false)));
+  TWGA_STEP((st.shape<1024, 32, 1024>(false)));
+  TWGA_STEP((st.shape<256, 16, 1024>(false)));
+done:
+  (void)hipStreamSynchronize(st.tm.s);
+  (void)hipFree(st.a);
+  (void)hipFree(st.c);
+  (void)hipFree(st.out);
+  (void)hipFree(st.ref);
+  (void)hipFree(st.bad);
   (void)hipStreamDestroy(st.tm.s);
   if (rc) return rc;
   return copy_out(st.res, out, cap);
