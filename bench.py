@@ -56,9 +56,10 @@ def main():
     ap.add_argument("--geometries", action="store_true",
                     help="instead of the benchmark: time add over families of broadcast and permuted "
                          "operands (~2^25 elements each) and print their spread as one JSON line")
-    ap.add_argument("--ablations", action="store_true",
-                    help="instead of the benchmark: time the launch shapes and kernel structures the hot "
-                         "kernels were chosen from (libtwg_ablate.so) and print them as one JSON line")
+    ap.add_argument("--first-launches", action="store_true",
+                    help="instead of the benchmark: time 40 consecutive gelu launches one by one on buffers "
+                         "in different states (fresh from hipMalloc, filled once, recycled by the pool, after "
+                         "2 s of idle time) and print the series as one JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this op path is single-GPU (no collectives, nothing to shard in one "
@@ -75,8 +76,8 @@ def main():
     if args.geometries:
         print(json.dumps(geometry_families(capi, L)), flush=True)
         return
-    if args.ablations:
-        print(json.dumps(ablations(args.log2n)), flush=True)
+    if args.first_launches:
+        print(json.dumps(first_launches(capi, L, torch, 1 << args.log2n)), flush=True)
         return
     dev_name, cus, mem = capi.device_info()
     log(f"device: {dev_name}  CUs={cus}  mem={mem / 2**30:.0f} GiB")
@@ -114,13 +115,18 @@ def main():
     # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE + WRITE_SIZE, each scaled by a
     # transfer of known size); recorded figures, not re-measured by this run
     traffic = {}
+    traffic_source = None
     tr = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
     if os.path.exists(tr):
+        commit = "unknown commit"
         with open(tr) as f:
             for line in f:
-                if "=" in line and not line.startswith("#"):
+                if line.startswith("# measured at commit"):
+                    commit = line.split()[-1]
+                elif "=" in line and not line.startswith("#"):
                     k, v = line.split("=")
                     traffic[k.strip()] = int(v)
+        traffic_source = f"recorded: profiles/hbm_traffic.txt @ {commit} (not measured by this run)"
 
     def summarize(name, kernel, nbytes, ms_list, nelem, extra=None):
         avg = getattr(ms_list, "batch_avg", None) or sum(ms_list) / len(ms_list)
@@ -140,6 +146,7 @@ def main():
             # FETCH_SIZE + WRITE_SIZE): below the algorithmic figure where source lines
             # without a selected element are never fetched
             "traffic": moved,
+            "traffic_source": traffic_source if moved else None,
             "pct_hbm_peak_on_traffic": (round(moved / avg / 1e6 / HBM_PEAK_GBS * 100, 2)
                                         if moved else None),
         }
@@ -202,7 +209,15 @@ def main():
     step_bytes = bytes_add + bytes_gelu + bytes_ms
 
     # ------------------------------------------------------------ timed steps
-    log(f"timing {K} steps after {Wm} warm-up steps ...")
+    # A GPU that has been idle (here: while the host generated and uploaded the inputs) runs
+    # its first 2-3 ms of work at full rate, then 10-20% slower for about 4 ms, then settles
+    # (profiles/first_launches_after_idle_gelu_2p28.md: the same on buffers that were never
+    # touched, filled once, or recycled, and again after any 2 s pause).  Forty untimed gelu
+    # launches (13 ms) put that transient behind the run before the W warm-up steps start.
+    settle = 40
+    for _ in range(settle):
+        run_gelu()
+    log(f"timing {K} steps after {settle} settling launches and {Wm} warm-up steps ...")
     for _ in range(Wm):
         run_add(); run_gelu(); assert run_ms() == k50
     capi.sync()
@@ -244,6 +259,7 @@ def main():
         "avg_launch_ms": dominant["avg_ms"],
     }
     roofline["traffic"] = dominant["traffic"]
+    roofline["traffic_source"] = dominant["traffic_source"]
     roofline["frac_on_traffic"] = (round(dominant["pct_hbm_peak_on_traffic"] / 100, 4)
                                    if dominant["traffic"] else None)
 
@@ -282,6 +298,7 @@ def main():
     out = {
         "metric": "HBM GB/s (% of peak) for add/gelu/masked_select at 2^28 fp32, 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": Wm,
+        "settle_launches_before_warmup": settle,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"one step = add.Tensor + gelu(approximate='none') + masked_select"
@@ -347,8 +364,9 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
     res = []
 
     def line(name, fn, nbytes, ref_ms):
-        # freshly allocated device memory is slower on its first few passes (the driver maps
-        # it on first touch), and these legs upload their own operands: warm up longer
+        # these legs upload their own operands, and after the idle time of an upload the GPU's
+        # first 7 ms of work hold a slow stretch (see the note at the timed steps): warm up
+        # past it
         ms = time_launches(fn, max(Wm, 2 * K), K)
         avg = ms.batch_avg
         d = {"op": name, "avg_ms": round(avg, 5), "GBps": round(nbytes / avg / 1e6, 1),
@@ -390,52 +408,57 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
     return res
 
 
-def ablations(log2n):
-    """The experiments the kernel shapes rest on, from the ablation library (built by
-    `python torch-webgpu_amd/build.py ablate`; not part of the product): copies of 2^log2n floats
-    in every launch shape considered for the streaming kernels, the transposed add in other tile
-    shapes, and masked_select cut off phase by phase and rebuilt in other structures.  % of
-    8 TB/s on algorithmic bytes."""
-    path = os.path.join(ROOT, "torch-webgpu_amd", "torch_webgpu", "libtwg_ablate.so")
-    if not os.path.exists(path):
-        raise SystemExit(f"{path} is missing: build it with `python torch-webgpu_amd/build.py ablate`")
-    A = ctypes.CDLL(path)
+def first_launches(capi, L, torch, n, launches=40):
+    """Is the first pass over freshly allocated device memory slower?  Times `launches`
+    consecutive gelu launches on n floats, each between its own pair of events, with the output
+    (and input) buffer in different states.  Microseconds per launch, in launch order."""
+    it = capi.dense_iter(n)
+    series = []
 
-    class Result(ctypes.Structure):
-        _fields_ = [("name", ctypes.c_char * 96), ("ms", ctypes.c_float), ("bytes", ctypes.c_double),
-                    ("ok", ctypes.c_int32)]
+    def run(label, din, dout):
+        evs = [capi.Event() for _ in range(launches + 1)]
+        evs[0].record()
+        for i in range(launches):
+            capi.check(L.twg_unary_f32(capi.UNARY_GELU_ERF, dout.ptr, din.ptr, ctypes.byref(it), None))
+            evs[i + 1].record()
+        evs[-1].sync()
+        us = [round(evs[i].elapsed_ms(evs[i + 1]) * 1000) for i in range(launches)]
+        log(f"  {label:64s} " + " ".join(str(x) for x in us))
+        series.append({"state": label, "us": us})
 
-    cap = 64
-    buf = (Result * cap)()
-    A.twga_copy_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(Result), ctypes.c_int]
-    A.twga_masked_select.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.POINTER(Result), ctypes.c_int]
-
-    def rows(count, with_pct=True):
-        if count < 0:
-            raise RuntimeError(f"ablation library returned {count}")
-        out = []
-        for r in buf[:count]:
-            d = {"what": r.name.decode(), "ms": round(r.ms, 4),
-                 "verified": {1: True, 0: False}.get(r.ok)}
-            if with_pct:
-                d["pct_hbm_peak"] = round(r.bytes / r.ms / 1e6 / HBM_PEAK_GBS * 100, 1)
-            log(f"  {d['what']:84s} {d['ms']:8.4f} ms" + (f"  {d['pct_hbm_peak']:5.1f}%" if with_pct else "")
-                + ("" if d["verified"] is not False else "  OUTPUT DIFFERS"))
-            out.append(d)
-        return out
-
-    res = {"elements": 1 << log2n}
-    log(f"copy of 2^{log2n} floats (4 B read + 4 B written per element) by launch shape")
-    res["copy_shapes"] = rows(A.twga_copy_shapes(log2n, buf, cap))
-    A.twga_transposed_add.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(Result), ctypes.c_int]
-    log("transposed add, out[8192][32768] = a + c^T with c stored [32768][8192] (12 B per element), by tile shape")
-    res["transposed_add"] = rows(A.twga_transposed_add(8192, 32768, buf, cap))
-    res["masked_select"] = {}
-    for p in (0.5, 0.99, 0.01):
-        log(f"masked_select of 2^{log2n} floats, Bernoulli({p}) mask: ms of each form; % of peak on the "
-            "full op's algorithmic bytes (meaningful for the complete forms only)")
-        res["masked_select"][f"p{p}"] = rows(A.twga_masked_select(log2n, ctypes.c_float(p), buf, cap))
-    return res
+    for rep in range(2):
+        capi.check(L.twg_empty_cache())
+        din = capi.DeviceBuffer(4 * n)
+        capi.check(L.twg_fill_bytes(din.ptr, 0x3c, 4 * n, None))
+        dout = capi.DeviceBuffer(4 * n)
+        capi.sync()
+        run(f"pass {rep}: output fresh from hipMalloc, never touched", din, dout)
+        run(f"pass {rep}: the same buffers, next {launches} launches", din, dout)
+        dout.free(); din.free()
+        capi.check(L.twg_empty_cache())
+        din = capi.DeviceBuffer(4 * n)
+        capi.check(L.twg_fill_bytes(din.ptr, 0x3c, 4 * n, None))
+        dout = capi.DeviceBuffer(4 * n)
+        capi.check(L.twg_fill_bytes(dout.ptr, 0, 4 * n, None))
+        capi.sync()
+        run(f"pass {rep}: output fresh from hipMalloc, filled once", din, dout)
+        dout.free()
+        dout = capi.DeviceBuffer(4 * n)  # the block just freed, from the pool
+        run(f"pass {rep}: output recycled by the pool", din, dout)
+        time.sleep(2.0)
+        run(f"pass {rep}: the same buffers after 2 s without GPU work", din, dout)
+        dout.free(); din.free()
+        capi.check(L.twg_empty_cache())
+        din = capi.DeviceBuffer(4 * n)
+        din.upload(torch.full((n,), 1.0))  # 20 ms of DMA, no kernels
+        dout = capi.DeviceBuffer(4 * n)
+        run(f"pass {rep}: input written by an upload only, output fresh", din, dout)
+        dout.free(); din.free()
+        capi.check(L.twg_empty_cache())
+        din, dout = capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * n)
+        run(f"pass {rep}: input and output fresh, right after the previous series", din, dout)
+        dout.free(); din.free()
+    return {"first_launches": series, "elements": n, "kernel": "ew_contig<GeluErfOp>", "unit": "us per launch"}
 
 
 def geometry_families(capi, L):
@@ -616,9 +639,16 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         del d_p, d_q, d_z, d_m1, d_m2, d_m3
 
     # config 5: the other masks
+    # (p = 0.05 / 0.1 / 0.25 sit around the density, one selected element in 16 per wavefront,
+    # at which a wavefront switches from gathering to streaming; the alternating mask has
+    # 8192-element spans at 1% and 90% in turn, so both kinds of wavefront share every tile)
     for name, make in (("masked_select_p0.01", lambda: W.bernoulli_mask(n, 0.01)),
+                       ("masked_select_p0.05", lambda: W.bernoulli_mask(n, 0.05)),
+                       ("masked_select_p0.10", lambda: W.bernoulli_mask(n, 0.10)),
+                       ("masked_select_p0.25", lambda: W.bernoulli_mask(n, 0.25)),
                        ("masked_select_p0.99", lambda: W.bernoulli_mask(n, 0.99)),
-                       ("masked_select_clustered", lambda: W.clustered_mask(n, 4096))):
+                       ("masked_select_clustered", lambda: W.clustered_mask(n, 4096)),
+                       ("masked_select_alternating", lambda: W.alternating_density_mask(n, 8192, 0.01, 0.9))):
         if not want(name):
             continue
         m_h = make()

@@ -42,6 +42,8 @@ extern "C" {
 #define TWG_E_SCRATCH_SMALL (-3) /* masked_select scratch buffer too small */
 #define TWG_E_OVERLAP (-4)       /* reserved */
 #define TWG_E_TOO_LARGE (-5)     /* more elements than an entry point with a fixed limit takes */
+#define TWG_E_BUSY (-6)          /* twg_masked_select_f32_static: its array is in use on another stream */
+#define TWG_E_WAIT_ABANDONED (-7) /* masked_select: a tile waited for a status word nobody published */
 
 typedef struct ihipStream_t *twg_stream_t; /* == hipStream_t */
 typedef struct ihipEvent_t *twg_event_t;   /* == hipEvent_t  */
@@ -254,7 +256,15 @@ size_t twg_masked_select_scratch_bytes(int64_t numel);
  * the broadcast logical shape: stride[TWG_A] addresses src, stride[TWG_B]
  * addresses mask, stride[TWG_OUT] is ignored; dim 0 fastest, so logical index i
  * is the row-major index of the broadcast shape reversed.  Asynchronous: read
- * *d_count with twg_memcpy_d2h (or call twg_masked_select_count, below). */
+ * *d_count with twg_memcpy_d2h (or call twg_masked_select_count, below).
+ * The scratch must belong to this call alone until its kernels have finished: it holds a
+ * ticket counter and one status word per tile.  No wait inside the kernels is unbounded:
+ * if the scratch is shared by two launches in flight, or overwritten under a running one,
+ * a tile that has polled for a predecessor's word about a second gives up, it and every
+ * tile whose output position rests on it write nothing, *d_count receives -1 instead of a
+ * count when the last tile is among them, and the second 32-bit word of the scratch is set
+ * to 1 (the first is the ticket counter; both are cleared by every launch of more than one
+ * tile).  All workgroups exit either way. */
 int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
                           const uint8_t *mask, const twg_iter_t *it, void *scratch,
                           size_t scratch_bytes, twg_stream_t stream);
@@ -267,12 +277,27 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
  * reference.  The call allocates nothing and frees nothing once the library is
  * initialised (call twg_init() first: initialisation itself creates the stream).
  * it->numel may be at most TWG_MS_STATIC_MAX_NUMEL; larger inputs return TWG_E_TOO_LARGE.
- * All calls on one GPU share the one array: calls that overlap in time (on different
- * streams) race; calls on one stream are ordered and each clears what it needs. */
+ * All calls on one GPU share the one array.  Calls on one stream are ordered and each clears
+ * what it needs; a call on another stream while the previous call's kernels are still
+ * running is refused with TWG_E_BUSY (the library records an event behind every call and
+ * queries it; the event is created by twg_init).  Under graph capture that check cannot be
+ * made and is skipped: a capturing caller orders its own uses of the array. */
 #define TWG_MS_STATIC_MAX_NUMEL (INT64_C(1) << 30)
 int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
                                  const uint8_t *mask, const twg_iter_t *it,
                                  twg_stream_t stream);
+
+/* Test hook, no counterpart in the reference: twg_masked_select_f32 with the ticket counter
+ * started at first_ticket (0..255) instead of 0 and the look-back's polling limit set to
+ * max_poll_rounds (0 = the library's own).  Tiles below first_ticket are then never
+ * compacted or published, so with first_ticket >= 1 on an input of two or more tiles every
+ * look-back runs into the limit by construction: the way to exercise the give-up path of the
+ * bounded wait with every workgroup still exiting normally.  Expect *d_count == -1 and the
+ * scratch's error word set; `out` is not written by the tiles that gave up. */
+int twg_masked_select_f32_wait_probe(float *out, int64_t *d_count, const float *src,
+                                     const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                                     size_t scratch_bytes, uint32_t first_ticket,
+                                     uint32_t max_poll_rounds, twg_stream_t stream);
 
 /* The same compaction for elements of `elem_size` = 1, 2, 4 or 8 bytes (moved without
  * being looked at, so any dtype of that size; the CPU fallback the reference registers,
@@ -281,7 +306,8 @@ int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
  * like any other launch (work queued afterwards sees them).  The kernel stores K into
  * pinned host memory the moment the last tile knows it and the host polls that word,
  * which saves the separate read-back of twg_masked_select_f32 + twg_memcpy_d2h (one
- * launch and one wait per call).  This is what the masked_select registration calls:
+ * launch and one wait per call; returns TWG_E_WAIT_ABANDONED where twg_masked_select_f32
+ * would have delivered -1).  This is what the masked_select registration calls:
  * it needs K to shape the result.  `out` and `src` must be aligned to elem_size; every
  * element size takes the kernels of twg_masked_select_f32, instantiated for it (dense
  * operands with `src` aligned to four elements, 16 bytes for 8-byte elements; anything

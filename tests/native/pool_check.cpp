@@ -22,7 +22,7 @@ struct FakeBackend {
   static std::set<void *> device;   // live backend allocations
   static std::set<int> completed;   // events that have finished
   static std::set<int> destroyed;
-  static int next_event, syncs, capturing_stream;
+  static int next_event, syncs, capturing_stream, sync_error;
   static std::map<int, int> event_stream;
   static int alloc(void **p, size_t n) {
     if (n > budget) return kOutOfMemory;
@@ -47,7 +47,10 @@ struct FakeBackend {
   static bool done(int e) { return completed.count(e) != 0; }
   static void wait(int e) { completed.insert(e); }
   static void destroy(int e) { destroyed.insert(e); }
-  static void sync_library_stream() { ++syncs; }
+  static int sync_library_stream() {
+    ++syncs;
+    return sync_error;
+  }
   static std::map<void *, size_t> &sizes() {
     static std::map<void *, size_t> m;
     return m;
@@ -56,7 +59,8 @@ struct FakeBackend {
 size_t FakeBackend::budget = size_t(64) << 20;
 std::set<void *> FakeBackend::device;
 std::set<int> FakeBackend::completed, FakeBackend::destroyed;
-int FakeBackend::next_event = 1, FakeBackend::syncs = 0, FakeBackend::capturing_stream = -1;
+int FakeBackend::next_event = 1, FakeBackend::syncs = 0, FakeBackend::capturing_stream = -1,
+    FakeBackend::sync_error = 0;
 std::map<int, int> FakeBackend::event_stream;
 
 int main() {
@@ -126,7 +130,9 @@ int main() {
   CHECK(pool.stats().bytes_pending == 1024);
   CHECK(pool.free(g) == 0);
 
-  // out of memory: pending and cached blocks are waited for, released, and the request retried
+  // out of memory: pending and cached blocks are waited for, released, and the request
+  // retried; the block held for the captured stream (f, 1024 bytes) is NOT released: nobody
+  // has waited for that stream and a captured graph may still replay into it
   void *h = nullptr;
   CHECK(pool.malloc(&h, 1 << 20) == 0);
   CHECK(pool.record_stream(h, 3) == 0);
@@ -135,11 +141,18 @@ int main() {
   void *big = nullptr;
   CHECK(pool.malloc(&big, size_t(60) << 20) == 0);  // only fits once everything else is released
   CHECK(FakeBackend::syncs == syncs + 1);
-  CHECK(pool.stats().bytes_pending == 0 && pool.stats().bytes_cached == 0);
-  CHECK(FakeBackend::device.size() == 1);
+  CHECK(pool.stats().bytes_pending == 1024 && pool.stats().bytes_cached == 0);
+  CHECK(FakeBackend::device.size() == 2 && FakeBackend::device.count(f) == 1);
   CHECK(pool.malloc(&h, size_t(60) << 20) == FakeBackend::kOutOfMemory);
+  CHECK(pool.stats().bytes_pending == 1024 && FakeBackend::device.count(f) == 1);
   CHECK(pool.free(big) == 0);
 
+  // empty_cache reports a failed synchronisation and releases nothing then
+  FakeBackend::sync_error = 77;
+  CHECK(pool.empty_cache() == 77);
+  CHECK(FakeBackend::device.size() == 2);
+  FakeBackend::sync_error = 0;
+  // ... and otherwise lets the held block go as well
   CHECK(pool.empty_cache() == 0);
   CHECK(FakeBackend::device.empty() && FakeBackend::budget == (size_t(64) << 20));
   CHECK(pool.stats().bytes_in_use == 0);

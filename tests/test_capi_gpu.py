@@ -875,6 +875,99 @@ def test_masked_select_streaming_edge_patterns(twg):
                 assert k == ref.numel() and bit_equal(vals, ref), (n, name, off)
 
 
+def test_masked_select_alternating_sparse_and_dense_wavefronts(twg):
+    # neighbouring 8192-element spans (one wavefront's share of a 131072-element tile) at 1% and
+    # 90% selected: the gather path and the streaming loop side by side inside every tile;
+    # also with spans that straddle the wavefront boundaries
+    for n, span in (((1 << 25) + 131072 + 4099, 8192), ((1 << 25) + 5, 5000), ((1 << 23) + 17, 4096),
+                    ((1 << 21) + 8192 + 3, 2048)):
+        x = W.select_source(n, seed=4)
+        m = W.alternating_density_mask(n, span=span)
+        ref = torch.masked_select(x, m)
+        for off in (0, 5):
+            _say(f"masked_select alternating density n={n} span={span} out_offset={off}")
+            vals, k = H.masked_select(x, m, out_offset=off, check_guard=True)
+            assert k == ref.numel() and bit_equal(vals, ref), (n, span, off)
+
+
+def test_masked_select_int64_source_that_ends_with_its_block(twg):
+    # An int64 source of 2^21 + 2^18 elements fills an 18 MiB block of the allocator exactly;
+    # the view x[2:] is 16-byte aligned (fast path) and its length leaves two elements in the
+    # last lane's quad, whose second 16-byte half would start at the end of the block.  The
+    # kernel must not fetch that half.
+    n_store = (1 << 21) + (1 << 18)
+    g = torch.Generator().manual_seed(77)
+    x = torch.randint(-(1 << 62), 1 << 62, (n_store,), generator=g, dtype=torch.int64)
+    for xv in (x[2:], x[2:-1], x[2:-3]):   # two, one and three elements in the last quad
+        m = torch.rand(xv.numel(), generator=g) < 0.99
+        m[-8:] = True
+        _say(f"masked_select int64 view of {xv.numel()} elements at the end of its block")
+        vals, k = H.masked_select(xv, m, check_guard=True)
+        ref = torch.masked_select(xv, m)
+        assert k == ref.numel() and bit_equal(vals, ref)
+    # float64 through the same path, mask dense only at the very end
+    xd = x.view(torch.float64)[2:]
+    m = torch.zeros(xd.numel(), dtype=torch.bool)
+    m[-3:] = True
+    vals, k = H.masked_select(xd, m, check_guard=True)
+    assert k == 3 and bit_equal(vals, xd[-3:])
+
+
+def test_masked_select_wait_gives_up_instead_of_hanging(twg):
+    # The look-back's wait is bounded.  With the ticket counter started at 1 (or 3) instead of
+    # 0 the first tiles are never compacted or published, so every later tile polls a word
+    # that nobody will write: it must give up after max_poll_rounds, write nothing, report -1
+    # as the count and set the error word of the scratch header - and every workgroup exits.
+    L = twg.load()
+    g = torch.Generator().manual_seed(5)
+    cases = [
+        ("tile variant, 2 tiles", 16384, 0, 1),
+        ("tile variant, 40 tiles", 8192 * 40 - 100, 0, 3),
+        ("streaming variant, 129 tiles of 16384", (1 << 21) + 5, 0, 3),
+        ("streaming variant, 257 tiles of 131072", (1 << 25) + 9, 0, 1),
+        ("one element per lane (misaligned source), 3 tiles", 3 * 16384 - 7, 1, 1),
+    ]
+    for name, n, shift, first in cases:
+        _say(f"masked_select abandoned wait: {name}")
+        x = torch.rand(n + shift, generator=g)
+        m = torch.rand(n, generator=g) < 0.5
+        d_x, d_m = twg.to_device(x), twg.to_device(m)
+        out = twg.DeviceBuffer(4 * n)
+        twg.check(L.twg_fill_bytes(out.ptr, 0xAB, out.nbytes, None))
+        cnt = twg.DeviceBuffer(8)
+        twg.check(L.twg_fill_bytes(cnt.ptr, 0x11, 8, None))
+        sb = L.twg_masked_select_scratch_bytes(n)
+        scratch = twg.DeviceBuffer(sb)
+        it = twg.dense_iter(n)
+        twg.check(L.twg_masked_select_f32_wait_probe(out.ptr, cnt.ptr, d_x.ptr + 4 * shift, d_m.ptr,
+                                                     ctypes.byref(it), scratch.ptr, sb, first, 64, None))
+        twg.sync()
+        assert int(cnt.download((1,), torch.int64)[0]) == -1, name
+        hdr = scratch.download((2,), torch.int32)
+        assert int(hdr[1]) == 1, "the error word of the scratch header is not set"
+        assert bool((out.download((out.nbytes,), torch.uint8) == 0xAB).all()), "a tile that gave up wrote output"
+        # the same scratch serves a normal call afterwards: every launch clears what it needs
+        twg.check(L.twg_masked_select_f32(out.ptr, cnt.ptr, d_x.ptr + 4 * shift, d_m.ptr,
+                                          ctypes.byref(it), scratch.ptr, sb, None))
+        k = int(cnt.download((1,), torch.int64)[0])
+        assert k == int(m.sum())
+        assert bit_equal(out.download((k,), torch.float32), x[shift:shift + n][m])
+        assert int(scratch.download((2,), torch.int32)[1]) == 0
+    # the probe with nothing forced is the ordinary call
+    n = 8192 * 5 + 3
+    x, m = torch.rand(n, generator=g), torch.rand(n, generator=g) < 0.3
+    d_x, d_m, out, cnt = twg.to_device(x), twg.to_device(m), twg.DeviceBuffer(4 * n), twg.DeviceBuffer(8)
+    sb = L.twg_masked_select_scratch_bytes(n)
+    scratch = twg.DeviceBuffer(sb)
+    it = twg.dense_iter(n)
+    twg.check(L.twg_masked_select_f32_wait_probe(out.ptr, cnt.ptr, d_x.ptr, d_m.ptr, ctypes.byref(it),
+                                                 scratch.ptr, sb, 0, 0, None))
+    assert int(cnt.download((1,), torch.int64)[0]) == int(m.sum())
+    assert L.twg_masked_select_f32_wait_probe(out.ptr, cnt.ptr, d_x.ptr, d_m.ptr, ctypes.byref(it),
+                                              scratch.ptr, sb, 256, 0, None) == twg.E_INVALID_ARG
+    assert b"gave up" in L.twg_error_string(twg.E_WAIT_ABANDONED)
+
+
 def test_masked_select_clustered_and_empty(twg):
     n = (1 << 22) + 1234
     x = W.select_source(n, seed=4)

@@ -62,7 +62,7 @@ def test_streaming_masked_select_counts_its_loads():
     seen = set()
     for i in range(1, len(parts), 2):
         name, body = parts[i], parts[i + 1].split("s_endpgm")[0]
-        m = re.search(r"ms_compact_streamILi16ELi4ELi5E([fmth])E", name)
+        m = re.search(r"ms_compact_streamILi16ELi4E([fmth])E", name)
         if not m:
             continue
         waits = re.findall(r"s_waitcnt vmcnt\((\d+)\)", body)

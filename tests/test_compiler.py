@@ -49,6 +49,42 @@ def test_forms_that_must_not_fuse():
     assert torch.equal(gm(a, b), torch.relu(a + 2.0 * b))
 
 
+def test_operand_modified_between_add_and_relu():
+    # Dynamo graphs are not functionalized: the fused node must read the operands where the
+    # add read them, not where the relu stood
+    from torch_webgpu.compiler import add_relu, fuse_add_relu
+
+    def f(a, b):
+        s = a + b
+        a.mul_(2.0)
+        return torch.relu(s)
+
+    gm = torch.fx.symbolic_trace(f)
+    a, b = torch.tensor([1.0, -3.0]), torch.tensor([0.5, 1.0])
+    ref = f(a.clone(), b.clone())
+    assert fuse_add_relu(gm) == 1 and _count(gm, add_relu) == 1
+    assert torch.equal(gm(a.clone(), b.clone()), ref)
+    assert torch.equal(ref, torch.tensor([1.5, 0.0]))
+
+    # the sum itself modified in place before the relu: two users, nothing is fused
+    def h(a, b):
+        s = a + b
+        s.mul_(2.0)
+        return torch.relu(s)
+
+    gm = torch.fx.symbolic_trace(h)
+    assert fuse_add_relu(gm) == 0
+    assert torch.equal(gm(a.clone(), b.clone()), h(a.clone(), b.clone()))
+
+
+def test_reference_import_paths():
+    import torch_webgpu
+    from torch_webgpu.compiler.webgpu_compiler import webgpu_backend  # python/torch_webgpu/__init__.py:15
+    assert webgpu_backend is torch_webgpu.webgpu_backend
+    for name in torch_webgpu.__all__:
+        assert hasattr(torch_webgpu, name), name
+
+
 def test_compiled_function_on_cpu_tensors():
     # the backend is usable for any graph: on CPU tensors the fused node runs the eager pair
     import torch_webgpu  # noqa: F401

@@ -10,12 +10,29 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
+_hip = None
 
-def _both(twg, L, n, p, seed):
+
+def _free_device_bytes():
+    """Free device memory as the driver reports it (hipMemGetInfo): unlike the allocator's
+    own counters it also sees a hipMalloc made behind the allocator's back."""
+    global _hip
+    if _hip is None:
+        _hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert _hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def _both(twg, L, n, p, seed, shift=0):
+    """shift: elements the source pointer is moved off its 16-byte alignment (the
+    one-element-per-lane variant of the kernel then runs, on the same static array)."""
     g = torch.Generator().manual_seed(seed)
-    src = torch.rand(n, generator=g) * 2 - 1
+    src_all = torch.rand(n + shift, generator=g) * 2 - 1
+    src = src_all[shift:]
     mask = torch.rand(n, generator=g) < p
-    d_src, d_mask = twg.to_device(src), twg.to_device(mask)
+    d_src_buf, d_mask = twg.to_device(src_all), twg.to_device(mask)
+    d_src = d_src_buf.at(4 * shift)
     it = twg.dense_iter(n)
     res = []
     for static in (False, True):
@@ -23,15 +40,17 @@ def _both(twg, L, n, p, seed):
         cnt = twg.DeviceBuffer(8)
         twg.check(L.twg_fill_bytes(out.ptr, 0xAB, out.nbytes, None))
         if static:
-            before = twg.mem_stats()
-            twg.check(L.twg_masked_select_f32_static(out.ptr, cnt.ptr, d_src.ptr, d_mask.ptr,
+            twg.sync()
+            before, free_before = twg.mem_stats(), _free_device_bytes()
+            twg.check(L.twg_masked_select_f32_static(out.ptr, cnt.ptr, d_src, d_mask.ptr,
                                                      ctypes.byref(it), None))
-            after = twg.mem_stats()
+            after, free_after = twg.mem_stats(), _free_device_bytes()
             assert after == before, "the call went to the allocator"
+            assert free_after == free_before, "the call allocated or freed device memory"
         else:
             sb = L.twg_masked_select_scratch_bytes(n)
             scratch = twg.DeviceBuffer(sb)
-            twg.check(L.twg_masked_select_f32(out.ptr, cnt.ptr, d_src.ptr, d_mask.ptr,
+            twg.check(L.twg_masked_select_f32(out.ptr, cnt.ptr, d_src, d_mask.ptr,
                                               ctypes.byref(it), scratch.ptr, sb, None))
         k = int(cnt.download((1,), torch.int64)[0])
         raw = out.download((out.nbytes,), torch.uint8)
@@ -54,6 +73,51 @@ def test_static_scratch_matches_allocated_scratch(twg):
     _both(twg, L, 70001, 0.3, 2)
     # and a third that fits one tile (no ticket, no look-back)
     _both(twg, L, 1000, 0.9, 3)
+    # a source that is not 16-byte aligned: the one-element-per-lane variant, several tiles
+    _both(twg, L, 5 * 16384 + 77, 0.4, 4, shift=1)
+    _both(twg, L, 40000, 0.6, 5, shift=3)
+
+
+def test_static_scratch_is_refused_to_a_second_stream_while_in_use(twg):
+    # One array per GPU: a call on another stream while the previous call's kernels may still
+    # be running must be refused (TWG_E_BUSY), not left to corrupt the tickets; once that work
+    # has finished the other stream is served.
+    L = twg.load()
+    hip = ctypes.CDLL("libamdhip64.so")
+    stream_a, stream_b = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(stream_a), 1) == 0  # hipStreamNonBlocking
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(stream_b), 1) == 0
+    n = (1 << 22) + 777
+    g = torch.Generator().manual_seed(8)
+    src, mask = torch.rand(n, generator=g), torch.rand(n, generator=g) < 0.5
+    d_src, d_mask = twg.to_device(src), twg.to_device(mask)
+    out_a, out_b = twg.DeviceBuffer(4 * n), twg.DeviceBuffer(4 * n)
+    cnt_a, cnt_b = twg.DeviceBuffer(8), twg.DeviceBuffer(8)
+    big = twg.DeviceBuffer(1 << 30)
+    it = twg.dense_iter(n)
+    twg.sync()
+    # ~20 ms of fills keep stream A busy, the static call queues up behind them
+    print("static masked_select: second stream while the first is busy", flush=True)
+    for _ in range(60):
+        twg.check(L.twg_fill_bytes(big.ptr, 1, big.nbytes, stream_a))
+    twg.check(L.twg_masked_select_f32_static(out_a.ptr, cnt_a.ptr, d_src.ptr, d_mask.ptr,
+                                             ctypes.byref(it), stream_a))
+    rc = L.twg_masked_select_f32_static(out_b.ptr, cnt_b.ptr, d_src.ptr, d_mask.ptr,
+                                        ctypes.byref(it), stream_b)
+    assert rc == twg.E_BUSY, rc
+    assert b"another stream" in L.twg_error_string(rc)
+    # the same stream is never refused: its calls are ordered
+    twg.check(L.twg_masked_select_f32_static(out_a.ptr, cnt_a.ptr, d_src.ptr, d_mask.ptr,
+                                             ctypes.byref(it), stream_a))
+    assert hip.hipStreamSynchronize(stream_a) == 0
+    twg.check(L.twg_masked_select_f32_static(out_b.ptr, cnt_b.ptr, d_src.ptr, d_mask.ptr,
+                                             ctypes.byref(it), stream_b))
+    assert hip.hipStreamSynchronize(stream_b) == 0
+    k = int(mask.sum())
+    for cnt, out in ((cnt_a, out_a), (cnt_b, out_b)):
+        assert int(cnt.download((1,), torch.int64)[0]) == k
+        assert torch.equal(out.download((k,), torch.float32), src[mask])
+    assert hip.hipStreamDestroy(stream_a) == 0 and hip.hipStreamDestroy(stream_b) == 0
 
 
 def test_static_scratch_limits(twg):

@@ -11,7 +11,7 @@ Plays the part of the reference's setup.py (setup.py:16-42), which links
 csrc/**/*.cpp against Google Dawn.  Both outputs land next to the Python package
 in torch_webgpu/ so that `import torch_webgpu` finds them without installation.
 
-Usage: python build.py [hip] [torch] [ablate] [-j N]
+Usage: python build.py [hip] [torch] [-j N]
 """
 import argparse
 import concurrent.futures
@@ -80,17 +80,6 @@ def build_hip(nproc=8, extra_flags=()):
     return out
 
 
-def build_ablate():
-    """libtwg_ablate.so: the timing experiments `bench.py --ablations` runs (copy launch shapes,
-    masked_select cut off phase by phase and in two other structures).  Not part of the product:
-    nothing else loads it."""
-    hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
-    src = os.path.join(HERE, "csrc", "ablate", "twg_ablate.hip")
-    out = os.path.join(PKG, "libtwg_ablate.so")
-    _run([hipcc, *HIP_FLAGS, "-shared", src, "-o", out, "-Wl,-rpath," + os.path.join(ROCM, "lib")])
-    return out
-
-
 def build_torch(nproc=8):
     import torch  # noqa: F401  (headers and ABI flag come from the installed torch)
     from torch.utils import cpp_extension
@@ -127,8 +116,6 @@ def main():
     a = ap.parse_args()
     if "hip" in a.what:
         print("built", build_hip(a.j))
-    if "ablate" in a.what:
-        print("built", build_ablate())
     if "torch" in a.what:
         print("built", build_torch(a.j))
 

@@ -40,9 +40,16 @@ int canonicalize(const twg_iter_t *it, int nops, Geom *g);
 // bytes, count written to *d_count (device memory, or host memory the device can
 // address).  Dense 16-byte-aligned sources of 4-byte elements take the vectorised
 // kernels, everything else the one-element-per-lane kernel.
+// `wait` is only ever set by the test hook: the ticket counter's first value (0..255; tiles
+// below it are never compacted or published) and the number of polling rounds after which
+// a look-back gives up (0 = the library's limit).
+struct MsWait {
+  uint32_t first_ticket = 0;
+  uint32_t max_rounds = 0;
+};
 int masked_select_launch(void *out, int64_t *d_count, const void *src, int elem_size,
                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                         size_t scratch_bytes, twg_stream_t stream);
+                         size_t scratch_bytes, twg_stream_t stream, MsWait wait = MsWait());
 
 
 // Look up the address the current device gives the masked_select scratch array that is

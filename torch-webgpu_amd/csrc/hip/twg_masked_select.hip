@@ -6,6 +6,8 @@
 // ATen's CPU kernel, one host->device copy.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "twg_internal.h"
 #include "twg_ms_kernels.h"
 
@@ -31,7 +33,16 @@ struct MsLaunch {
   uint64_t *status;
   void *scratch;
   twg_stream_t stream;
+  MsWait wait;
 };
+
+// Clear the header and `words` status words; a first ticket other than 0 (the test hook)
+// goes into the low byte of the ticket counter.
+int clear_scratch(void *scratch, size_t words, const MsWait &wait, twg_stream_t stream) {
+  int rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * words, stream);
+  if (rc == 0 && wait.first_ticket) rc = twg_fill_bytes(scratch, (int)wait.first_ticket, 1, stream);
+  return rc;
+}
 
 // One launch of the streaming kernel; its last tile may be incomplete.
 template <int WAVES, int GROUPS, typename T>
@@ -41,10 +52,11 @@ int launch_stream(const MsLaunch<T> &m) {
   if (ntiles > INT32_MAX) return TWG_E_UNSUPPORTED;
   // status words kStreamStatusStride apart
   const size_t words = (size_t)ntiles * kStreamStatusStride;
-  int rc = twg_fill_bytes(m.scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * words, m.stream);
+  int rc = clear_scratch(m.scratch, words, m.wait, m.stream);
   if (rc) return rc;
-  ms_compact_stream<WAVES, GROUPS, 5, T><<<(unsigned)ntiles, WAVES * 64, 0, resolve_stream(m.stream)>>>(
-      m.out, m.d_count, m.src, m.mask, m.numel, (uint32_t)ntiles, m.ticket, m.status);
+  ms_compact_stream<WAVES, GROUPS, T><<<(unsigned)ntiles, WAVES * 64, 0, resolve_stream(m.stream)>>>(
+      m.out, m.d_count, m.src, m.mask, m.numel, (uint32_t)ntiles, m.ticket, m.status,
+      m.wait.max_rounds);
   return (int)hipGetLastError();
 }
 
@@ -52,14 +64,14 @@ int launch_stream(const MsLaunch<T> &m) {
 // variant below that.
 template <typename T>
 int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t *mask, int64_t numel,
-                void *scratch, twg_stream_t stream) {
+                void *scratch, twg_stream_t stream, const MsWait &wait) {
   // scratch: [0] ticket, [256...] the tiles' status words
   uint32_t *ticket = static_cast<uint32_t *>(scratch);
   uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
   T *out = static_cast<T *>(out_v);
   const T *src = static_cast<const T *>(src_v);
   if (numel >= kStreamMinElems) {
-    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, status, scratch, stream};
+    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, status, scratch, stream, wait};
     if (numel >= (int64_t(1) << 25)) return launch_stream<16, 4>(m);
     if (numel >= (int64_t(1) << 23)) return launch_stream<16, 2>(m);
     return launch_stream<8, 1>(m);
@@ -68,11 +80,9 @@ int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t 
   const uint32_t ntiles = (uint32_t)ntiles64;
   int rc = 0;
   // one tile takes no ticket and looks back at nothing: the scratch may hold anything
-  if (ntiles > 1 &&
-      (rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
-    return rc;
+  if (ntiles > 1 && (rc = clear_scratch(scratch, ntiles, wait, stream))) return rc;
   ms_compact_vec<kSmallWaves, T><<<ntiles, kSmallWaves * 64, 0, resolve_stream(stream)>>>(
-      out, d_count, src, mask, numel, ntiles, ticket, status);
+      out, d_count, src, mask, numel, ntiles, ticket, status, wait.max_rounds);
   return (int)hipGetLastError();
 }
 
@@ -93,7 +103,9 @@ namespace twg {
 
 int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int elem_size,
                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                         size_t scratch_bytes, twg_stream_t stream) {
+                         size_t scratch_bytes, twg_stream_t stream, MsWait wait) {
+  if (wait.max_rounds == 0) wait.max_rounds = kMsMaxPollRounds;
+  if (wait.first_ticket > 255) return TWG_E_INVALID_ARG;
   int rc = ensure_init();
   if (rc) return rc;
   if (!it || !d_count) return TWG_E_INVALID_ARG;
@@ -123,10 +135,10 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
                     reinterpret_cast<uintptr_t>(mask) % 4 == 0;
   if (fast) {
     switch (elem_size) {
-      case 1: return launch_fast<uint8_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
-      case 2: return launch_fast<uint16_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
-      case 4: return launch_fast<float>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
-      default: return launch_fast<uint64_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream);
+      case 1: return launch_fast<uint8_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
+      case 2: return launch_fast<uint16_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
+      case 4: return launch_fast<float>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
+      default: return launch_fast<uint64_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
     }
   }
 
@@ -137,9 +149,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
   if (ntiles64 > INT32_MAX) return TWG_E_UNSUPPORTED;
   const uint32_t ntiles = (uint32_t)ntiles64;
   // one tile takes no ticket and looks back at nothing: the scratch may hold anything
-  if (ntiles > 1 &&
-      (rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * ntiles, stream)))
-    return rc;
+  if (ntiles > 1 && (rc = clear_scratch(scratch, ntiles, wait, stream))) return rc;
 
   {
     MsGeom mg{};
@@ -154,11 +164,11 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
       if (dense)
         ms_compact_scalar<false, T><<<ntiles, kScalarWaves * 64, 0, s>>>(
             static_cast<T *>(out_v), d_count, static_cast<const T *>(src_v), mask, g.numel, ntiles,
-            ticket, status, mg);
+            ticket, status, wait.max_rounds, mg);
       else
         ms_compact_scalar<true, T><<<ntiles, kScalarWaves * 64, 0, s>>>(
             static_cast<T *>(out_v), d_count, static_cast<const T *>(src_v), mask, g.numel, ntiles,
-            ticket, status, mg);
+            ticket, status, wait.max_rounds, mg);
     };
     switch (elem_size) {
       case 1: scalar(uint8_t{}); break;
@@ -185,6 +195,18 @@ namespace twg {
 namespace {
 constexpr int kMaxDevices = 16;
 void *g_static_scratch[kMaxDevices] = {};  // per device; written during init only
+
+// Who used a device's array last: the stream, and an event recorded behind that call's
+// kernels.  A call on another stream is refused while that event is pending, because two
+// launches in flight on one set of tickets and status words would corrupt each other.
+// Calls on one stream are ordered by the stream.  The events are created during init.
+struct StaticUse {
+  std::mutex mu;
+  hipEvent_t done = nullptr;
+  hipStream_t last = nullptr;
+  bool used = false;
+};
+StaticUse g_static_use[kMaxDevices];
 }  // namespace
 
 int static_scratch_setup() {
@@ -194,6 +216,8 @@ int static_scratch_setup() {
   void *ptr = nullptr;
   TWG_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
   if (!ptr || reinterpret_cast<uintptr_t>(ptr) % 256 != 0) return TWG_E_INVALID_ARG;
+  if (!g_static_use[dev].done)
+    TWG_HIP_TRY(hipEventCreateWithFlags(&g_static_use[dev].done, hipEventDisableTiming));
   g_static_scratch[dev] = ptr;
   return 0;
 }
@@ -218,7 +242,36 @@ int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
   TWG_HIP_TRY(hipGetDevice(&dev));
   void *ptr = (dev >= 0 && dev < kMaxDevices) ? g_static_scratch[dev] : nullptr;
   if (!ptr) return TWG_E_UNSUPPORTED;  // not the device the library was initialised on
-  return masked_select_launch(out, d_count, src, 4, mask, it, ptr, kStaticScratchBytes, stream);
+  hipStream_t s = resolve_stream(stream);
+  StaticUse &use = g_static_use[dev];
+  std::lock_guard<std::mutex> lk(use.mu);
+  // A stream that is being captured can neither be asked whether earlier work has finished
+  // nor take part in this bookkeeping: such a caller orders its own uses of the array.
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  TWG_HIP_TRY(hipStreamIsCapturing(s, &cap));
+  const bool capturing = cap != hipStreamCaptureStatusNone;
+  if (!capturing && use.used && use.last != s) {
+    const hipError_t q = hipEventQuery(use.done);
+    if (q == hipErrorNotReady) return TWG_E_BUSY;
+    if (q != hipSuccess) return (int)q;
+  }
+  rc = masked_select_launch(out, d_count, src, 4, mask, it, ptr, kStaticScratchBytes, stream);
+  if (rc == 0 && !capturing) {
+    TWG_HIP_TRY(hipEventRecord(use.done, s));
+    use.last = s;
+    use.used = true;
+  }
+  return rc;
+}
+
+int twg_masked_select_f32_wait_probe(float *out, int64_t *d_count, const float *src,
+                                     const uint8_t *mask, const twg_iter_t *it, void *scratch,
+                                     size_t scratch_bytes, uint32_t first_ticket,
+                                     uint32_t max_poll_rounds, twg_stream_t stream) {
+  MsWait wait;
+  wait.first_ticket = first_ticket;
+  wait.max_rounds = max_poll_rounds;
+  return masked_select_launch(out, d_count, src, 4, mask, it, scratch, scratch_bytes, stream, wait);
 }
 
 }  // extern "C"

@@ -1,6 +1,5 @@
 // Device side of masked_select: the compaction kernels and what they share (status words,
-// look-back, ballot offsets).  Included by twg_masked_select.hip, which launches them, and by
-// the benchmark's ablation library, which times cut-down and alternative forms of them.
+// look-back, ballot offsets).  Included by twg_masked_select.hip, which launches them.
 //
 // masked_select as a single-pass, order-preserving stream compaction.
 //
@@ -25,6 +24,19 @@
 // A status word packs {flag:2, value:62} so one relaxed agent-scope 64-bit
 // load/store carries everything; no fences are needed because no other memory
 // is communicated between tiles.
+//
+// Every wait is bounded.  With a cleared scratch that one launch has to itself a tile only
+// waits for tiles that are already running, and the farthest wait measured is a few hundred
+// polling rounds.  A scratch shared by two launches in flight (or cleared under a running
+// launch) can leave a wavefront polling a word that nobody will publish, so a look-back that
+// has polled kMsMaxPollRounds times gives up: the tile publishes an inclusive word marked
+// BROKEN (so that its successors drain instead of waiting in turn), sets the error word of
+// the scratch header, writes nothing to the output, and every tile whose prefix rests on a
+// BROKEN word does the same; the last tile then reports kMsCountAbandoned instead of a
+// count.  A prefix that would place a tile's output beyond the numel elements the output
+// holds (only possible with status words of another launch) is treated the same way, and a
+// ticket beyond the launch's own tiles (a ticket counter that another launch also draws
+// from) makes its workgroup leave at once.
 //
 // Three facts about MI355X shape the streaming variant (inputs from 2^21 elements).
 // Same-address agent-scope atomics retire at about one per 7 ns, so the ticket must not
@@ -53,7 +65,13 @@ constexpr int kScalarSteps = 16;    //   16 wavefronts x 16 steps of 64 elements
 constexpr int kScalarTile = 64 * kScalarWaves * kScalarSteps;
 constexpr int kMsMinTile = 256 * kSteps * 4;  // smallest tile of any variant (ms_compact_vec<4>)
 static_assert(kScalarTile >= kMsMinTile, "the scratch is sized for kMsMinTile-element tiles");
-constexpr size_t kMsHeaderBytes = 256;                  // the ticket, padded
+constexpr size_t kMsHeaderBytes = 256;                  // ticket (u32), error word (u32), padding
+constexpr int kMsErrorWord = 1;                         // index of the error word, in u32s
+// Polling rounds after which a look-back gives up (each round is a sleep plus a load from
+// memory, about a microsecond under load: a second or so, four orders of magnitude beyond
+// the longest wait of a healthy launch).
+constexpr uint32_t kMsMaxPollRounds = 1u << 20;
+constexpr int64_t kMsCountAbandoned = -1;               // what *d_count receives instead of a count
 // Smallest tile of the streaming variant (8 wavefronts x 8 steps x 256 elements) and the
 // status words the scratch must hold: one per kMsMinTile elements for the small-tile
 // variants, or kStreamStatusStride per streaming tile, the incomplete last one included.
@@ -77,6 +95,7 @@ static_assert(kStreamStatusStride == 4, "ms_scratch_bytes sizes the scratch for 
 constexpr uint64_t kFlagShift = 62;
 constexpr uint64_t kFlagAggregate = 1ull << kFlagShift;
 constexpr uint64_t kFlagInclusive = 2ull << kFlagShift;
+constexpr uint64_t kFlagBroken = 3ull << kFlagShift;  // inclusive, but the value is not to be used
 constexpr uint64_t kValueMask = (1ull << kFlagShift) - 1;
 
 struct MsGeom {
@@ -128,14 +147,17 @@ __device__ __forceinline__ void wave_offsets(uint32_t c, uint32_t &below, uint32
 }
 
 // Exclusive prefix of tile `tile`: sum of the totals of all earlier tiles.  Run by
-// one full wavefront.  Each round inspects the 256 nearest unseen predecessors
-// (4 status words per lane, nearest first), waits until all of them have published
+// one full wavefront.  Each round inspects the 64 * LPL nearest unseen predecessors
+// (LPL status words per lane, nearest first), waits until all of them have published
 // at least an aggregate, and stops at the nearest one that carries an inclusive
-// prefix.
+// prefix.  Returns -1 if the wait was given up after max_rounds polls or if that
+// inclusive word is marked BROKEN.
 template <int LPL, int STRIDE>
-__device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t tile, int lane) {
+__device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t tile, int lane,
+                                             uint32_t max_rounds) {
   int64_t exclusive = 0;
   int64_t look = (int64_t)tile - 1 - lane;  // lane's nearest candidate
+  uint32_t rounds = 0;
   while (true) {
     uint64_t st[LPL];
     while (true) {
@@ -148,24 +170,27 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
         pending |= (st[q] >> kFlagShift) == 0;
       }
       if (__ballot(pending) == 0) break;
+      if (++rounds >= max_rounds) return -1;  // wavefront-uniform
       __builtin_amdgcn_s_sleep(1);
     }
     int64_t part = 0;
-    bool done = false;
+    bool done = false, broken = false;
 #pragma unroll
     for (int q = 0; q < LPL; ++q) {
       if (!done) {
-        const uint64_t incl = __ballot((st[q] >> kFlagShift) == 2);
+        const uint64_t incl = __ballot((st[q] >> kFlagShift) >= 2);
         const int64_t val = (int64_t)(st[q] & kValueMask);
         if (incl) {
           const int first = __builtin_ctzll(incl);  // nearest predecessor with a full prefix
           part += (lane <= first) ? val : 0;
+          broken = __ballot(lane == first && (st[q] >> kFlagShift) == 3) != 0;
           done = true;
         } else {
           part += val;
         }
       }
     }
+    if (broken) return -1;
     exclusive += wave_sum_i64(part);
     if (done) return exclusive;
     look -= 64 * LPL;
@@ -173,11 +198,14 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
 }
 
 // Aggregate, look-back, inclusive prefix: the part every variant shares.  Call
-// with all threads; returns the tile's exclusive prefix to all of them.  s_slot is
-// one int64 of LDS.  The last tile also writes the grand total.
+// with all threads; returns the tile's exclusive prefix to all of them, or -1 if the
+// tile has to leave without writing anything (see the note on bounded waits at the top).
+// s_slot is one int64 of LDS.  The last tile also writes the grand total.  `hdr` is the
+// scratch header, `room` the number of elements the output holds.
 template <int LPL = kLookPerLane, int STRIDE = 1>
-__device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, uint32_t ntiles,
-                                               uint32_t tile_total, int64_t *d_count,
+__device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t *hdr, uint32_t tile,
+                                               uint32_t ntiles, uint32_t tile_total, int64_t room,
+                                               uint32_t max_rounds, int64_t *d_count,
                                                int64_t *s_slot) {
   const int lane = threadIdx.x & 63;
   if (threadIdx.x < 64) {  // wave 0
@@ -186,15 +214,24 @@ __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t tile, 
       status_store(mine, (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
     int64_t exclusive = 0;
     if (tile != 0) {
-      exclusive = look_back<LPL, STRIDE>(status, tile, lane);
-      if (lane == 0) status_store(mine, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+      exclusive = look_back<LPL, STRIDE>(status, tile, lane, max_rounds);
+      if (exclusive >= 0 && exclusive + (int64_t)tile_total > room) exclusive = -1;
+      if (lane == 0) {
+        if (exclusive >= 0) {
+          status_store(mine, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+        } else {
+          status_store(mine, kFlagBroken);
+          __hip_atomic_store(hdr + kMsErrorWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
     }
     if (lane == 0) {
       *s_slot = exclusive;
       // One 8-byte store at system scope: the count may live in host memory that the
       // host polls while the rest of the grid is still compacting.
       if (tile == ntiles - 1)
-        __hip_atomic_store(d_count, exclusive + (int64_t)tile_total,
+        __hip_atomic_store(d_count,
+                           exclusive >= 0 ? exclusive + (int64_t)tile_total : kMsCountAbandoned,
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
@@ -222,6 +259,9 @@ struct Quad<float> {
   static __device__ __forceinline__ Quad load(const float *p) {
     return {__builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p))};
   }
+  static __device__ __forceinline__ Quad load_selected(const float *p, const float *dummy, uint32_t bits) {
+    return load(bits ? p : dummy);
+  }
 };
 template <>
 struct Quad<uint64_t> {
@@ -234,6 +274,15 @@ struct Quad<uint64_t> {
     return {__builtin_nontemporal_load(reinterpret_cast<const u64x2 *>(p)),
             __builtin_nontemporal_load(reinterpret_cast<const u64x2 *>(p) + 1)};
   }
+  // Each 16-byte half is fetched only where one of its own two elements is selected: in an
+  // incomplete last tile the half past the array's end (its elements count as not selected)
+  // is then never touched, and a half that holds the array's last element is an aligned
+  // 16-byte piece that starts inside the array.
+  static __device__ __forceinline__ Quad load_selected(const uint64_t *p, const uint64_t *dummy,
+                                                       uint32_t bits) {
+    return {__builtin_nontemporal_load(reinterpret_cast<const u64x2 *>((bits & 0x3u) ? p : dummy)),
+            __builtin_nontemporal_load(reinterpret_cast<const u64x2 *>((bits & 0xCu) ? p + 2 : dummy + 2))};
+  }
 };
 template <>
 struct Quad<uint16_t> {
@@ -242,6 +291,9 @@ struct Quad<uint16_t> {
   __device__ __forceinline__ void set(int j, uint16_t x) { v[j] = x; }
   static __device__ __forceinline__ Quad load(const uint16_t *p) {
     return {__builtin_nontemporal_load(reinterpret_cast<const u16x4 *>(p))};
+  }
+  static __device__ __forceinline__ Quad load_selected(const uint16_t *p, const uint16_t *dummy, uint32_t bits) {
+    return load(bits ? p : dummy);
   }
 };
 template <>
@@ -253,6 +305,9 @@ struct Quad<uint8_t> {
   }
   static __device__ __forceinline__ Quad load(const uint8_t *p) {
     return {__builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p))};
+  }
+  static __device__ __forceinline__ Quad load_selected(const uint8_t *p, const uint8_t *dummy, uint32_t bits) {
+    return load(bits ? p : dummy);
   }
 };
 
@@ -285,16 +340,13 @@ struct MsStreamShared {
   __attribute__((aligned(16))) unsigned char ring[WAVES][ring_bytes<T>()];
 };
 
-// STAGES cuts the kernel short for timing experiments (the benchmark's ablation library
-// instantiates 1..4; the library itself only ever runs all 5): 1 = take the ticket, 2 = + mask
-// loads, selection bits and counts, 3 = + aggregate, look-back and the first source loads,
-// 4 = + every source load and the compaction in LDS, 5 = + the stores.
-template <int WAVES, int GROUPS, int STAGES = 5, typename T = float>
+template <int WAVES, int GROUPS, typename T = float>
 __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t *d_count,
                                                                 const T *src,
                                                                 const uint8_t *mask, int64_t n,
                                                                 uint32_t ntiles, uint32_t *ticket,
-                                                                uint64_t *status) {
+                                                                uint64_t *status,
+                                                                uint32_t max_rounds) {
   constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
   constexpr int64_t kTileElems = (int64_t)kWaveSpan * WAVES;
   constexpr uint32_t kLine = 128u / sizeof(T);  // elements per 128-byte line
@@ -308,7 +360,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t tile = sh.tile;
-  if constexpr (STAGES < 2) return;
+  if (tile >= ntiles) return;  // workgroup-uniform; only with a ticket counter that is not ours alone
   const int64_t start = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
   const uint8_t *mask_w = mask + start + lane * 4;
   const T *src_w = src + start + lane * 4;
@@ -363,17 +415,12 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     tile_total += t;
   }
 
-  if constexpr (STAGES < 3) {
-    if (tile_total == 0xFFFFFFFFu) *d_count = wbase;  // never true: keeps the counts alive
-    return;
-  }
-
   // ---- 2. the first kDepth steps' values go in flight, then aggregate / look-back
   // (a lane with nothing selected reads the tile's first four elements; in an incomplete
   // last tile those may not all exist, so there it reads the array's first four)
   const T *dummy = whole ? src + (int64_t)tile * kTileElems : src;
   auto fetch = [&](uint32_t four_bits, int step) {
-    return Quad<T>::load(four_bits ? src_w + step * 256 : dummy);
+    return Quad<T>::load_selected(src_w + step * 256, dummy, four_bits);
   };
   uint32_t b_cur = sh.bits[0][threadIdx.x];
   constexpr uint32_t kSparseMax = kWaveSpan / kSparseDivisor;
@@ -386,14 +433,8 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
   }
   const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(
-      status, tile, ntiles, tile_total, d_count, &sh.base);
-  if constexpr (STAGES < 4) {
-    uint32_t acc = 0;
-#pragma unroll
-    for (int k = 0; k < kDepth; ++k) acc += (uint32_t)vals[k].get(0);
-    if (acc == 0x7E39A4C5u) out[base + wbase] = vals[0].get(0);  // practically never: keeps the loads alive
-    return;
-  }
+      status, ticket, tile, ntiles, tile_total, n, max_rounds, d_count, &sh.base);
+  if (base < 0) return;  // workgroup-uniform: the look-back was abandoned
 
   // ---- 3a. a wavefront with few selected elements gathers them one element per lane:
   //          every lane of a load then fetches something wanted, where a step of the
@@ -441,12 +482,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     const T *src_wave = src + start;
     T *wout = out + (base + wbase);
     for (uint32_t i = lane; i < wt; i += 64) {
-      const T x = __builtin_nontemporal_load(src_wave + lds[i]);
-      if constexpr (STAGES >= 5) {
-        wout[i] = x;
-      } else if ((uint32_t)x == 0x7E39A4C5u) {  // practically never
-        wout[i] = x;
-      }
+      wout[i] = __builtin_nontemporal_load(src_wave + lds[i]);
     }
     return;
   }
@@ -482,8 +518,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
           if (f & (1u << j)) {
             const T x = x4.get(j);
             ring[pos & (kRingElems - 1)] = x;
-            if constexpr (STAGES >= 5)
-              if (pos < kLine && shift) obase[pos] = x;  // shared first line: element by element
+            if (pos < kLine && shift) obase[pos] = x;  // shared first line: element by element
             ++pos;
           }
         }
@@ -495,12 +530,8 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
         for (uint32_t idx = flushed + lane; idx < end4; idx += 64) {
           const u32x4 x = *reinterpret_cast<const u32x4 *>(
               sh.ring[wave] + ((16u * idx) & (uint32_t)(kRingElems * sizeof(T) - 1)));
-          if constexpr (STAGES >= 5) {
-            __builtin_nontemporal_store(
-                x, reinterpret_cast<u32x4 *>(reinterpret_cast<unsigned char *>(obase) + 16 * (size_t)idx));
-          } else if (x[0] == 0x7E39A4C5u && x[3] == 0xFE39A4C5u) {  // practically never
-            obase[kSlot * (size_t)idx] = ring[(kSlot * idx) & (kRingElems - 1)];
-          }
+          __builtin_nontemporal_store(
+              x, reinterpret_cast<u32x4 *>(reinterpret_cast<unsigned char *>(obase) + 16 * (size_t)idx));
         }
         flushed = end4;
         __builtin_amdgcn_wave_barrier();
@@ -509,8 +540,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     b_cur = b_next;
   }
   // the last, incomplete line (its other elements belong to the next wavefront)
-  if constexpr (STAGES >= 5)
-    for (uint32_t p = kSlot * flushed + lane; p < run; p += 64) obase[p] = ring[p & (kRingElems - 1)];
+  for (uint32_t p = kSlot * flushed + lane; p < run; p += 64) obase[p] = ring[p & (kRingElems - 1)];
 }
 
 // ---- tile variant: any length.  One pass of 8 steps per wavefront, compacted in LDS at
@@ -528,7 +558,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
                                                              const T *src,
                                                              const uint8_t *mask, int64_t n,
                                                              uint32_t ntiles, uint32_t *ticket,
-                                                             uint64_t *status) {
+                                                             uint64_t *status, uint32_t max_rounds) {
   constexpr int64_t kTileElems = (int64_t)kWaveElems * WAVES;
   constexpr uint32_t kSlot = 16u / sizeof(T);  // elements per 16-byte store
   __shared__ MsShared<WAVES, T> sh;
@@ -541,6 +571,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
                   : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t tile = sh.tile;
+  if (tile >= ntiles) return;  // workgroup-uniform; only with a ticket counter that is not ours alone
   // tile bases are wavefront-uniform; everything per lane is a 32-bit offset
   const int64_t start = (int64_t)tile * kTileElems;
   const uint8_t *mask_tile = mask + start;
@@ -589,7 +620,9 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
       }
     }
   }
-  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &sh.base);
+  const int64_t base = tile_prefix(status, ticket, tile, ntiles, tile_total, n, max_rounds, d_count,
+                                   &sh.base);
+  if (base < 0) return;  // workgroup-uniform: the look-back was abandoned
 
   // ---- 3. compact in LDS, write aligned 16-byte packs; the ragged ends go out element by
   //         element: their neighbours belong to other wavefronts.
@@ -639,7 +672,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
 template <bool STRIDED, typename T>
 __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     T *out, int64_t *d_count, const T *src, const uint8_t *mask, int64_t n,
-    uint32_t ntiles, uint32_t *ticket, uint64_t *status, MsGeom g) {
+    uint32_t ntiles, uint32_t *ticket, uint64_t *status, uint32_t max_rounds, MsGeom g) {
   constexpr int kWaveSpan = 64 * kScalarSteps;
   constexpr int kTileElems = kWaveSpan * kScalarWaves;
 
@@ -655,6 +688,7 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
                  : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t tile = s_tile;
+  if (tile >= ntiles) return;  // workgroup-uniform; only with a ticket counter that is not ours alone
   const int64_t wstart = (int64_t)tile * kTileElems + (int64_t)wave * kWaveSpan;
 
   bool sel[kScalarSteps];
@@ -700,7 +734,9 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
 #pragma unroll
   for (int k = 0; k < kScalarSteps; ++k)
     if (sel[k]) vals[k] = src[soff[k]];
-  const int64_t base = tile_prefix(status, tile, ntiles, tile_total, d_count, &s_base);
+  const int64_t base = tile_prefix(status, ticket, tile, ntiles, tile_total, n, max_rounds, d_count,
+                                   &s_base);
+  if (base < 0) return;  // workgroup-uniform: the look-back was abandoned
   const int64_t wpos = base + wave_base;
 #pragma unroll
   for (int k = 0; k < kScalarSteps; ++k)

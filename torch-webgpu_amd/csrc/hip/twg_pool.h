@@ -19,7 +19,7 @@
 //   bool done(Event e)                     has the event completed?  never blocks
 //   void wait(Event e)
 //   void destroy(Event e)
-//   void sync_library_stream()
+//   int  sync_library_stream()              0, or an error code
 #pragma once
 
 #include <stddef.h>
@@ -65,7 +65,7 @@ class BlockPool {
     const size_t want = pool_round_size(n);
     std::lock_guard<std::mutex> lk(mu_);
     st_.n_allocs++;
-    reap_locked(false);
+    reap_locked(kPoll);
     // Best fit: the smallest cached block that is large enough, as long as it wastes at
     // most a quarter of itself (small blocks must match exactly).
     auto it = free_.lower_bound(want);
@@ -85,11 +85,16 @@ class BlockPool {
     int rc = Backend::alloc(&d, want);
     if (rc == Backend::kOutOfMemory) {
       // Everything cached or pending was freed by its owner; wait for the work that may
-      // still touch those blocks, hand them back to the driver and try once more.
-      Backend::sync_library_stream();
-      reap_locked(true);
-      release_cached_locked();
-      rc = Backend::alloc(&d, want);
+      // still touch those blocks, hand them back to the driver and try once more.  Blocks
+      // held for a stream that was being captured stay where they are: nothing here has
+      // waited for that stream, a graph captured with such a block may still replay into
+      // it, and releasing memory during a capture is not allowed.  Only empty_cache(),
+      // which the caller invokes knowing that, lets them go.
+      if (Backend::sync_library_stream() == 0) {
+        reap_locked(kWaitEvents);
+        release_cached_locked();
+        rc = Backend::alloc(&d, want);
+      }
     }
     if (rc != 0) return rc;
     st_.n_device_mallocs++;
@@ -146,9 +151,10 @@ class BlockPool {
 
   // Return every unused block to the driver, pending ones included (their work is waited for).
   int empty_cache() {
-    Backend::sync_library_stream();
+    const int rc = Backend::sync_library_stream();
+    if (rc != 0) return rc;
     std::lock_guard<std::mutex> lk(mu_);
-    reap_locked(true);
+    reap_locked(kEverything);
     return release_cached_locked();
   }
 
@@ -169,12 +175,15 @@ class BlockPool {
     bool held;  // a stream could not take an event: only empty_cache() lets the block go
   };
 
-  // Move the pending blocks whose events have completed to the free lists.  wait = true:
-  // wait for every event and take the held blocks too (the caller has synchronised).
-  void reap_locked(bool wait) {
+  // Move pending blocks to the free lists.  kPoll: those whose events have completed, never
+  // blocking.  kWaitEvents: wait for the events; held blocks (no event could be recorded)
+  // stay pending.  kEverything: held blocks too (empty_cache: the caller vouches for them).
+  enum Reap { kPoll, kWaitEvents, kEverything };
+  void reap_locked(Reap mode) {
+    const bool wait = mode != kPoll;
     for (size_t i = 0; i < pending_.size();) {
       Pending &pd = pending_[i];
-      bool ready = wait || !pd.held;
+      bool ready = mode == kEverything || !pd.held;
       for (size_t k = 0; k < pd.events.size() && ready; ++k) {
         if (wait) {
           Backend::wait(pd.events[k]);

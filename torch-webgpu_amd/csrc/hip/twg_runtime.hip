@@ -97,7 +97,7 @@ struct HipPoolBackend {
   }
   static void wait(hipEvent_t e) { (void)hipEventSynchronize(e); }
   static void destroy(hipEvent_t e) { (void)hipEventDestroy(e); }
-  static void sync_library_stream() { (void)hipStreamSynchronize(rt().stream); }
+  static int sync_library_stream() { return (int)hipStreamSynchronize(rt().stream); }
 };
 
 BlockPool<HipPoolBackend> &pool() {
@@ -579,6 +579,10 @@ const char *twg_error_string(int code) {
     case TWG_E_SCRATCH_SMALL: return "twg: scratch buffer too small";
     case TWG_E_OVERLAP: return "twg: overlapping ranges";
     case TWG_E_TOO_LARGE: return "twg: input larger than this entry point's fixed limit";
+    case TWG_E_BUSY: return "twg: the library's static scratch is still in use by a call on another stream";
+    case TWG_E_WAIT_ABANDONED:
+      return "twg: masked_select gave up waiting for a tile that never published (scratch shared by "
+             "two launches in flight, or overwritten under a running one)";
     case -1000: return "twg: not initialised";
     default: break;
   }
@@ -883,6 +887,7 @@ int twg_masked_select_count(void *out, int64_t *count_host, const void *src, int
   }
   mailbox_give_back(st, mb);
   if (rc) return rc;
+  if (k < 0) return TWG_E_WAIT_ABANDONED;  // the kernel's sentinel: no count to report
   *count_host = k;
   return 0;
 }

@@ -55,6 +55,11 @@ def _install_repr():
 
 _install_repr()
 
-from .compiler import webgpu_backend  # noqa: E402,F401  (python/torch_webgpu/__init__.py:15)
+from .compiler.webgpu_compiler import webgpu_backend  # noqa: E402,F401  (python/torch_webgpu/__init__.py:15)
 
-__all__ = ["webgpu", "webgpu_backend"]
+# The reference lists "webgpu_ops" in __all__ (python/torch_webgpu/__init__.py:17) without
+# defining it; here the name is the namespace of the webgpu:: operators, so that
+# `from torch_webgpu import *` works.
+webgpu_ops = torch.ops.webgpu
+
+__all__ = ["webgpu", "webgpu_backend", "webgpu_ops"]

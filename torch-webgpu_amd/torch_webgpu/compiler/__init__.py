@@ -62,7 +62,11 @@ def fuse_add_relu(gm: torch.fx.GraphModule) -> int:
         src = node.args[0]
         if not isinstance(src, torch.fx.Node) or not _is_add(src) or len(src.users) != 1:
             continue
-        with gm.graph.inserting_before(node):
+        # The fused node takes the add's place, not the relu's: Dynamo graphs are not
+        # functionalized, so an in-place op on one of the add's operands may sit between the
+        # two (`s = a + b; a.mul_(2); relu(s)`), and the operands must be read where the add
+        # read them.  Moving the relu up is safe because the add has no other user.
+        with gm.graph.inserting_before(src):
             new = gm.graph.call_function(add_relu, args=tuple(src.args))
         new.meta = dict(node.meta)
         node.replace_all_uses_with(new)

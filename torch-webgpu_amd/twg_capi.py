@@ -25,6 +25,7 @@ DTYPES = {torch.bool: 0, torch.uint8: 1, torch.int32: 2, torch.int64: 3, torch.f
 
 E_INVALID_ARG, E_UNSUPPORTED, E_SCRATCH_SMALL = -1, -2, -3
 E_TOO_LARGE = -5
+E_BUSY, E_WAIT_ABANDONED = -6, -7
 MS_STATIC_MAX_NUMEL = 1 << 30
 
 
@@ -63,7 +64,7 @@ SYMBOLS = [
     "twg_add_relu_f32", "twg_unary_f32", "twg_copy_strided", "twg_cast",
     "twg_eq_f32", "twg_ne_scalar_f32", "twg_and_u8",
     "twg_masked_select_scratch_bytes", "twg_masked_select_f32", "twg_masked_select_count",
-    "twg_masked_select_f32_static",
+    "twg_masked_select_f32_static", "twg_masked_select_f32_wait_probe",
     "twg_eq", "twg_ne_scalar", "twg_and", "twg_abs",
 ]
 
@@ -121,6 +122,8 @@ def load():
     L.twg_masked_select_scratch_bytes.restype = sz
     L.twg_masked_select_f32.argtypes = [vp, vp, vp, vp, ip, vp, sz, vp]
     L.twg_masked_select_f32_static.argtypes = [vp, vp, vp, vp, ip, vp]
+    L.twg_masked_select_f32_wait_probe.argtypes = [vp, vp, vp, vp, ip, vp, sz, ctypes.c_uint32,
+                                                   ctypes.c_uint32, vp]
     L.twg_masked_select_count.argtypes = [vp, ctypes.POINTER(ctypes.c_int64), vp, i32, vp, ip, vp, sz, vp]
     L.twg_eq.argtypes = [vp, vp, vp, i32, ip, vp]
     L.twg_ne_scalar.argtypes = [vp, vp, i32, ctypes.c_double, i64, ip, vp]

@@ -73,6 +73,16 @@ def bernoulli_mask(n, p, seed=5):
     return torch.rand(n, generator=g, dtype=torch.float32) < p
 
 
+def alternating_density_mask(n, span=8192, p_lo=0.01, p_hi=0.9, seed=7):
+    """Spans of `span` elements that alternate between Bernoulli(p_lo) and Bernoulli(p_hi):
+    with span = 8192 (one wavefront's share of a masked_select tile) neighbouring
+    wavefronts of one tile take the gather path and the streaming loop in turn."""
+    g = _gen(seed)
+    u = torch.rand(n, generator=g, dtype=torch.float32)
+    hi = (torch.arange(n, dtype=torch.int64) // span) % 2 == 1
+    return torch.where(hi, u < p_hi, u < p_lo)
+
+
 def clustered_mask(n, mean_run=4096, seed=6):
     """Config 5 clustered mask: alternating runs of true/false whose lengths are
     geometric with the given mean."""
