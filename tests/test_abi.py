@@ -87,7 +87,7 @@ def test_masked_select_scratch_covers_every_launch_variant():
 
 HOT_PATH_OPS = [
     "empty.memory_format", "empty_strided", "as_strided", "resize_", "view", "_reshape_alias",
-    "copy_", "_copy_from", "_copy_from_and_resize",
+    "copy_", "_copy_from", "_copy_from_and_resize", "to.device",
     "add.out", "mul.out", "relu", "relu_", "relu.out", "gelu", "gelu.out", "silu", "silu.out",
     "abs.out", "eq.Tensor", "eq.Tensor_out", "ne.Scalar", "ne.Scalar_out",
     "bitwise_and.Tensor", "bitwise_and.Tensor_out", "masked_select", "masked_select.out",

@@ -13,6 +13,8 @@
 
 #include <ATen/MemoryOverlap.h>
 
+#include <ATen/NativeFunctions.h>
+
 #include "twg_torch.h"
 
 namespace torch_webgpu {
@@ -188,9 +190,18 @@ at::Scalar _local_scalar_dense(const at::Tensor &self) {
   return host.item();
 }
 
+// csrc/ops/copy.cpp:172-181,188: the reference registers aten::to.device for its backend and
+// hands it straight to ATen's composite implementation, which is also what runs without the
+// registration; kept so that the dispatch table of the backend matches the reference's.
+at::Tensor to_device(const at::Tensor &self, at::Device device, at::ScalarType dtype,
+                     bool non_blocking, bool copy, std::optional<c10::MemoryFormat> memory_format) {
+  return at::native::to(self, device, dtype, non_blocking, copy, memory_format);
+}
+
 }  // namespace ops
 
 TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
+  m.impl("to.device", TORCH_FN(ops::to_device));
   m.impl("copy_", TORCH_FN(ops::copy_));
   m.impl("_copy_from", TORCH_FN(ops::_copy_from));
   m.impl("_copy_from_and_resize", TORCH_FN(ops::_copy_from_and_resize));
