@@ -286,6 +286,12 @@ def test_add_transposed_operand(twg, rows, cols):
     ((4, 3, 23, 100), (2, 0, 3, 1)), ((3, 5, 9, 33), (0, 2, 3, 1)), ((2, 2, 7, 250), (2, 0, 3, 1)),
     ((6, 3, 224), (0, 2, 1)), ((2, 31, 40), (0, 2, 1)), ((16, 3, 224, 96), (2, 0, 3, 1)),
     ((40, 3, 510), (0, 2, 1)),
+    # short output rows (fewer than 256 elements) with the operand's unit stride along a
+    # dimension beyond the second: the two innermost output dimensions walked as one, aligned
+    # and ragged, one or two batch dimensions, merged extents that end inside a tile
+    ((8, 130, 64, 64), (3, 2, 0, 1)), ((3, 40, 9, 64), (3, 2, 0, 1)), ((5, 33, 7, 50), (3, 2, 0, 1)),
+    ((4, 64, 10, 96), (2, 3, 0, 1)), ((2, 3, 70, 5, 24), (0, 4, 3, 1, 2)), ((37, 11, 20), (2, 1, 0)),
+    ((2, 100, 3, 85), (3, 2, 0, 1)),
 ])
 def test_add_permuted_operand_tiles(twg, shape, order):
     # `a` is stored with its dimensions in `order` (outermost first) and viewed in the logical

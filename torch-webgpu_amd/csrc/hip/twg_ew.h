@@ -472,10 +472,12 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
   const uint32_t chunk = blockIdx.x - row * g.chunks_per_row;
   int64_t off_o = 0, off_a = 0, off_b = 0;
   {
-    int64_t r = row;
+    // (row indices fit 32 bits, the grid does: 32-bit divisions cost a third of 64-bit ones)
+    uint32_t r = row;
     for (int d = 0; d < g.nouter; ++d) {
-      const int64_t q = r / g.oshape[d];
-      const int64_t c = r - q * g.oshape[d];
+      const uint32_t extent = (uint32_t)g.oshape[d];
+      const uint32_t q = r / extent;
+      const int64_t c = r - q * extent;
       r = q;
       off_o += c * g.ostride[0][d];
       off_a += c * g.ostride[1][d];
@@ -532,11 +534,57 @@ struct TileGeom {
   // the other operands.  psplit == 1: t is one dimension.
   int64_t sp[3];
   uint32_t psplit;
+  // ew_tile_vec / ew_tile_any: dimension 0 may be the product of two dimensions, the inner one
+  // of extent n0in (strides s0) and the next one (strides s1), that lie back to back in the
+  // memory of the output and of the operands that are not transposed (their offset along
+  // dimension 0 is the index itself) but not in the transposed operands, whose row r sits at
+  // (r % n0in) * s0 + (r / n0in) * s1.  n0in == 0: dimension 0 is one dimension.
+  uint32_t n0in;
+  int64_t s1[3];
   uint32_t tiles0, tilest; // tile counts
+  // ew_tile_vec / ew_tile_any: 0, or the number of (tile along dimension 0, batch index) pairs
+  // when the tiles that follow one another along t are to run on one XCD (tile_of_block)
+  uint32_t ngroups;
   int32_t nbatch;          // remaining dimensions
   int64_t bshape[TWG_MAX_DIMS - 2];
   int64_t bstride[3][TWG_MAX_DIMS - 2];
 };
+
+// Offset of row r (an index along dimension 0) of a transposed operand.
+__device__ __forceinline__ int64_t tile_row_off(const TileGeom &g, int o, int64_t r) {
+  if (g.n0in == 0) return r * g.s0[o];
+  const uint32_t q = (uint32_t)r / g.n0in;
+  const uint32_t rem = (uint32_t)r - q * g.n0in;
+  return (int64_t)rem * g.s0[o] + (int64_t)q * g.s1[o];
+}
+
+// Which tile a workgroup takes.  Plain order: tiles along dimension 0 first, then along t,
+// then the batch.  Where the pieces of a transposed operand do not start and end on
+// 128-byte lines (a row pitch of 197 or 56 elements), tiles that are neighbours along t
+// read the same lines, and in the plain order they run on different XCDs, each of which
+// fetches the line into its own L2 (measured: 1.9-2.1 times the operand's bytes fetched).
+// Workgroups are dealt to the 8 XCDs round-robin by their index, so with ngroups set the
+// index is decoded as (XCD, position on that XCD) and each XCD walks along t through one
+// (tile along dimension 0, batch index) pair after the other: the second reader of a line
+// finds it in the L2 its neighbour filled.  Returns false for the workgroups that pad the
+// grid to a multiple of 8 pairs.
+__device__ __forceinline__ bool tile_of_block(const TileGeom &g, uint32_t bid, uint32_t &t0i,
+                                              uint32_t &tti, int64_t &r) {
+  if (g.ngroups == 0) {
+    t0i = bid % g.tiles0;
+    bid /= g.tiles0;
+    tti = bid % g.tilest;
+    r = bid / g.tilest;
+    return true;
+  }
+  const uint32_t xcd = bid & 7u, k = bid >> 3;
+  tti = k % g.tilest;
+  const uint32_t grp = (k / g.tilest) * 8u + xcd;
+  if (grp >= g.ngroups) return false;
+  t0i = grp % g.tiles0;
+  r = grp / g.tiles0;
+  return true;
+}
 
 // Lane x (0..63) runs along dimension 0, the 4 wavefronts and 16 steps cover 64
 // positions along t.  An operand marked *_T has its unit stride along t: it is
@@ -554,8 +602,9 @@ __global__ __launch_bounds__(kThreads) void ew_tile(TO *out, const TA *a, const 
   int64_t r = bid / g.tilest;
   int64_t off_o = 0, off_a = 0, off_b = 0;
   for (int d = 0; d < g.nbatch; ++d) {
-    const int64_t q = r / g.bshape[d];
-    const int64_t c = r - q * g.bshape[d];
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = (uint32_t)r / extent;  // batch indices fit 32 bits, the grid does
+    const int64_t c = (uint32_t)r - q * extent;
     r = q;
     off_o += c * g.bstride[0][d];
     off_a += c * g.bstride[1][d];
@@ -624,8 +673,10 @@ __global__ __launch_bounds__(kThreads) void ew_tile(TO *out, const TA *a, const 
 // 256 x 32 tiles) runs 1.2-1.5 points of HBM peak faster without them (77.9% -> 79.3%).
 // The operands that need no transpose are requested first: their loads do not depend on
 // LDS, and ahead of the transposed operand's scatter they are in flight while it waits.
-template <bool FULL, int NIN, bool A_T, bool B_T, int TD0, int TT, int THREADS, typename Op,
-          typename TO, typename TA, typename TB, typename SA, typename SB>
+// SPLIT0: dimension 0 is the product of two dimensions (TileGeom::n0in); kept out of the plain
+// body at compile time, where even a never-taken branch per row cost a point on config 3b.
+template <bool FULL, bool SPLIT0, int NIN, bool A_T, bool B_T, int TD0, int TT, int THREADS,
+          typename Op, typename TO, typename TA, typename TB, typename SA, typename SB>
 __device__ __forceinline__ void tile_vec_body(TO *out, const TA *a, const TB *b, const TileGeom &g,
                                               const Op &op, int64_t base0, int64_t baset,
                                               SA &sa, SB &sb) {
@@ -661,7 +712,8 @@ __device__ __forceinline__ void tile_vec_body(TO *out, const TA *a, const TB *b,
       for (int p = 0; p < kPassT; ++p) {
         const int64_t r0 = base0 + ty + kRowsT * p;
         if (FULL || (r0 < g.n0 && tt < g.nt))
-          v[p] = load_pack<true>(reinterpret_cast<const PA *>(a + r0 * g.s0[1] + tt));
+          v[p] = load_pack<true>(reinterpret_cast<const PA *>(
+              a + (SPLIT0 ? tile_row_off(g, 1, r0) : r0 * g.s0[1]) + tt));
       }
 #pragma unroll
       for (int p = 0; p < kPassT; ++p) {
@@ -678,7 +730,8 @@ __device__ __forceinline__ void tile_vec_body(TO *out, const TA *a, const TB *b,
       for (int p = 0; p < kPassT; ++p) {
         const int64_t r0 = base0 + ty + kRowsT * p;
         if (FULL || (r0 < g.n0 && tt < g.nt))
-          v[p] = load_pack<true>(reinterpret_cast<const PB *>(b + r0 * g.s0[2] + tt));
+          v[p] = load_pack<true>(reinterpret_cast<const PB *>(
+              b + (SPLIT0 ? tile_row_off(g, 2, r0) : r0 * g.s0[2]) + tt));
       }
 #pragma unroll
       for (int p = 0; p < kPassT; ++p) {
@@ -716,15 +769,17 @@ __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, con
   __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
   __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
 
+  // (this kernel only gets line-aligned pieces, so its tiles are always dealt in plain order)
   uint32_t bid = blockIdx.x;
   const uint32_t t0i = bid % g.tiles0;
   bid /= g.tiles0;
   const uint32_t tti = bid % g.tilest;
-  int64_t r = bid / g.tilest;
+  uint32_t r = bid / g.tilest;
   int64_t off_o = 0, off_a = 0, off_b = 0;
   for (int d = 0; d < g.nbatch; ++d) {
-    const int64_t q = r / g.bshape[d];
-    const int64_t c = r - q * g.bshape[d];
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = r / extent;
+    const int64_t c = r - q * extent;
     r = q;
     off_o += c * g.bstride[0][d];
     off_a += c * g.bstride[1][d];
@@ -733,12 +788,16 @@ __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, con
   const int64_t base0 = (int64_t)t0i * TD0;
   const int64_t baset = (int64_t)tti * TT;
   // workgroup-uniform: whole tiles take the unpredicated body
-  if (base0 + TD0 <= g.n0 && baset + TT <= g.nt)
-    tile_vec_body<true, NIN, A_T, B_T, TD0, TT, THREADS>(out + off_o, a + off_a, b + off_b, g, op,
-                                                         base0, baset, sa, sb);
-  else
-    tile_vec_body<false, NIN, A_T, B_T, TD0, TT, THREADS>(out + off_o, a + off_a, b + off_b, g, op,
-                                                          base0, baset, sa, sb);
+  const bool whole = base0 + TD0 <= g.n0 && baset + TT <= g.nt;
+#define TWG_TILE_BODY(FULL, SPLIT0)                                                              \
+  tile_vec_body<FULL, SPLIT0, NIN, A_T, B_T, TD0, TT, THREADS>(out + off_o, a + off_a, b + off_b, g, \
+                                                               op, base0, baset, sa, sb)
+  if (g.n0in == 0) {
+    if (whole) TWG_TILE_BODY(true, false); else TWG_TILE_BODY(false, false);
+  } else {
+    if (whole) TWG_TILE_BODY(true, true); else TWG_TILE_BODY(false, true);
+  }
+#undef TWG_TILE_BODY
 }
 
 // The same tile kernel without its alignment conditions.  Wide global loads and stores need
@@ -750,9 +809,14 @@ __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, con
 // the output rows are addressed by (t / p, t % p).
 typedef uint32_t U32x4A4 __attribute__((ext_vector_type(4), aligned(4)));
 
-template <typename T>
+template <bool NT = true, typename T>
 __device__ __forceinline__ Pack<T, 4> load4_any(const T *p) {
-  const U32x4A4 r = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4 *>(p));
+  U32x4A4 r;
+  if constexpr (NT) {
+    r = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4 *>(p));
+  } else {
+    r = *reinterpret_cast<const U32x4A4 *>(p);
+  }
   Pack<T, 4> out;
   __builtin_memcpy(&out, &r, 16);
   return out;
@@ -764,9 +828,9 @@ __device__ __forceinline__ void store4_any(T *p, const Pack<T, 4> &x) {
   __builtin_nontemporal_store(r, reinterpret_cast<U32x4A4 *>(p));
 }
 // up to 4 elements from p, `valid` of them inside the extent
-template <typename T>
+template <bool NT = true, typename T>
 __device__ __forceinline__ Pack<T, 4> load4_edge(const T *p, int64_t valid) {
-  if (valid >= 4) return load4_any(p);
+  if (valid >= 4) return load4_any<NT>(p);
   Pack<T, 4> out;
 #pragma unroll
   for (int c = 0; c < 4; ++c) out.v[c] = c < valid ? p[c] : T();
@@ -785,15 +849,14 @@ __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, con
   __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
   __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
 
-  uint32_t bid = blockIdx.x;
-  const uint32_t t0i = bid % g.tiles0;
-  bid /= g.tiles0;
-  const uint32_t tti = bid % g.tilest;
-  int64_t r = bid / g.tilest;
+  uint32_t t0i, tti;
+  int64_t r;
+  if (!tile_of_block(g, blockIdx.x, t0i, tti, r)) return;  // workgroup-uniform
   int64_t off_o = 0, off_a = 0, off_b = 0;
   for (int d = 0; d < g.nbatch; ++d) {
-    const int64_t q = r / g.bshape[d];
-    const int64_t c = r - q * g.bshape[d];
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = (uint32_t)r / extent;  // batch indices fit 32 bits, the grid does
+    const int64_t c = (uint32_t)r - q * extent;
     r = q;
     off_o += c * g.bstride[0][d];
     off_a += c * g.bstride[1][d];
@@ -814,7 +877,8 @@ __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, con
 #pragma unroll
       for (int p = 0; p < kPassT; ++p) {
         const int64_t d0 = base0 + ty + kRowsT * p;
-        if (d0 < g.n0 && left > 0) v[p] = load4_edge(a + off_a + d0 * g.s0[1] + tt, left);
+        // (default caching: a neighbouring tile reads the other part of these lines)
+        if (d0 < g.n0 && left > 0) v[p] = load4_edge<false>(a + off_a + tile_row_off(g, 1, d0) + tt, left);
       }
 #pragma unroll
       for (int p = 0; p < kPassT; ++p) {
@@ -830,7 +894,7 @@ __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, con
 #pragma unroll
       for (int p = 0; p < kPassT; ++p) {
         const int64_t d0 = base0 + ty + kRowsT * p;
-        if (d0 < g.n0 && left > 0) v[p] = load4_edge(b + off_b + d0 * g.s0[2] + tt, left);
+        if (d0 < g.n0 && left > 0) v[p] = load4_edge<false>(b + off_b + tile_row_off(g, 2, d0) + tt, left);
       }
 #pragma unroll
       for (int p = 0; p < kPassT; ++p) {
@@ -917,8 +981,8 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   uint32_t nrows = 1;
   int d_first = 0;
   if (rows > 1) {
-    const int64_t q = r / g.tilest;
-    const int64_t row0 = (r - q * g.tilest) * rows;
+    const uint32_t q = (uint32_t)r / g.tilest;
+    const int64_t row0 = (int64_t)((uint32_t)r - q * g.tilest) * rows;
     r = q;
     nrows = (uint32_t)(g.bshape[0] - row0 < (int64_t)rows ? g.bshape[0] - row0 : (int64_t)rows);
     off_o = row0 * g.bstride[0][0];
@@ -927,8 +991,9 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
     d_first = 1;
   }
   for (int d = d_first; d < g.nbatch; ++d) {
-    const int64_t q = r / g.bshape[d];
-    const int64_t c = r - q * g.bshape[d];
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = (uint32_t)r / extent;  // batch indices fit 32 bits, the grid does
+    const int64_t c = (uint32_t)r - q * extent;
     r = q;
     off_o += c * g.bstride[0][d];
     off_a += c * g.bstride[1][d];
@@ -939,59 +1004,81 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)tx_elems ? g.n0 - x0 : (int64_t)tx_elems);
   const uint32_t strip = nx * P;  // consecutive elements of a deinterleaved operand
   const uint32_t pitch = (strip + 3u) & ~3u;  // of a strip in LDS
-  if constexpr (A_D) {
-    const TA *src = a + off_a + x0 * (int64_t)P;
-    for (uint32_t i = 4 * threadIdx.x; i < nrows * pitch; i += 4 * kThreads) {
-      const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
-      if (j < strip)
-        *reinterpret_cast<PA *>(&sa[i]) = load4_edge(src + row * g.bstride[1][0] + j, (int64_t)strip - j);
+  // Loads are issued kDeintUnroll at a time before the first of them is used: one load per
+  // trip, waited for at once, left a block with a single request in flight per lane.
+  constexpr uint32_t kU = 4;
+  auto park = [&](auto *lds, const auto *src, int64_t row_stride) {
+    using P4 = Pack<std::remove_cv_t<std::remove_pointer_t<decltype(src)>>, 4>;
+    const uint32_t total = nrows * pitch;
+    for (uint32_t i0 = 4 * threadIdx.x; i0 < total; i0 += 4 * kThreads * kU) {
+      P4 v[kU];
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * 4 * kThreads;
+        const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
+        if (i < total && j < strip) v[u] = load4_edge(src + row * row_stride + j, (int64_t)strip - j);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * 4 * kThreads;
+        const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
+        if (i < total && j < strip) *reinterpret_cast<P4 *>(&lds[i]) = v[u];
+      }
     }
-  }
-  if constexpr (NIN == 2 && B_D) {
-    const TB *src = b + off_b + x0 * (int64_t)P;
-    for (uint32_t i = 4 * threadIdx.x; i < nrows * pitch; i += 4 * kThreads) {
-      const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
-      if (j < strip)
-        *reinterpret_cast<PB *>(&sb[i]) = load4_edge(src + row * g.bstride[2][0] + j, (int64_t)strip - j);
-    }
-  }
+  };
+  if constexpr (A_D) park(sa, a + off_a + x0 * (int64_t)P, g.bstride[1][0]);
+  if constexpr (NIN == 2 && B_D) park(sb, b + off_b + x0 * (int64_t)P, g.bstride[2][0]);
   __syncthreads();
   const uint32_t packs = (nx + 3) / 4;  // per channel
   const uint32_t per_row = packs * P;
-  for (uint32_t idx = threadIdx.x; idx < nrows * per_row; idx += kThreads) {
-    const uint32_t row = rows > 1 ? idx / per_row : 0u, rem = idx - row * per_row;
-    const uint32_t c = rem / packs, j = rem - c * packs;
-    const uint32_t x = 4 * j;
-    const int64_t left = (int64_t)nx - x;
-    PA va;
-    PB vb;
-    if constexpr (A_D) {
-      const TA *l = sa + row * pitch;
+  const uint32_t total = nrows * per_row;
+  for (uint32_t idx0 = threadIdx.x; idx0 < total; idx0 += kThreads * kU) {
+    PA va[kU];
+    PB vb[kU];
+    uint32_t row[kU], c[kU], x[kU];
+    // the operands that come straight from memory first, all kU of them
 #pragma unroll
-      for (int k = 0; k < 4; ++k) va.v[k] = k < left ? l[(x + k) * P + c] : TA();
-    } else {
-      va = load4_edge(a + off_a + row * g.bstride[1][0] + x0 + x + (int64_t)c * g.st[1], left);
-    }
-    if constexpr (NIN == 2) {
-      if constexpr (B_D) {
-        const TB *l = sb + row * pitch;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) vb.v[k] = k < left ? l[(x + k) * P + c] : TB();
-      } else {
-        vb = load4_edge(b + off_b + row * g.bstride[2][0] + x0 + x + (int64_t)c * g.st[2], left);
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t idx = idx0 + u * kThreads;
+      row[u] = rows > 1 ? idx / per_row : 0u;
+      const uint32_t rem = idx - row[u] * per_row;
+      c[u] = rem / packs;
+      x[u] = 4 * (rem - c[u] * packs);
+      if (idx < total) {
+        const int64_t left = (int64_t)nx - x[u];
+        if constexpr (!A_D)
+          va[u] = load4_edge(a + off_a + row[u] * g.bstride[1][0] + x0 + x[u] + (int64_t)c[u] * g.st[1], left);
+        if constexpr (NIN == 2 && !B_D)
+          vb[u] = load4_edge(b + off_b + row[u] * g.bstride[2][0] + x0 + x[u] + (int64_t)c[u] * g.st[2], left);
       }
     }
-    PO o;
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
-    TO *dst = out + off_o + row * g.bstride[0][0] + x0 + x + (int64_t)c * g.st[0];
-    if (left >= 4) {
-      store4_any(dst, o);
-    } else {
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t idx = idx0 + u * kThreads;
+      if (idx >= total) continue;
+      const int64_t left = (int64_t)nx - x[u];
+      if constexpr (A_D) {
+        const TA *l = sa + row[u] * pitch;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) va[u].v[k] = k < left ? l[(x[u] + k) * P + c[u]] : TA();
+      }
+      if constexpr (NIN == 2 && B_D) {
+        const TB *l = sb + row[u] * pitch;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) vb[u].v[k] = k < left ? l[(x[u] + k) * P + c[u]] : TB();
+      }
+      PO o;
 #pragma unroll
       for (int k = 0; k < 4; ++k)
-        if (k < left) dst[k] = o.v[k];
+        o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va[u].v[k], NIN == 2 ? vb[u].v[k] : TB());
+      TO *dst = out + off_o + row[u] * g.bstride[0][0] + x0 + x[u] + (int64_t)c[u] * g.st[0];
+      if (left >= 4) {
+        store4_any(dst, o);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (k < left) dst[k] = o.v[k];
+      }
     }
   }
 }
@@ -1250,10 +1337,13 @@ int launch_rows(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStre
 
 // t: the dimension the transposed operands have their unit stride along; or, with pin >= 1,
 // the outer one of two dimensions (t, pin) that lie back to back in those operands' memory
-// (unit stride along pin, stride shape[pin] along t) and are walked as one.
+// (unit stride along pin, stride shape[pin] along t) and are walked as one.  merge01: the
+// output and the operands that are not transposed are dense across dimensions 0 and 1 (the
+// caller has checked), which are then walked as one dimension of shape[0] * shape[1] elements,
+// so that short rows (64 elements against a 256-wide tile) still move in pieces of 1 KiB.
 template <int NIN, typename Op, typename TO, typename TA, typename TB>
 int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
-                hipStream_t s, int pin = -1) {
+                hipStream_t s, int pin = -1, bool merge01 = false) {
   TileGeom tg{};
   tg.n0 = g.shape[0];
   tg.nt = g.shape[t];
@@ -1262,6 +1352,13 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     tg.s0[o] = g.stride[o][0];
     tg.st[o] = g.stride[o][t];
     tg.sp[o] = 0;
+  }
+  if (merge01) {
+    if (t < 2 || pin >= 0 || g.ndim < 3) return TWG_E_UNSUPPORTED;
+    if (g.shape[0] * g.shape[1] >= (int64_t(1) << 31)) return TWG_E_UNSUPPORTED;
+    tg.n0 = g.shape[0] * g.shape[1];
+    tg.n0in = (uint32_t)g.shape[0];
+    for (int o = 0; o < 3; ++o) tg.s1[o] = g.stride[o][1];
   }
   if (pin >= 1) {
     if (g.shape[t] * g.shape[pin] >= (int64_t(1) << 31)) return TWG_E_UNSUPPORTED;
@@ -1272,12 +1369,20 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
   int64_t batch = 1;
   tg.nbatch = 0;
   for (int d = 1; d < g.ndim; ++d) {
-    if (d == t || d == pin) continue;
+    if (d == t || d == pin || (merge01 && d == 1)) continue;
     tg.bshape[tg.nbatch] = g.shape[d];
     for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
     tg.nbatch++;
     batch *= g.shape[d];
   }
+  // Do the pieces of a transposed operand (32 or 64 elements along t) start and end on
+  // 128-byte lines?  If not, tiles that are neighbours along t share lines.
+  auto ragged = [&](int o, const void *base) {
+    bool lines = reinterpret_cast<uintptr_t>(base) % 128 == 0 && tg.s0[o] % 32 == 0 && tg.s1[o] % 32 == 0;
+    for (int d = 0; d < tg.nbatch && lines; ++d) lines = tg.bstride[o][d] % 32 == 0;
+    return !lines;
+  };
+  const bool ragged_t = (a_t && ragged(1, a)) || (NIN == 2 && b_t && ragged(2, b));
   auto set_tiles = [&](int td0, int tt, unsigned *grid) {
     const int64_t tiles0 = (tg.n0 + td0 - 1) / td0;
     const int64_t tilest = (tg.nt + tt - 1) / tt;
@@ -1285,7 +1390,18 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     if (tiles0 * tilest > INT32_MAX || tiles0 * tilest * batch > INT32_MAX) return false;
     tg.tiles0 = (uint32_t)tiles0;
     tg.tilest = (uint32_t)tilest;
+    tg.ngroups = 0;
     *grid = (unsigned)(tiles0 * tilest * batch);
+    // pieces of a transposed operand that share 128-byte lines with their neighbours along
+    // t: let one XCD walk along t (tile_of_block)
+    if (tilest > 1 && ragged_t) {
+      const int64_t groups = tiles0 * batch;
+      const int64_t padded = (groups + 7) / 8 * 8 * tilest;
+      if (groups <= UINT32_MAX && padded <= INT32_MAX) {
+        tg.ngroups = (uint32_t)groups;
+        *grid = (unsigned)padded;
+      }
+    }
     return true;
   };
   unsigned grid = 0;
@@ -1295,12 +1411,16 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
   if constexpr (sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4) {
     bool ok = tg.n0 % 4 == 0 && tg.nt % 4 == 0 && tg.s0[0] == 1 && tg.st[0] % 4 == 0 &&
               aligned_to(out, 16) && aligned_to(a, 16) && (NIN == 1 || aligned_to(b, 16));
-    ok = ok && (a_t ? (tg.st[1] == 1 && tg.s0[1] % 4 == 0) : (tg.s0[1] == 1 && tg.st[1] % 4 == 0));
+    ok = ok && (a_t ? (tg.st[1] == 1 && tg.s0[1] % 4 == 0 && tg.s1[1] % 4 == 0)
+                    : (tg.s0[1] == 1 && tg.st[1] % 4 == 0));
     if (NIN == 2)
-      ok = ok && (b_t ? (tg.st[2] == 1 && tg.s0[2] % 4 == 0) : (tg.s0[2] == 1 && tg.st[2] % 4 == 0));
+      ok = ok && (b_t ? (tg.st[2] == 1 && tg.s0[2] % 4 == 0 && tg.s1[2] % 4 == 0)
+                      : (tg.s0[2] == 1 && tg.st[2] % 4 == 0));
     for (int d = 0; d < tg.nbatch && ok; ++d)
       for (int o = 0; o <= NIN; ++o) ok = ok && tg.bstride[o][d] % 4 == 0;
-    ok = ok && pin < 0;
+    // (pieces that share lines with their neighbours go to the kernel below, which reads the
+    // transposed operands with default caching and lets one XCD walk along t)
+    ok = ok && pin < 0 && !ragged_t;
     // tile shape by the extent of dimension 0: 256 x 32 from 256 on, 128 x 64 where a 128-wide
     // tile wastes no more lanes than two 64-wide ones (96: 54% -> 6x% of peak), else 64 x 64
     const bool wide = tg.n0 >= 256;
@@ -1366,7 +1486,7 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     }
   }
 
-  if (pin >= 1) return TWG_E_UNSUPPORTED;  // the dword kernel walks one dimension only
+  if (pin >= 1 || merge01) return TWG_E_UNSUPPORTED;  // the dword kernel walks one dimension only
   if (!set_tiles(kTile, kTile, &grid)) return TWG_E_UNSUPPORTED;
   if (a_t && b_t) {
     if constexpr (NIN == 2)
@@ -1390,7 +1510,8 @@ int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool 
     return TWG_E_UNSUPPORTED;
   } else {
     const int64_t P = g.shape[pd];
-    if (P < 2 || P > 32 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
+    // (from 32 elements on, a run of P is a whole 128-byte line and the tile kernels do better)
+    if (P < 2 || P >= 32 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
     auto run_of = [&](int o) { return g.stride[o][pd] == 1 && g.stride[o][0] == P; };
     if (a_d ? !run_of(1) : g.stride[1][0] != 1) return TWG_E_UNSUPPORTED;
     if (NIN == 2 && (b_d ? !run_of(2) : g.stride[2][0] != 1)) return TWG_E_UNSUPPORTED;
@@ -1581,6 +1702,29 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
             g.shape[pd] * g.shape[qd] >= 32) {
           int r = launch_tile<NIN, Op, TO, TA, TB>(out, a, b, g, qd, a_x, b_x, op, s, pd);
           if (r != TWG_E_UNSUPPORTED) return r;
+        }
+      }
+      // (iii-m) the same where the output and the inputs that need no transpose are dense
+      // across dimensions 0 and 1 (and t is a later one): the two are walked as one, so that
+      // a tile covers 256 consecutive output elements however short the rows are, and
+      // consecutive workgroups write consecutive memory across the rows
+      if (g.ndim >= 3 && g.shape[0] >= 4 && g.shape[0] * g.shape[1] >= 128) {
+        int t = -1;
+        for (int d = 2; d < g.ndim && t < 0; ++d) {
+          if (g.shape[d] < 16) continue;
+          if ((sa0 != 0 && sa0 != 1 && g.stride[1][d] == 1) ||
+              (NIN == 2 && sb0 != 0 && sb0 != 1 && g.stride[2][d] == 1))
+            t = d;
+        }
+        if (t > 0) {
+          const bool a_t = sa0 != 0 && sa0 != 1 && g.stride[1][t] == 1;
+          const bool b_t = NIN == 2 && sb0 != 0 && sb0 != 1 && g.stride[2][t] == 1;
+          auto dense01 = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == g.shape[0]; };
+          bool ok = dense01(0) && (a_t || dense01(1)) && (NIN == 1 || b_t || dense01(2));
+          if (ok) {
+            int r = launch_tile<NIN, Op, TO, TA, TB>(out, a, b, g, t, a_t, b_t, op, s, -1, true);
+            if (r != TWG_E_UNSUPPORTED) return r;
+          }
         }
       }
       // (iii) an input with its unit stride along another dimension
