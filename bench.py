@@ -33,6 +33,19 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 
+# Every masked_select launch of the run, by mask, in launch order (run-length encoded in the JSON
+# line as "masked_select_launch_order"): a kernel trace or counter run of this script shows one
+# kernel name for all masks, and this is what tells its dispatches apart.
+MS_LAUNCHES = []
+
+
+def note_ms(name):
+    if MS_LAUNCHES and MS_LAUNCHES[-1][0] == name:
+        MS_LAUNCHES[-1][1] += 1
+    else:
+        MS_LAUNCHES.append([name, 1])
+
+
 class Durations(list):
     """Per-launch durations with room for the back-to-back average."""
     batch_avg = None
@@ -198,6 +211,7 @@ def main():
     def run_ms(mask_buf=None):
         """The op as the dispatcher runs it: compaction with the count handed to the host
         (the call returns once the count is known; the output is stream ordered)."""
+        note_ms("masked_select_p0.50")
         capi.check(L.twg_masked_select_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr, 4,
                                              (mask_buf or d_m).ptr, ctypes.byref(it),
                                              d_scratch.ptr, scratch_bytes, None))
@@ -314,6 +328,7 @@ def main():
         "ops": ops,
         "device": {"name": dev_name, "compute_units": cus},
         "counter_calibration_transfers": cal,
+        "masked_select_launch_order": MS_LAUNCHES,
     }
     print(json.dumps(out), flush=True)
 
@@ -399,11 +414,16 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
     line("add_transposed", lambda: at + c, 12 * n, c_abi("add_transposed"))
     del at, a, c
     src, m = src_h.to("webgpu"), m_h.to("webgpu")
+    note_ms("dispatcher masked_select_p0.50")
     got = torch.masked_select(src, m)
     if got.numel() != k50:
         raise RuntimeError(f"dispatcher masked_select: {got.numel()} != {k50}")
     del got
-    line("masked_select_p0.50", lambda: torch.masked_select(src, m), W.masked_select_bytes(n, k50),
+    def ms_call():
+        note_ms("dispatcher masked_select_p0.50")
+        return torch.masked_select(src, m)
+
+    line("masked_select_p0.50", ms_call, W.masked_select_bytes(n, k50),
          c_abi("masked_select_p0.50", "op_ms_with_count_readback"))
     return res
 
@@ -656,13 +676,15 @@ def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summariz
         d_mask = capi.to_device(m_h)
         del m_h
 
-        def launch():
+        def launch(name=name):
+            note_ms(name)
             capi.check(L.twg_masked_select_f32(d_out.ptr, d_cnt.ptr, d_src.ptr, d_mask.ptr,
                                                ctypes.byref(it), d_scratch.ptr, scratch_bytes, None))
 
         k_host = ctypes.c_int64(-1)
 
-        def full():
+        def full(name=name):
+            note_ms(name)
             capi.check(L.twg_masked_select_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr, 4,
                                                  d_mask.ptr, ctypes.byref(it), d_scratch.ptr,
                                                  scratch_bytes, None))
