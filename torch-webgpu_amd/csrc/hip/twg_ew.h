@@ -1004,8 +1004,8 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)tx_elems ? g.n0 - x0 : (int64_t)tx_elems);
   const uint32_t strip = nx * P;  // consecutive elements of a deinterleaved operand
   const uint32_t pitch = (strip + 3u) & ~3u;  // of a strip in LDS
-  // Loads are issued kDeintUnroll at a time before the first of them is used: one load per
-  // trip, waited for at once, left a block with a single request in flight per lane.
+  // Loads are issued kU at a time before the first of them is used: one load per trip,
+  // waited for at once, left a block with a single request in flight per lane.
   constexpr uint32_t kU = 4;
   auto park = [&](auto *lds, const auto *src, int64_t row_stride) {
     using P4 = Pack<std::remove_cv_t<std::remove_pointer_t<decltype(src)>>, 4>;
@@ -1383,7 +1383,8 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     return !lines;
   };
   const bool ragged_t = (a_t && ragged(1, a)) || (NIN == 2 && b_t && ragged(2, b));
-  auto set_tiles = [&](int td0, int tt, unsigned *grid) {
+  // xcd_walk: only ew_tile_any decodes the block index that way
+  auto set_tiles = [&](int td0, int tt, unsigned *grid, bool xcd_walk = false) {
     const int64_t tiles0 = (tg.n0 + td0 - 1) / td0;
     const int64_t tilest = (tg.nt + tt - 1) / tt;
     if (tiles0 > UINT32_MAX || tilest > UINT32_MAX) return false;
@@ -1394,7 +1395,7 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     *grid = (unsigned)(tiles0 * tilest * batch);
     // pieces of a transposed operand that share 128-byte lines with their neighbours along
     // t: let one XCD walk along t (tile_of_block)
-    if (tilest > 1 && ragged_t) {
+    if (xcd_walk && tilest > 1 && ragged_t) {
       const int64_t groups = tiles0 * batch;
       const int64_t padded = (groups + 7) / 8 * 8 * tilest;
       if (groups <= UINT32_MAX && padded <= INT32_MAX) {
@@ -1434,7 +1435,7 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       bool any = tg.s0[0] == 1 && (a_t ? unit_t(1) : tg.s0[1] == 1);
       if (NIN == 2) any = any && (b_t ? unit_t(2) : tg.s0[2] == 1);
       if (any) {
-        if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid)) return TWG_E_UNSUPPORTED;
+        if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid, true)) return TWG_E_UNSUPPORTED;
         const bool big = g.numel >= (int64_t(1) << 27);
 #define TWG_LAUNCH_TILE_ANY(AT, BT)                                                              \
   do {                                                                                           \
