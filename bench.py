@@ -483,8 +483,8 @@ def first_launches(capi, L, torch, n, launches=40):
 
 def geometry_families(capi, L):
     """add.Tensor on ~2^25 fp32 elements with (a) the second operand broadcast in every possible
-    way over a set of 2- to 4-dimensional shapes and (b) the first operand stored in every
-    permutation of its dimensions.  Reports algorithmic bytes / time as % of the HBM peak: the
+    way over a set of 2- to 4-dimensional shapes, (b) the first operand stored in every
+    permutation of its dimensions and (c) one or both operands slices of a larger storage.  Reports algorithmic bytes / time as % of the HBM peak: the
     slowest patterns and the median of each family.  Median of three batches of 10 launches,
     each batch between one pair of events on the library's stream."""
     import itertools
@@ -559,8 +559,74 @@ def geometry_families(capi, L):
                                      "slowest": rows_[:5], "all": rows_}
     log(f"permutation family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
         f"slowest {rows_[0]['pct_hbm_peak']}%")
+    # (c) the first operand a slice of a larger storage: stepped, shifted or narrowed along one
+    # dimension or all of them (x[:, ::2], x[1:], x[:, :, 3:-2] ...), the second operand and the
+    # output contiguous; and both operands sliced alike
+    def timed_view(shape, storage, starts, steps, both):
+        n = 1
+        for s_ in shape:
+            n *= s_
+        ns = 1
+        for s_ in storage:
+            ns *= s_
+        st_storage = contig(storage)
+        a_st = [st * k for st, k in zip(st_storage, steps)]
+        off = sum(b0 * st for b0, st in zip(starts, st_storage))
+        da, do = capi.DeviceBuffer(4 * ns), capi.DeviceBuffer(4 * n)
+        db = capi.DeviceBuffer(4 * (ns if both else n))
+        b_st = a_st if both else contig(shape)
+        it = capi.make_iter(shape, contig(shape), a_st, b_st)
+        pa, pb = da.ptr + 4 * off, db.ptr + (4 * off if both else 0)
+
+        def run():
+            capi.check(L.twg_add_f32(do.ptr, pa, pb, ctypes.c_float(1.0), ctypes.byref(it), None))
+        for _ in range(3):
+            run()
+        capi.sync()
+        batches = []
+        for _ in range(3):
+            e0, e1 = capi.Event(), capi.Event()
+            e0.record()
+            for _ in range(10):
+                run()
+            e1.record()
+            capi.sync()
+            batches.append(e0.elapsed_ms(e1) / 10)
+        t = statistics.median(batches) / 1e3
+        return round(12 * n / t / 1e9 / HBM_PEAK_GBS * 100, 1), round(t * 1e3, 4)
+
+    rows_ = []
+    for shape in ([4096, 8192], [64, 512, 1024], [32, 16, 256, 256], [8192, 4000]):
+        nd = len(shape)
+        variants = []
+        for d in sorted({0, nd // 2, nd - 1}):
+            for step in (2, 3):
+                storage = list(shape)
+                storage[d] *= step
+                steps = [1] * nd
+                steps[d] = step
+                variants.append((f"dim {d} stepped by {step}", storage, [0] * nd, steps))
+            for pad in (1, 5, 32):
+                storage = list(shape)
+                storage[d] += pad
+                starts = [0] * nd
+                starts[d] = pad if pad == 1 else 0
+                variants.append((f"dim {d} of {storage[d]} " + ("from 1 on" if pad == 1 else f"narrowed by {pad}"),
+                                 storage, starts, [1] * nd))
+        variants.append(("every dim from 1 on, to the last but one", [s_ + 2 for s_ in shape], [1] * nd, [1] * nd))
+        for what, storage, starts, steps in variants:
+            for both in (False, True):
+                pct, ms = timed_view(shape, storage, starts, steps, both)
+                rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "slice": what,
+                              "operands_sliced": "both" if both else "first"})
+    rows_.sort(key=lambda r: r["pct_hbm_peak"])
+    fam["sliced_operands"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
+                              "slowest": rows_[:5], "all": rows_}
+    log(f"slice family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
+        f"slowest {rows_[0]['pct_hbm_peak']}%")
     return {"geometry_families": fam, "elements_per_pattern": "about 2^25", "op": "add.Tensor fp32",
-            "bytes": "4 B per element read per full operand + 4 B written; a broadcast operand counts its own size"}
+            "bytes": "4 B per element read per full operand + 4 B written; a broadcast operand counts its own size; "
+                     "a stepped operand counts the elements used, not the lines touched"}
 
 
 def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summarize,

@@ -316,6 +316,36 @@ def test_add_permuted_operand_tiles(twg, shape, order):
         assert bit_equal(r, torch.relu(a))
 
 
+@pytest.mark.parametrize("rows,cols,pad,start", [
+    (37, 1000, 1, 1), (37, 1000, 5, 0), (50, 1001, 3, 2), (9, 4099, 1, 1), (300, 256, 2, 1),
+    (3, 70001, 7, 3), (64, 999, 0, 0), (130, 66, 1, 1)])
+def test_rows_that_start_anywhere(twg, rows, cols, pad, start):
+    # x[:, 1:], a row pitch that is not a multiple of 4 elements, rows whose length is not one:
+    # the row kernel moves 16-byte packs at 4-byte alignment and finishes each row element by
+    # element.  One or both inputs sliced, the output contiguous or sliced as well, a bias row,
+    # and activations over the same views.
+    import twg_capi as C
+    g = torch.Generator().manual_seed(rows * cols + pad)
+    big_a = torch.randn(rows, cols + pad, generator=g)
+    big_b = torch.randn(rows, cols + pad, generator=g)
+    a = big_a[:, start:start + cols]
+    b = big_b[:, start:start + cols]
+    bc = torch.randn(rows, cols, generator=g)
+    assert bit_equal(H.add(a, bc, alpha=0.5), oracle.add(a, bc, alpha=0.5))
+    assert bit_equal(H.add(bc, a), oracle.add(bc, a))
+    assert bit_equal(H.add(a, b, alpha=-1.5), oracle.add(a, b, alpha=-1.5))
+    out = torch.zeros(rows, cols + pad)[:, start:start + cols]
+    assert bit_equal(H.add(a, b, out=out), oracle.add(a, b))
+    bias = torch.randn(1, cols + pad, generator=g)[:, start:start + cols]
+    assert bit_equal(H.add(a, bias), oracle.add(a, bias))
+    col = torch.randn(rows, 1, generator=g)
+    assert bit_equal(H.add(a, col), oracle.add(a, col))
+    assert bit_equal(_unary(C.UNARY_RELU, a), torch.relu(a))
+    got = _unary(C.UNARY_GELU_ERF, a)
+    assert rel_err_ok(got, closed_form64("gelu_erf", a))[0]
+    assert bit_equal(H.binary("twg_eq_f32", a, b, out_dtype=torch.bool), torch.eq(a, b))
+
+
 def test_add_generic_strides_bruteforce(twg):
     g = torch.Generator().manual_seed(5)
     sizes = [3, 4, 2, 5]

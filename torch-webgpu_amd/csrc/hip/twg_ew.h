@@ -457,14 +457,56 @@ struct RowGeom {
   int64_t ostride[3][TWG_MAX_DIMS - 1];
 };
 
+// 16-byte packs of 4-byte elements at 4-byte alignment.  Wide global loads and stores need
+// only that much on this hardware, so rows that start anywhere (x[:, 1:], a row pitch of 8193
+// elements) and rows whose length is not a multiple of 4 still move as packs; the last pack
+// of a row is handled element by element.
+typedef uint32_t U32x4A4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <bool NT = true, typename T>
+__device__ __forceinline__ Pack<T, 4> load4_any(const T *p) {
+  U32x4A4 r;
+  if constexpr (NT) {
+    r = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4 *>(p));
+  } else {
+    r = *reinterpret_cast<const U32x4A4 *>(p);
+  }
+  Pack<T, 4> out;
+  __builtin_memcpy(&out, &r, 16);
+  return out;
+}
+template <bool NT = true, typename T>
+__device__ __forceinline__ void store4_any(T *p, const Pack<T, 4> &x) {
+  U32x4A4 r;
+  __builtin_memcpy(&r, &x, 16);
+  if constexpr (NT) {
+    __builtin_nontemporal_store(r, reinterpret_cast<U32x4A4 *>(p));
+  } else {
+    *reinterpret_cast<U32x4A4 *>(p) = r;
+  }
+}
+// up to 4 elements from p, `valid` of them inside the extent
+template <bool NT = true, typename T>
+__device__ __forceinline__ Pack<T, 4> load4_edge(const T *p, int64_t valid) {
+  if (valid >= 4) return load4_any<NT>(p);
+  Pack<T, 4> out;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out.v[c] = c < valid ? p[c] : T();
+  return out;
+}
+
 // HINTS says which accesses carry the nontemporal hint: bit 0 the store, bit 1 operand a,
 // bit 2 operand b.  A row that every block re-reads (a bias) keeps default caching so it
 // stays in L2; which operands that is has to be a compile-time fact, because a run-time
 // choice between a hinted and a plain load of one address is folded into one plain load.
+// ANY (4-byte elements, VEC == 4): packs at 4-byte alignment and rows of any length; one
+// element per lane, which such rows took before, ran at 31-43% of peak.
 template <int THREADS, int NIN, int VEC, int UNROLL, int HINTS, bool A_BC, bool B_BC, typename Op,
-          typename TO, typename TA, typename TB>
+          typename TO, typename TA, typename TB, bool ANY = false>
 __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
                                                     Op op) {
+  static_assert(!ANY || (VEC == 4 && sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4),
+                "packs at 4-byte alignment are for 4-byte elements");
   using PO = Pack<TO, VEC>;
   using PA = Pack<TA, VEC>;
   using PB = Pack<TB, VEC>;
@@ -499,10 +541,15 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
   for (int u = 0; u < UNROLL; ++u) {
     const int64_t e = e0 + (int64_t)u * THREADS * VEC;
     if (e < g.len) {
-      if constexpr (!A_BC)
-        va[u] = load_pack<(HINTS & 2) != 0>(reinterpret_cast<const PA *>(arow + e));
-      if constexpr (NIN == 2 && !B_BC)
-        vb[u] = load_pack<(HINTS & 4) != 0>(reinterpret_cast<const PB *>(brow + e));
+      if constexpr (ANY) {
+        if constexpr (!A_BC) va[u] = load4_edge<(HINTS & 2) != 0>(arow + e, g.len - e);
+        if constexpr (NIN == 2 && !B_BC) vb[u] = load4_edge<(HINTS & 4) != 0>(brow + e, g.len - e);
+      } else {
+        if constexpr (!A_BC)
+          va[u] = load_pack<(HINTS & 2) != 0>(reinterpret_cast<const PA *>(arow + e));
+        if constexpr (NIN == 2 && !B_BC)
+          vb[u] = load_pack<(HINTS & 4) != 0>(reinterpret_cast<const PB *>(brow + e));
+      }
     }
   }
 #pragma unroll
@@ -516,7 +563,16 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
         const TB y = (NIN == 2) ? (B_BC ? bbc : vb[u].v[k]) : TB();
         r.v[k] = apply<NIN, Op, TO, TA, TB>(op, x, y);
       }
-      store_pack<(HINTS & 1) != 0 && sizeof(PO) == 16>(reinterpret_cast<PO *>(orow + e), r);
+      if constexpr (ANY) {
+        if (g.len - e >= 4) {
+          store4_any<(HINTS & 1) != 0>(orow + e, r);
+        } else {
+          for (int k = 0; k < 4; ++k)
+            if (k < g.len - e) orow[e + k] = r.v[k];
+        }
+      } else {
+        store_pack<(HINTS & 1) != 0 && sizeof(PO) == 16>(reinterpret_cast<PO *>(orow + e), r);
+      }
     }
   }
 }
@@ -807,36 +863,6 @@ __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, con
 // the product of two dimensions (TileGeom::psplit): an operand stored as [.., q, p] with a short
 // innermost extent p (3 channels, 16, 56) is read in unit-stride runs across q and p, while
 // the output rows are addressed by (t / p, t % p).
-typedef uint32_t U32x4A4 __attribute__((ext_vector_type(4), aligned(4)));
-
-template <bool NT = true, typename T>
-__device__ __forceinline__ Pack<T, 4> load4_any(const T *p) {
-  U32x4A4 r;
-  if constexpr (NT) {
-    r = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4 *>(p));
-  } else {
-    r = *reinterpret_cast<const U32x4A4 *>(p);
-  }
-  Pack<T, 4> out;
-  __builtin_memcpy(&out, &r, 16);
-  return out;
-}
-template <typename T>
-__device__ __forceinline__ void store4_any(T *p, const Pack<T, 4> &x) {
-  U32x4A4 r;
-  __builtin_memcpy(&r, &x, 16);
-  __builtin_nontemporal_store(r, reinterpret_cast<U32x4A4 *>(p));
-}
-// up to 4 elements from p, `valid` of them inside the extent
-template <bool NT = true, typename T>
-__device__ __forceinline__ Pack<T, 4> load4_edge(const T *p, int64_t valid) {
-  if (valid >= 4) return load4_any<NT>(p);
-  Pack<T, 4> out;
-#pragma unroll
-  for (int c = 0; c < 4; ++c) out.v[c] = c < valid ? p[c] : T();
-  return out;
-}
-
 template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO, typename TA,
           typename TB, int THREADS>
 __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, const TB *b,
@@ -1275,7 +1301,7 @@ int launch_generic_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, 
 }
 
 template <int NIN, int VEC, bool A_BC, bool B_BC, typename Op, typename TO, typename TA,
-          typename TB>
+          typename TB, bool ANY = false>
 int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
   constexpr int U = TWG_ROWS_UNROLL;
   RowGeom rg{};
@@ -1307,7 +1333,7 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
   const unsigned grid = (unsigned)(cpr * rows);
 #define TWG_LAUNCH_ROWS(HINTS) \
-  ew_rows<kBlock, NIN, VEC, U, HINTS, A_BC, B_BC, Op, TO, TA, TB><<<grid, kBlock, 0, s>>>(out, a, b, rg, op)
+  ew_rows<kBlock, NIN, VEC, U, HINTS, A_BC, B_BC, Op, TO, TA, TB, ANY><<<grid, kBlock, 0, s>>>(out, a, b, rg, op)
   if (!stream)
     TWG_LAUNCH_ROWS(0);
   else if (reused[1])
@@ -1332,6 +1358,9 @@ int launch_rows(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStre
              (NIN == 1 || B_BC || g.stride[2][d] % VEC == 0);
   }
   if (vec_ok) return launch_rows_v<NIN, VEC, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
+  // 4-byte elements: packs at 4-byte alignment, rows of any length
+  if constexpr (sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4)
+    return launch_rows_v<NIN, 4, A_BC, B_BC, Op, TO, TA, TB, true>(out, a, b, g, op, s);
   return launch_rows_v<NIN, 1, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
 }
 
