@@ -22,7 +22,10 @@
  *    reference's uniform `Params` blocks (csrc/ops/binary.h:108-124,
  *    csrc/ops/unary.h:88-101).  Dimension 0 is the fastest-moving one, which is
  *    the order at::TensorIterator presents.  Strides are in elements, may be 0
- *    (broadcast) and may be negative.
+ *    (broadcast) and may be negative.  The elementwise entry points visit the
+ *    dimensions by ascending output stride whatever order they come in (the result
+ *    does not depend on it); for masked_select the order of the dimensions is the
+ *    order of the output.
  */
 #ifndef TWG_H_
 #define TWG_H_

@@ -346,6 +346,33 @@ def test_rows_that_start_anywhere(twg, rows, cols, pad, start):
     assert bit_equal(H.binary("twg_eq_f32", a, b, out_dtype=torch.bool), torch.eq(a, b))
 
 
+def test_outputs_that_no_input_streams_into(twg):
+    # outer sums and doubly broadcast operands: both inputs are re-read from cache and a block
+    # only streams its store (four packs per lane there); rows from 1024 elements on, with a
+    # ragged length, misaligned, and too short for that path
+    g = torch.Generator().manual_seed(77)
+    for n, m in ((300, 4096), (257, 4100), (64, 1024), (33, 5001), (70, 1000)):
+        col, row = torch.randn(n, 1, generator=g), torch.randn(1, m, generator=g)
+        assert bit_equal(H.add(col, row, alpha=1.25), oracle.add(col, row, alpha=1.25)), (n, m)
+        assert bit_equal(H.add(row, col), oracle.add(row, col)), (n, m)
+        rowv = torch.randn(1, m + 3, generator=g)[:, 1:m + 1]
+        assert bit_equal(H.add(col, rowv), oracle.add(col, rowv)), (n, m)
+    a = torch.randn(37, 1, 2048, generator=g)
+    b = torch.randn(1, 19, 2048, generator=g)
+    assert bit_equal(H.add(a, b), oracle.add(a, b))
+    # the same geometry whatever order the dimensions are passed in: a transposed output with
+    # transposed inputs, all in logical order (no sorting by output stride on the caller's side)
+    x, y = torch.randn(130, 515, generator=g).t(), torch.randn(130, 515, generator=g).t()
+    out = torch.zeros(130, 515).t()
+    got = H.binary("twg_add_f32", x, y, out=out, extra=(ctypes.c_float(1.0),), sort_by_out=False)
+    assert bit_equal(got, x + y)
+    nhwc = torch.randn(3, 20, 20, 64, generator=g).permute(0, 3, 1, 2)
+    bias = torch.randn(1, 64, 1, 1, generator=g)
+    out = torch.zeros(3, 20, 20, 64).permute(0, 3, 1, 2)
+    got = H.binary("twg_add_f32", nhwc, bias, out=out, extra=(ctypes.c_float(1.0),), sort_by_out=False)
+    assert bit_equal(got, nhwc + bias)
+
+
 def test_add_generic_strides_bruteforce(twg):
     g = torch.Generator().manual_seed(5)
     sizes = [3, 4, 2, 5]

@@ -1303,15 +1303,9 @@ int launch_generic_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, 
 template <int NIN, int VEC, bool A_BC, bool B_BC, typename Op, typename TO, typename TA,
           typename TB, bool ANY = false>
 int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
-  constexpr int U = TWG_ROWS_UNROLL;
   RowGeom rg{};
   rg.len = g.shape[0];
   constexpr int kBlock = 64;  // single-wavefront blocks stream best (see ew_contig)
-  const int64_t per_block = (int64_t)kBlock * VEC * U;
-  const int64_t cpr = (rg.len + per_block - 1) / per_block;
-  const int64_t rows = g.numel / rg.len;
-  if (cpr * rows > INT32_MAX || cpr > UINT32_MAX) return TWG_E_UNSUPPORTED;
-  rg.chunks_per_row = (uint32_t)cpr;
   rg.nouter = g.ndim - 1;
   for (int d = 1; d < g.ndim; ++d) {
     rg.oshape[d - 1] = g.shape[d];
@@ -1331,17 +1325,39 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
     reused[o] = again && footprint <= (int64_t(64) << 20);
   }
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
-  const unsigned grid = (unsigned)(cpr * rows);
-#define TWG_LAUNCH_ROWS(HINTS) \
+  const int64_t rows = g.numel / rg.len;
+  // Blocks of the grid for packs-per-lane U; 0 if that does not fit a launch.
+  auto grid_for = [&](int U) -> unsigned {
+    const int64_t per_block = (int64_t)kBlock * VEC * U;
+    const int64_t cpr = (rg.len + per_block - 1) / per_block;
+    if (cpr * rows > INT32_MAX || cpr > UINT32_MAX) return 0u;
+    rg.chunks_per_row = (uint32_t)cpr;
+    return (unsigned)(cpr * rows);
+  };
+#define TWG_LAUNCH_ROWS(U, HINTS) \
   ew_rows<kBlock, NIN, VEC, U, HINTS, A_BC, B_BC, Op, TO, TA, TB, ANY><<<grid, kBlock, 0, s>>>(out, a, b, rg, op)
+  // No input is streamed from memory (an outer sum a[:, None] + b[None, :], an expanded
+  // operand made dense): all a block moves is its store, and 1 KiB per block is less than the
+  // grid can launch blocks for (4 blocks per ns: 52% of peak); four packs per lane, 83%.
+  const bool a_cached = A_BC || reused[1];
+  const bool b_cached = NIN == 1 || B_BC || reused[2];
+  if (stream && a_cached && b_cached && rg.len >= 4 * kBlock * VEC) {
+    const unsigned grid = grid_for(4);
+    if (grid == 0) return TWG_E_UNSUPPORTED;
+    TWG_LAUNCH_ROWS(4, 1);
+    return (int)hipGetLastError();
+  }
+  constexpr int U = TWG_ROWS_UNROLL;
+  const unsigned grid = grid_for(U);
+  if (grid == 0) return TWG_E_UNSUPPORTED;
   if (!stream)
-    TWG_LAUNCH_ROWS(0);
+    TWG_LAUNCH_ROWS(U, 0);
   else if (reused[1])
-    TWG_LAUNCH_ROWS(1 | 4);
+    TWG_LAUNCH_ROWS(U, 1 | 4);
   else if (NIN == 2 && reused[2])
-    TWG_LAUNCH_ROWS(1 | 2);
+    TWG_LAUNCH_ROWS(U, 1 | 2);
   else
-    TWG_LAUNCH_ROWS(1 | 2 | 4);
+    TWG_LAUNCH_ROWS(U, 1 | 2 | 4);
 #undef TWG_LAUNCH_ROWS
   return (int)hipGetLastError();
 }

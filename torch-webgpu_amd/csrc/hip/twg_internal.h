@@ -33,8 +33,10 @@ struct Geom {
 };
 
 // Validate `it` and build the canonical geometry for the first `nops` operand
-// slots (2 = out + a, 3 = out + a + b).  Returns 0 or TWG_E_INVALID_ARG.
-int canonicalize(const twg_iter_t *it, int nops, Geom *g);
+// slots (2 = out + a, 3 = out + a + b).  Returns 0 or TWG_E_INVALID_ARG.  reorder: the
+// dimensions may be visited in any order (elementwise work), so they are taken by ascending
+// output stride; masked_select, whose output order is the order of the dimensions, passes false.
+int canonicalize(const twg_iter_t *it, int nops, Geom *g, bool reorder = true);
 
 // The compaction behind the masked_select entry points: elements of 1, 2, 4 or 8
 // bytes, count written to *d_count (device memory, or host memory the device can

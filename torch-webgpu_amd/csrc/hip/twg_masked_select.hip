@@ -116,7 +116,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
   if (local.ndim < 0 || local.ndim > TWG_MAX_DIMS) return TWG_E_INVALID_ARG;
   for (int d = 0; d < local.ndim; ++d) local.stride[TWG_OUT][d] = local.stride[TWG_A][d];
   Geom g;
-  if ((rc = canonicalize(&local, 3, &g))) return rc;
+  if ((rc = canonicalize(&local, 3, &g, false))) return rc;
   if (g.numel == 0) return twg_fill_bytes(d_count, 0, sizeof(int64_t), stream);
   if (!out_v || !src_v || !mask || !scratch) return TWG_E_INVALID_ARG;
   if (reinterpret_cast<uintptr_t>(out_v) % elem_size || reinterpret_cast<uintptr_t>(src_v) % elem_size)
