@@ -344,6 +344,11 @@ def test_rows_that_start_anywhere(twg, rows, cols, pad, start):
     got = _unary(C.UNARY_GELU_ERF, a)
     assert rel_err_ok(got, closed_form64("gelu_erf", a))[0]
     assert bit_equal(H.binary("twg_eq_f32", a, b, out_dtype=torch.bool), torch.eq(a, b))
+    # compares over the same rows: four bools per lane, into an aligned and a shifted output
+    z = torch.where(torch.rand(rows, cols + pad, generator=g) < 0.3, torch.zeros(()), big_a)[:, start:start + cols]
+    assert bit_equal(H.unary("twg_ne_scalar_f32", z, out_dtype=torch.bool, extra=(ctypes.c_float(0.0),)), z.ne(0.0))
+    mout = torch.zeros(rows, cols + pad, dtype=torch.bool)[:, start:start + cols]
+    assert bit_equal(H.binary("twg_eq_f32", a, b, out=mout), torch.eq(a, b))
 
 
 def test_outputs_that_no_input_streams_into(twg):

@@ -505,8 +505,9 @@ template <int THREADS, int NIN, int VEC, int UNROLL, int HINTS, bool A_BC, bool 
           typename TO, typename TA, typename TB, bool ANY = false>
 __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const TB *b, RowGeom g,
                                                     Op op) {
-  static_assert(!ANY || (VEC == 4 && sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4),
-                "packs at 4-byte alignment are for 4-byte elements");
+  static_assert(!ANY || (VEC == 4 && (sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 &&
+                         sizeof(TB) == 4),
+                "packs at 4-byte alignment are for 4-byte inputs and 4- or 1-byte outputs");
   using PO = Pack<TO, VEC>;
   using PA = Pack<TA, VEC>;
   using PB = Pack<TB, VEC>;
@@ -563,9 +564,18 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
         const TB y = (NIN == 2) ? (B_BC ? bbc : vb[u].v[k]) : TB();
         r.v[k] = apply<NIN, Op, TO, TA, TB>(op, x, y);
       }
-      if constexpr (ANY) {
+      if constexpr (ANY && sizeof(TO) == 4) {
         if (g.len - e >= 4) {
           store4_any<(HINTS & 1) != 0>(orow + e, r);
+        } else {
+          for (int k = 0; k < 4; ++k)
+            if (k < g.len - e) orow[e + k] = r.v[k];
+        }
+      } else if constexpr (ANY) {
+        // four 1-byte results (a compare over rows of floats that start anywhere): one dword
+        // where the output row happens to be aligned for it, bytes otherwise
+        if (g.len - e >= 4 && (reinterpret_cast<uintptr_t>(orow + e) & 3u) == 0) {
+          store_pack<false>(reinterpret_cast<PO *>(orow + e), r);
         } else {
           for (int k = 0; k < 4; ++k)
             if (k < g.len - e) orow[e + k] = r.v[k];
@@ -1374,8 +1384,8 @@ int launch_rows(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStre
              (NIN == 1 || B_BC || g.stride[2][d] % VEC == 0);
   }
   if (vec_ok) return launch_rows_v<NIN, VEC, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
-  // 4-byte elements: packs at 4-byte alignment, rows of any length
-  if constexpr (sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4)
+  // 4-byte inputs (and a 4- or 1-byte output): packs at 4-byte alignment, rows of any length
+  if constexpr ((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4)
     return launch_rows_v<NIN, 4, A_BC, B_BC, Op, TO, TA, TB, true>(out, a, b, g, op, s);
   return launch_rows_v<NIN, 1, A_BC, B_BC, Op, TO, TA, TB>(out, a, b, g, op, s);
 }
