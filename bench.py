@@ -380,13 +380,21 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
 
     def line(name, fn, nbytes, ref_ms):
         # these legs upload their own operands, and after the idle time of an upload the GPU's
-        # first 7 ms of work hold a slow stretch (see the note at the timed steps): warm up
-        # past it
-        ms = time_launches(fn, max(Wm, 2 * K), K)
+        # first 9 ms of work hold a slow stretch (see the note at the timed steps): keep it busy
+        # for 25 ms before the warm-up launches
+        t_busy = time.perf_counter()
+        settled = 0
+        while time.perf_counter() - t_busy < 0.025:
+            for _ in range(10):
+                fn()
+            settled += 10
+            capi.sync()
+        ms = time_launches(fn, Wm, K)
         avg = ms.batch_avg
         d = {"op": name, "avg_ms": round(avg, 5), "GBps": round(nbytes / avg / 1e6, 1),
              "pct_hbm_peak": round(nbytes / avg / 1e6 / HBM_PEAK_GBS * 100, 2),
-             "c_abi_ms": ref_ms, "vs_c_abi": round(avg / ref_ms, 4) if ref_ms else None}
+             "c_abi_ms": ref_ms, "vs_c_abi": round(avg / ref_ms, 4) if ref_ms else None,
+             "settling_launches": settled}
         log(f"  {name:28s} {avg:9.4f} ms  {d['GBps']:8.1f} GB/s  {d['pct_hbm_peak']:6.2f}% of peak"
             f"  ({d['vs_c_abi']} x the C-ABI line)")
         res.append(d)
