@@ -54,6 +54,7 @@
 #include <stdint.h>
 
 #include "twg.h"
+#include "twg_ms_bounds.h"
 
 namespace twg {
 namespace {
@@ -260,7 +261,7 @@ struct Quad<float> {
     return {__builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p))};
   }
   static __device__ __forceinline__ Quad load_selected(const float *p, const float *dummy, uint32_t bits) {
-    return load(bits ? p : dummy);
+    return load(quad_fetched(bits) ? p : dummy);
   }
 };
 template <>
@@ -280,8 +281,9 @@ struct Quad<uint64_t> {
   // 16-byte piece that starts inside the array.
   static __device__ __forceinline__ Quad load_selected(const uint64_t *p, const uint64_t *dummy,
                                                        uint32_t bits) {
-    return {__builtin_nontemporal_load(reinterpret_cast<const u64x2 *>((bits & 0x3u) ? p : dummy)),
-            __builtin_nontemporal_load(reinterpret_cast<const u64x2 *>((bits & 0xCu) ? p + 2 : dummy + 2))};
+    const uint32_t halves = quad64_halves(bits);
+    return {__builtin_nontemporal_load(reinterpret_cast<const u64x2 *>((halves & 1u) ? p : dummy)),
+            __builtin_nontemporal_load(reinterpret_cast<const u64x2 *>((halves & 2u) ? p + 2 : dummy + 2))};
   }
 };
 template <>
@@ -293,7 +295,7 @@ struct Quad<uint16_t> {
     return {__builtin_nontemporal_load(reinterpret_cast<const u16x4 *>(p))};
   }
   static __device__ __forceinline__ Quad load_selected(const uint16_t *p, const uint16_t *dummy, uint32_t bits) {
-    return load(bits ? p : dummy);
+    return load(quad_fetched(bits) ? p : dummy);
   }
 };
 template <>
@@ -307,7 +309,7 @@ struct Quad<uint8_t> {
     return {__builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p))};
   }
   static __device__ __forceinline__ Quad load_selected(const uint8_t *p, const uint8_t *dummy, uint32_t bits) {
-    return load(bits ? p : dummy);
+    return load(quad_fetched(bits) ? p : dummy);
   }
 };
 
