@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "twg_internal.h"
+#include "twg_tile_walk.h"
 
 namespace twg {
 namespace {
@@ -624,32 +625,10 @@ __device__ __forceinline__ int64_t tile_row_off(const TileGeom &g, int o, int64_
   return (int64_t)rem * g.s0[o] + (int64_t)q * g.s1[o];
 }
 
-// Which tile a workgroup takes.  Plain order: tiles along dimension 0 first, then along t,
-// then the batch.  Where the pieces of a transposed operand do not start and end on
-// 128-byte lines (a row pitch of 197 or 56 elements), tiles that are neighbours along t
-// read the same lines, and in the plain order they run on different XCDs, each of which
-// fetches the line into its own L2 (measured: 1.9-2.1 times the operand's bytes fetched).
-// Workgroups are dealt to the 8 XCDs round-robin by their index, so with ngroups set the
-// index is decoded as (XCD, position on that XCD) and each XCD walks along t through one
-// (tile along dimension 0, batch index) pair after the other: the second reader of a line
-// finds it in the L2 its neighbour filled.  Returns false for the workgroups that pad the
-// grid to a multiple of 8 pairs.
+// Which tile a workgroup takes (twg_tile_walk.h); false for the workgroups that pad the grid.
 __device__ __forceinline__ bool tile_of_block(const TileGeom &g, uint32_t bid, uint32_t &t0i,
                                               uint32_t &tti, int64_t &r) {
-  if (g.ngroups == 0) {
-    t0i = bid % g.tiles0;
-    bid /= g.tiles0;
-    tti = bid % g.tilest;
-    r = bid / g.tilest;
-    return true;
-  }
-  const uint32_t xcd = bid & 7u, k = bid >> 3;
-  tti = k % g.tilest;
-  const uint32_t grp = (k / g.tilest) * 8u + xcd;
-  if (grp >= g.ngroups) return false;
-  t0i = grp % g.tiles0;
-  r = grp / g.tiles0;
-  return true;
+  return decode_tile(g.tiles0, g.tilest, g.ngroups, bid, t0i, tti, r);
 }
 
 // Lane x (0..63) runs along dimension 0, the 4 wavefronts and 16 steps cover 64
@@ -1442,22 +1421,13 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
   auto set_tiles = [&](int td0, int tt, unsigned *grid, bool xcd_walk = false) {
     const int64_t tiles0 = (tg.n0 + td0 - 1) / td0;
     const int64_t tilest = (tg.nt + tt - 1) / tt;
-    if (tiles0 > UINT32_MAX || tilest > UINT32_MAX) return false;
-    if (tiles0 * tilest > INT32_MAX || tiles0 * tilest * batch > INT32_MAX) return false;
+    // pieces of a transposed operand that share 128-byte lines with their neighbours along
+    // t: let one XCD walk along t (decode_tile)
+    const int64_t blocks = tile_grid(tiles0, tilest, batch, xcd_walk && ragged_t, &tg.ngroups);
+    if (blocks == 0) return false;
     tg.tiles0 = (uint32_t)tiles0;
     tg.tilest = (uint32_t)tilest;
-    tg.ngroups = 0;
-    *grid = (unsigned)(tiles0 * tilest * batch);
-    // pieces of a transposed operand that share 128-byte lines with their neighbours along
-    // t: let one XCD walk along t (tile_of_block)
-    if (xcd_walk && tilest > 1 && ragged_t) {
-      const int64_t groups = tiles0 * batch;
-      const int64_t padded = (groups + 7) / 8 * 8 * tilest;
-      if (groups <= UINT32_MAX && padded <= INT32_MAX) {
-        tg.ngroups = (uint32_t)groups;
-        *grid = (unsigned)padded;
-      }
-    }
+    *grid = (unsigned)blocks;
     return true;
   };
   unsigned grid = 0;

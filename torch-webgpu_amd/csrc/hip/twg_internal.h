@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "twg.h"
+#include "twg_geom.h"
 
 namespace twg {
 
@@ -21,22 +22,6 @@ int ensure_init();
     hipError_t twg_e_ = (expr);                \
     if (twg_e_ != hipSuccess) return (int)twg_e_; \
   } while (0)
-
-// Canonical iteration geometry derived from a caller's twg_iter_t: size-1
-// dimensions dropped and adjacent dimensions merged wherever every used operand
-// stays linear across them.  Dimension 0 remains the fastest one.
-struct Geom {
-  int ndim;
-  int64_t numel;
-  int64_t shape[TWG_MAX_DIMS];
-  int64_t stride[3][TWG_MAX_DIMS];
-};
-
-// Validate `it` and build the canonical geometry for the first `nops` operand
-// slots (2 = out + a, 3 = out + a + b).  Returns 0 or TWG_E_INVALID_ARG.  reorder: the
-// dimensions may be visited in any order (elementwise work), so they are taken by ascending
-// output stride; masked_select, whose output order is the order of the dimensions, passes false.
-int canonicalize(const twg_iter_t *it, int nops, Geom *g, bool reorder = true);
 
 // The compaction behind the masked_select entry points: elements of 1, 2, 4 or 8
 // bytes, count written to *d_count (device memory, or host memory the device can
