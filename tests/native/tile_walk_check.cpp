@@ -1,14 +1,16 @@
 // Every workgroup index of a tile-kernel launch decoded on the CPU (csrc/hip/twg_tile_walk.h):
-// each (tile along dimension 0, tile along t, batch index) is taken by exactly one workgroup,
-// the workgroups that pad the grid take none, and in the per-XCD order the tiles that follow
-// one another along t sit on one XCD (workgroup index modulo 8) in consecutive positions.
+// each (tile along dimension 0, tile along t, batch entry) is taken by exactly one workgroup and
+// the workgroups that pad the grid take none.  In the plain order the walk is: tiles along
+// dimension 0 fastest, then the first nb_inner batch dimensions, then t, then the other batch
+// dimensions.  In the per-XCD order the tiles that follow one another along t sit on one XCD
+// (workgroup index modulo 8) in consecutive positions.
 #include <cstdio>
 #include <vector>
 
 #include "twg_tile_walk.h"
 
 static int fail(const char *what, long a, long b, long c, int walk) {
-  std::printf("FAILED: %s (tiles0 %ld, tilest %ld, batch %ld, xcd walk %d)\n", what, a, b, c, walk);
+  std::printf("FAILED: %s (tiles0 %ld, tilest %ld, batch shape #%ld, xcd walk %d)\n", what, a, b, c, walk);
   return 1;
 }
 
@@ -16,50 +18,81 @@ int main() {
   int launches = 0;
   const long t0s[] = {1, 2, 3, 7, 8, 9, 31, 128};
   const long tts[] = {1, 2, 3, 5, 8, 24, 197};
-  const long batches[] = {1, 2, 5, 8, 12, 17};
+  const std::vector<std::vector<long>> batch_shapes = {{}, {2}, {5}, {8}, {3, 4}, {17}, {2, 3, 2}, {7, 1, 5}};
   for (long tiles0 : t0s)
     for (long tilest : tts)
-      for (long batch : batches)
-        for (int walk = 0; walk < 2; ++walk) {
-          uint32_t ngroups = 77;
-          const int64_t grid = twg::tile_grid(tiles0, tilest, batch, walk != 0, &ngroups);
-          if (grid <= 0) return fail("no grid", tiles0, tilest, batch, walk);
-          const bool per_xcd = walk && tilest > 1;
-          if (per_xcd != (ngroups != 0)) return fail("ngroups", tiles0, tilest, batch, walk);
-          if (per_xcd) {
-            if (ngroups != tiles0 * batch) return fail("ngroups value", tiles0, tilest, batch, walk);
-            if (grid % (8 * tilest) != 0 || grid < tiles0 * tilest * batch ||
-                grid >= (tiles0 * batch + 8) * tilest)
-              return fail("padded grid", tiles0, tilest, batch, walk);
-          } else if (grid != tiles0 * tilest * batch) {
-            return fail("plain grid", tiles0, tilest, batch, walk);
-          }
-          std::vector<int> taken((size_t)(tiles0 * tilest * batch), 0);
-          std::vector<int64_t> owner_xcd((size_t)(tiles0 * batch), -1);
-          int64_t idle = 0;
-          for (int64_t bid = 0; bid < grid; ++bid) {
-            uint32_t t0i = ~0u, tti = ~0u;
-            int64_t r = -1;
-            if (!twg::decode_tile((uint32_t)tiles0, (uint32_t)tilest, ngroups, (uint32_t)bid, t0i, tti, r)) {
-              ++idle;
-              continue;
+      for (size_t bs = 0; bs < batch_shapes.size(); ++bs)
+        for (int nb_inner = 0; nb_inner <= (int)batch_shapes[bs].size(); ++nb_inner)
+          for (int walk = 0; walk < 2; ++walk) {
+            const std::vector<long> &bshape = batch_shapes[bs];
+            twg::TileWalk w{};
+            w.tiles0 = (uint32_t)tiles0;
+            w.tilest = (uint32_t)tilest;
+            w.nbatch = (int)bshape.size();
+            w.nb_inner = nb_inner;
+            long batch = 1;
+            for (int d = 0; d < w.nbatch; ++d) {
+              w.bshape[d] = bshape[d];
+              batch *= bshape[d];
             }
-            if (t0i >= tiles0 || tti >= tilest || r < 0 || r >= batch)
-              return fail("tile out of range", tiles0, tilest, batch, walk);
-            ++taken[(size_t)((r * tilest + tti) * tiles0 + t0i)];
+            w.ngroups = 77;
+            const int64_t grid = twg::tile_grid(tiles0, tilest, batch, walk != 0, &w.ngroups);
+            if (grid <= 0) return fail("no grid", tiles0, tilest, bs, walk);
+            const bool per_xcd = walk && tilest > 1;
+            if (per_xcd != (w.ngroups != 0)) return fail("ngroups", tiles0, tilest, bs, walk);
             if (per_xcd) {
-              // one XCD per (t0i, r) pair, and its tiles along t in consecutive positions
-              const size_t pair = (size_t)(r * tiles0 + t0i);
-              if (owner_xcd[pair] < 0) owner_xcd[pair] = bid & 7;
-              if (owner_xcd[pair] != (bid & 7)) return fail("a pair is spread over XCDs", tiles0, tilest, batch, walk);
-              if (((bid >> 3) % tilest) != tti) return fail("position along t", tiles0, tilest, batch, walk);
+              if (w.ngroups != tiles0 * batch) return fail("ngroups value", tiles0, tilest, bs, walk);
+              if (grid % (8 * tilest) != 0 || grid < tiles0 * tilest * batch ||
+                  grid >= (tiles0 * batch + 8) * tilest)
+                return fail("padded grid", tiles0, tilest, bs, walk);
+            } else if (grid != tiles0 * tilest * batch) {
+              return fail("plain grid", tiles0, tilest, bs, walk);
             }
+            std::vector<int> taken((size_t)(tiles0 * tilest * batch), 0);
+            std::vector<int64_t> owner_xcd((size_t)(tiles0 * batch), -1);
+            int64_t idle = 0;
+            for (int64_t bid = 0; bid < grid; ++bid) {
+              uint32_t t0i = ~0u, tti = ~0u;
+              long idx[TWG_MAX_DIMS] = {};
+              int seen = 0;
+              auto note = [&](int d, uint32_t i) {
+                idx[d] = i;
+                seen |= 1 << d;
+              };
+              const bool has_tile = walk ? twg::decode_tile<true>(w, (uint32_t)bid, t0i, tti, note)
+                                         : twg::decode_tile<false>(w, (uint32_t)bid, t0i, tti, note);
+              if (!has_tile) {
+                ++idle;
+                continue;
+              }
+              if (seen != (1 << w.nbatch) - 1) return fail("a batch dimension was not reported", tiles0, tilest, bs, walk);
+              if (t0i >= tiles0 || tti >= tilest) return fail("tile out of range", tiles0, tilest, bs, walk);
+              long r = 0, inner = 0, inner_count = 1, outer = 0;
+              for (int d = w.nbatch - 1; d >= 0; --d) {
+                if (idx[d] < 0 || idx[d] >= bshape[d]) return fail("batch index out of range", tiles0, tilest, bs, walk);
+                r = r * bshape[d] + idx[d];
+              }
+              for (int d = w.nbatch - 1; d >= w.nb_inner; --d) outer = outer * bshape[d] + idx[d];
+              for (int d = w.nb_inner - 1; d >= 0; --d) inner = inner * bshape[d] + idx[d];
+              for (int d = 0; d < w.nb_inner; ++d) inner_count *= bshape[d];
+              ++taken[(size_t)((r * tilest + tti) * tiles0 + t0i)];
+              if (per_xcd) {
+                // one XCD per (t0i, batch entry) pair, and its tiles along t in consecutive positions
+                const size_t pair = (size_t)(r * tiles0 + t0i);
+                if (owner_xcd[pair] < 0) owner_xcd[pair] = bid & 7;
+                if (owner_xcd[pair] != (bid & 7)) return fail("a pair is spread over XCDs", tiles0, tilest, bs, walk);
+                if (((bid >> 3) % tilest) != tti) return fail("position along t", tiles0, tilest, bs, walk);
+              } else {
+                // the plain order, spelled out: position = ((outer * tilest + tti) * inner_count + inner) * tiles0 + t0i
+                const int64_t pos = ((outer * tilest + tti) * inner_count + inner) * tiles0 + t0i;
+                if (pos != bid) return fail("plain order", tiles0, tilest, bs, walk);
+              }
+            }
+            for (int n : taken)
+              if (n != 1) return fail("a tile is taken by no workgroup or by several", tiles0, tilest, bs, walk);
+            if (idle != grid - tiles0 * tilest * batch) return fail("idle workgroups", tiles0, tilest, bs, walk);
+            ++launches;
           }
-          for (int n : taken)
-            if (n != 1) return fail("a tile is taken by no workgroup or by several", tiles0, tilest, batch, walk);
-          if (idle != grid - tiles0 * tilest * batch) return fail("idle workgroups", tiles0, tilest, batch, walk);
-          ++launches;
-        }
   // counts that do not fit the 32-bit decoding are refused, the per-XCD order is dropped
   // where only its padding does not fit
   uint32_t ng;

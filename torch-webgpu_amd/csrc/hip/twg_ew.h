@@ -592,7 +592,7 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
 
 constexpr int kTile = 64;
 
-struct TileGeom {
+struct TileGeom : TileWalk {  // tile counts, batch extents and the walk order come from there
   int64_t n0, nt;          // extents of dimension 0 and of the transposed dimension t
   int64_t s0[3], st[3];    // strides along those two, per operand
   // ew_tile_any only: t may be the product of two dimensions, q (outer, extent nt / psplit,
@@ -608,12 +608,6 @@ struct TileGeom {
   // (r % n0in) * s0 + (r / n0in) * s1.  n0in == 0: dimension 0 is one dimension.
   uint32_t n0in;
   int64_t s1[3];
-  uint32_t tiles0, tilest; // tile counts
-  // ew_tile_vec / ew_tile_any: 0, or the number of (tile along dimension 0, batch index) pairs
-  // when the tiles that follow one another along t are to run on one XCD (tile_of_block)
-  uint32_t ngroups;
-  int32_t nbatch;          // remaining dimensions
-  int64_t bshape[TWG_MAX_DIMS - 2];
   int64_t bstride[3][TWG_MAX_DIMS - 2];
 };
 
@@ -625,10 +619,18 @@ __device__ __forceinline__ int64_t tile_row_off(const TileGeom &g, int o, int64_
   return (int64_t)rem * g.s0[o] + (int64_t)q * g.s1[o];
 }
 
-// Which tile a workgroup takes (twg_tile_walk.h); false for the workgroups that pad the grid.
+// Which tile a workgroup takes (twg_tile_walk.h) and the operand offsets of its batch entry;
+// false for the workgroups that pad the grid.
+template <bool XCD_ORDER, int NIN>
 __device__ __forceinline__ bool tile_of_block(const TileGeom &g, uint32_t bid, uint32_t &t0i,
-                                              uint32_t &tti, int64_t &r) {
-  return decode_tile(g.tiles0, g.tilest, g.ngroups, bid, t0i, tti, r);
+                                              uint32_t &tti, int64_t &off_o, int64_t &off_a,
+                                              int64_t &off_b) {
+  off_o = off_a = off_b = 0;
+  return decode_tile<XCD_ORDER>(g, bid, t0i, tti, [&](int d, uint32_t i) {
+    off_o += (int64_t)i * g.bstride[0][d];
+    off_a += (int64_t)i * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += (int64_t)i * g.bstride[2][d];
+  });
 }
 
 // Lane x (0..63) runs along dimension 0, the 4 wavefronts and 16 steps cover 64
@@ -640,21 +642,9 @@ __global__ __launch_bounds__(kThreads) void ew_tile(TO *out, const TA *a, const 
   __shared__ TA sa[A_T ? kTile : 1][kTile + 1];
   __shared__ TB sb[(NIN == 2 && B_T) ? kTile : 1][kTile + 1];
 
-  uint32_t bid = blockIdx.x;
-  const uint32_t t0i = bid % g.tiles0;
-  bid /= g.tiles0;
-  const uint32_t tti = bid % g.tilest;
-  int64_t r = bid / g.tilest;
-  int64_t off_o = 0, off_a = 0, off_b = 0;
-  for (int d = 0; d < g.nbatch; ++d) {
-    const uint32_t extent = (uint32_t)g.bshape[d];
-    const uint32_t q = (uint32_t)r / extent;  // batch indices fit 32 bits, the grid does
-    const int64_t c = (uint32_t)r - q * extent;
-    r = q;
-    off_o += c * g.bstride[0][d];
-    off_a += c * g.bstride[1][d];
-    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
-  }
+  uint32_t t0i, tti;
+  int64_t off_o, off_a, off_b;
+  tile_of_block<false, NIN>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b);
   const int x = threadIdx.x & 63;
   const int y = threadIdx.x >> 6;  // 0..3
   const int64_t base0 = (int64_t)t0i * kTile;
@@ -815,21 +805,9 @@ __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, con
   __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
 
   // (this kernel only gets line-aligned pieces, so its tiles are always dealt in plain order)
-  uint32_t bid = blockIdx.x;
-  const uint32_t t0i = bid % g.tiles0;
-  bid /= g.tiles0;
-  const uint32_t tti = bid % g.tilest;
-  uint32_t r = bid / g.tilest;
-  int64_t off_o = 0, off_a = 0, off_b = 0;
-  for (int d = 0; d < g.nbatch; ++d) {
-    const uint32_t extent = (uint32_t)g.bshape[d];
-    const uint32_t q = r / extent;
-    const int64_t c = r - q * extent;
-    r = q;
-    off_o += c * g.bstride[0][d];
-    off_a += c * g.bstride[1][d];
-    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
-  }
+  uint32_t t0i, tti;
+  int64_t off_o, off_a, off_b;
+  tile_of_block<false, NIN>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b);
   const int64_t base0 = (int64_t)t0i * TD0;
   const int64_t baset = (int64_t)tti * TT;
   // workgroup-uniform: whole tiles take the unpredicated body
@@ -865,18 +843,8 @@ __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, con
   __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
 
   uint32_t t0i, tti;
-  int64_t r;
-  if (!tile_of_block(g, blockIdx.x, t0i, tti, r)) return;  // workgroup-uniform
-  int64_t off_o = 0, off_a = 0, off_b = 0;
-  for (int d = 0; d < g.nbatch; ++d) {
-    const uint32_t extent = (uint32_t)g.bshape[d];
-    const uint32_t q = (uint32_t)r / extent;  // batch indices fit 32 bits, the grid does
-    const int64_t c = (uint32_t)r - q * extent;
-    r = q;
-    off_o += c * g.bstride[0][d];
-    off_a += c * g.bstride[1][d];
-    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
-  }
+  int64_t off_o, off_a, off_b;
+  if (!tile_of_block<true, NIN>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b)) return;  // workgroup-uniform
   const int64_t base0 = (int64_t)t0i * TD0;
   const int64_t baset = (int64_t)tti * TT;
 
@@ -1408,6 +1376,15 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
     for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
     tg.nbatch++;
     batch *= g.shape[d];
+  }
+  // the leading batch dimensions along which the output is denser than along t are walked
+  // before t (decode_tile)
+  tg.nb_inner = 0;
+  {
+    auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+    int64_t along_t = mag(tg.st[0]);
+    if (tg.psplit > 1 && mag(tg.sp[0]) < along_t) along_t = mag(tg.sp[0]);
+    while (tg.nb_inner < tg.nbatch && mag(tg.bstride[0][tg.nb_inner]) < along_t) ++tg.nb_inner;
   }
   // Do the pieces of a transposed operand (32 or 64 elements along t) start and end on
   // 128-byte lines?  If not, tiles that are neighbours along t share lines.

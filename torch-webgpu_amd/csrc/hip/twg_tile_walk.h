@@ -6,6 +6,8 @@
 
 #include <stdint.h>
 
+#include "twg.h"
+
 #if defined(__HIPCC__)
 #define TWG_WALK_FN __host__ __device__ __forceinline__
 #else
@@ -14,31 +16,66 @@
 
 namespace twg {
 
-// Plain order: tiles along dimension 0 first, then along t, then the batch.  Where the
-// pieces of a transposed operand do not start and end on 128-byte lines (a row pitch of 197
-// or 56 elements), tiles that are neighbours along t read the same lines, and in the plain
-// order they run on different XCDs, each of which fetches the line into its own L2
-// (measured: 1.9-2.1 times the operand's bytes fetched).  Workgroups are dealt to the 8 XCDs
-// round-robin by their index, so with ngroups set (the number of (tile along dimension 0,
-// batch index) pairs) the index is decoded as (XCD, position on that XCD) and each XCD walks
-// along t through one pair after the other: the second reader of a line finds it in the L2
-// its neighbour filled.  Returns false for the workgroups that pad the grid to a multiple of
-// 8 pairs.  r is the batch index.
-TWG_WALK_FN bool decode_tile(uint32_t tiles0, uint32_t tilest, uint32_t ngroups, uint32_t bid,
-                               uint32_t &t0i, uint32_t &tti, int64_t &r) {
-  if (ngroups == 0) {
-    t0i = bid % tiles0;
-    bid /= tiles0;
-    tti = bid % tilest;
-    r = bid / tilest;
+// The part of a tile kernel's geometry that says which tile a workgroup takes.
+struct TileWalk {
+  uint32_t tiles0, tilest;  // tiles along dimension 0 and along t
+  // 0, or the number of (tile along dimension 0, batch entry) pairs when the tiles that follow
+  // one another along t are to run on one XCD (see decode_tile)
+  uint32_t ngroups;
+  int32_t nbatch;    // remaining (batch) dimensions
+  int32_t nb_inner;  // the first nb_inner of them are walked before t
+  int64_t bshape[TWG_MAX_DIMS - 2];
+};
+
+// Workgroup index -> tile (t0i along dimension 0, tti along t) and batch entry;
+// batch_index(d, i) is called once per batch dimension with the entry's index i along it.
+//
+// Plain order: tiles along dimension 0 first, then the batch dimensions the output is denser
+// along than along t (the first nb_inner), then t, then the other batch dimensions: that is
+// the order of the output's memory, so consecutive workgroups extend the same runs of output
+// (and of the operands laid out like it) for as long as the geometry allows.  An output
+// [n][h][w*c] read against an operand stored [c][w][h][n] writes, per tile, 32 runs of 1 KiB
+// along n; walking h before the tiles along n makes those runs grow through a whole
+// [h][w*c] plane (1.2 MB) instead of stopping after one [w*c] row (21 KiB).
+//
+// Per-XCD order (XCD_ORDER and ngroups != 0): where the pieces of a transposed operand do not
+// start and end on 128-byte lines (a row pitch of 197 or 56 elements), tiles that are
+// neighbours along t read the same lines, and in the plain order they run on different XCDs,
+// each of which fetches the line into its own L2 (measured: 1.9-2.1 times the operand's bytes
+// fetched).  Workgroups are dealt to the 8 XCDs round-robin by their index, so the index is
+// decoded as (XCD, position on that XCD) and each XCD walks along t through one (tile along
+// dimension 0, batch entry) pair after the other: the second reader of a line finds it in the
+// L2 its neighbour filled.  Returns false for the workgroups that pad the grid to a multiple
+// of 8 pairs.
+template <bool XCD_ORDER, typename F>
+TWG_WALK_FN bool decode_tile(const TileWalk &w, uint32_t bid, uint32_t &t0i, uint32_t &tti,
+                             F &&batch_index) {
+  uint32_t rem;
+  auto batch_dims = [&](int lo, int hi) {
+    for (int d = lo; d < hi; ++d) {
+      const uint32_t extent = (uint32_t)w.bshape[d];  // batch indices fit 32 bits, the grid does
+      const uint32_t q = rem / extent;
+      batch_index(d, rem - q * extent);
+      rem = q;
+    }
+  };
+  if (!XCD_ORDER || w.ngroups == 0) {
+    rem = bid / w.tiles0;
+    t0i = bid - rem * w.tiles0;
+    batch_dims(0, w.nb_inner);
+    const uint32_t q = rem / w.tilest;
+    tti = rem - q * w.tilest;
+    rem = q;
+    batch_dims(w.nb_inner, w.nbatch);
     return true;
   }
   const uint32_t xcd = bid & 7u, k = bid >> 3;
-  tti = k % tilest;
-  const uint32_t grp = (k / tilest) * 8u + xcd;
-  if (grp >= ngroups) return false;
-  t0i = grp % tiles0;
-  r = grp / tiles0;
+  tti = k % w.tilest;
+  const uint32_t grp = (k / w.tilest) * 8u + xcd;
+  if (grp >= w.ngroups) return false;
+  rem = grp / w.tiles0;
+  t0i = grp - rem * w.tiles0;
+  batch_dims(0, w.nbatch);
   return true;
 }
 
