@@ -101,6 +101,20 @@ int main() {
   if (twg::tile_grid(1, (int64_t(1) << 31) - 2, 1, true, &ng) != (int64_t(1) << 31) - 2 || ng != 0)
     return fail("padding that does not fit", 0, 0, 0, 1);
   if (twg::tile_grid(0, 4, 1, false, &ng) != 0) return fail("zero tiles accepted", 0, 0, 0, 0);
+  // the one-multiplication division: exact for every divisor up to 10 000 and every numerator
+  // with n * d <= 2^32 that is near a multiple of d, small, or at the top of the range
+  for (uint32_t d = 1; d <= 10000; ++d) {
+    const twg::SmallDiv s = twg::small_div(d);
+    const uint64_t top = (uint64_t(1) << 32) / d;  // n <= top
+    auto check = [&](uint64_t n) {
+      return n > top || n > 0xFFFFFFFFull || twg::div_by((uint32_t)n, s) == (uint32_t)(n / d);
+    };
+    for (uint64_t n = 0; n < 70; ++n)
+      if (!check(n) || !check(top - n)) return fail("small_div", d, (long)n, 0, 0);
+    for (uint64_t q = 1; q < 400; q += 7)
+      for (int64_t e = -2; e <= 2; ++e)
+        if (!check(q * d + e) || !check((top / d > q ? top / d - q : 0) * d + e)) return fail("small_div near a multiple", d, (long)q, (long)e, 0);
+  }
   std::printf("tile walk ok (%d launches)\n", launches);
   return 0;
 }

@@ -282,6 +282,7 @@ def test_add_transposed_operand(twg, rows, cols):
     ((5, 3, 40, 96), (0, 2, 3, 1)), ((5, 3, 40, 96), (2, 0, 3, 1)), ((3, 1000), (1, 0)),
     ((4, 4, 1027), (0, 2, 1)), ((2, 16, 700), (0, 2, 1)), ((2, 32, 301), (0, 2, 1)),
     ((2, 33, 300), (0, 2, 1)), ((7, 2, 5000), (0, 2, 1)), ((3, 5, 255), (0, 2, 1)),
+    ((2, 8, 3001), (0, 2, 1)), ((3, 16, 1100), (0, 2, 1)), ((2, 24, 777), (0, 2, 1)),
     # the same with fewer than 256 elements per strip: several strips per block
     ((4, 3, 23, 100), (2, 0, 3, 1)), ((3, 5, 9, 33), (0, 2, 3, 1)), ((2, 2, 7, 250), (2, 0, 3, 1)),
     ((6, 3, 224), (0, 2, 1)), ((2, 31, 40), (0, 2, 1)), ((16, 3, 224, 96), (2, 0, 3, 1)),

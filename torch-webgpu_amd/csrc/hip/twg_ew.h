@@ -940,21 +940,51 @@ __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, con
 // ------------------------------------------------------------ ew_deint
 // An operand stored as [.., x, c] with a short innermost extent c (3 colour channels, a handful
 // of heads) against an output laid out [.., c, x]: the operand's stride along dimension 0 is the
-// extent of c.  A block reads a strip of TX * c consecutive elements with 16-byte loads, parks
-// it in LDS as it lies in memory, and writes c runs of TX output elements, picking the strip up
-// with a stride of c.  (Through the gather kernel these layouts ran at 51% of HBM peak.)
-constexpr int kDeintLds = 8192;  // elements of one strip at most
+// extent of c.  A block reads a strip of TX * c consecutive elements with 16-byte loads and
+// parks it in LDS one run of x per channel, so that the second phase picks up four consecutive
+// x of one channel with one 16-byte LDS read and writes c runs of TX output elements.
+// (Through the gather kernel these layouts ran at 51% of HBM peak.)
+//
+// The transposition happens on the way into LDS, element by element, because that is the side
+// where it can be had without bank conflicts: with the strip parked as it lies in memory, the
+// lanes of a wavefront that pick up x, x+4, x+8.. of one channel are 4*c words apart, which
+// for c = 16 is the same bank for all 64 of them.  A channel's run starts deint_pitch(nx)
+// words after the previous one's, a multiple of 4 (16-byte reads) that is 4 modulo 32: the
+// four words a lane scatters and the words of its neighbours then fall into different banks
+// for every c but multiples of 8 (two lanes per bank).  (Worth 2 points at c = 16.)
+//
+// What sets the rate is how many blocks a CU holds, not how much one block keeps in flight: a
+// block goes through load strip -> LDS -> barrier -> load the straight operands -> store, and
+// only other blocks fill the gaps.  With 36 KiB of LDS per block (4 blocks per CU, 8192
+// elements each) these layouts ran at 65-74% of peak; with 9 KiB (the 8 blocks the CU's
+// wavefront slots allow, ~2000 elements each, two 16-byte loads per lane in flight) at 75-82%.
+// Issuing all of a big block's loads at once was the worst of all (44-50%).
+constexpr int kDeintLds = 2304;  // words of LDS per deinterleaved operand and block at most
+__host__ __device__ constexpr uint32_t deint_pitch(uint32_t nx) { return (nx + 27u) / 32u * 32u + 4u; }
+
+struct DeintShape {
+  uint32_t tx_elems;  // elements of dimension 0 per strip
+  uint32_t rows;      // strips per block (consecutive indices of the first batch dimension)
+  uint32_t lds_words; // words of LDS per deinterleaved operand
+  SmallDiv by_p;      // the channel count
+  SmallDiv by_strip4; // a full strip's length in memory, rounded up to packs
+  SmallDiv by_packs;  // packs of output per channel and full strip
+  SmallDiv by_per_row;  // by_packs.d * P
+};
 
 template <int NIN, bool A_D, bool B_D, typename Op, typename TO, typename TA, typename TB>
 __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const TB *b, TileGeom g,
-                                                     uint32_t tx_elems, uint32_t rows, Op op) {
+                                                     DeintShape sh, Op op) {
   static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
   using PO = Pack<TO, 4>;
   using PA = Pack<TA, 4>;
   using PB = Pack<TB, 4>;
-  __shared__ __attribute__((aligned(16))) TA sa[A_D ? kDeintLds : 4];
-  __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_D) ? kDeintLds : 4];
+  // sh.lds_words words per deinterleaved operand, sized by the launch
+  extern __shared__ __attribute__((aligned(16))) unsigned char deint_lds[];
+  TA *sa = reinterpret_cast<TA *>(deint_lds);
+  TB *sb = reinterpret_cast<TB *>(deint_lds) + (A_D ? sh.lds_words : 0u);
 
+  const uint32_t rows = sh.rows;
   uint32_t bid = blockIdx.x;
   const uint32_t t0i = bid % g.tiles0;
   int64_t r = bid / g.tiles0;
@@ -983,29 +1013,44 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
     if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
   }
   const uint32_t P = (uint32_t)g.nt;
-  const int64_t x0 = (int64_t)t0i * tx_elems;
-  const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)tx_elems ? g.n0 - x0 : (int64_t)tx_elems);
+  const int64_t x0 = (int64_t)t0i * sh.tx_elems;
+  const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)sh.tx_elems ? g.n0 - x0 : (int64_t)sh.tx_elems);
   const uint32_t strip = nx * P;  // consecutive elements of a deinterleaved operand
-  const uint32_t pitch = (strip + 3u) & ~3u;  // of a strip in LDS
-  // Loads are issued kU at a time before the first of them is used: one load per trip,
-  // waited for at once, left a block with a single request in flight per lane.
-  constexpr uint32_t kU = 4;
+  // (the last strip along dimension 0 may be shorter than the one the divisors were made for;
+  // then a block takes one strip only and those divisors are not used)
+  const uint32_t strip4 = (strip + 3u) & ~3u;
+  const uint32_t xpitch = deint_pitch(nx);  // words between the runs of two channels in LDS
+  // Loads are issued two at a time before the first of them is used.
+  constexpr uint32_t kU = 2;
   auto park = [&](auto *lds, const auto *src, int64_t row_stride) {
-    using P4 = Pack<std::remove_cv_t<std::remove_pointer_t<decltype(src)>>, 4>;
-    const uint32_t total = nrows * pitch;
-    for (uint32_t i0 = 4 * threadIdx.x; i0 < total; i0 += 4 * kThreads * kU) {
+    using T = std::remove_cv_t<std::remove_pointer_t<decltype(src)>>;
+    using P4 = Pack<T, 4>;
+    const uint32_t words = nrows * strip4;
+    for (uint32_t i0 = 4 * threadIdx.x; i0 < words; i0 += 4 * kThreads * kU) {
       P4 v[kU];
+      uint32_t prow[kU], j[kU];
 #pragma unroll
       for (uint32_t u = 0; u < kU; ++u) {
         const uint32_t i = i0 + u * 4 * kThreads;
-        const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
-        if (i < total && j < strip) v[u] = load4_edge(src + row * row_stride + j, (int64_t)strip - j);
+        prow[u] = rows > 1 ? div_by(i, sh.by_strip4) : 0u;
+        j[u] = i - prow[u] * strip4;
+        if (i < words && j[u] < strip) v[u] = load4_edge(src + prow[u] * row_stride + j[u], (int64_t)strip - j[u]);
       }
 #pragma unroll
       for (uint32_t u = 0; u < kU; ++u) {
         const uint32_t i = i0 + u * 4 * kThreads;
-        const uint32_t row = rows > 1 ? i / pitch : 0u, j = i - row * pitch;
-        if (i < total && j < strip) *reinterpret_cast<P4 *>(&lds[i]) = v[u];
+        if (i < words && j[u] < strip) {
+          uint32_t px = div_by(j[u], sh.by_p), pc = j[u] - px * P;
+          T *l = lds + prow[u] * P * xpitch;
+#pragma unroll
+          for (uint32_t m = 0; m < 4; ++m) {
+            if (j[u] + m < strip) l[pc * xpitch + px] = v[u].v[m];
+            if (++pc == P) {
+              pc = 0;
+              ++px;
+            }
+          }
+        }
       }
     }
   };
@@ -1015,6 +1060,8 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   const uint32_t packs = (nx + 3) / 4;  // per channel
   const uint32_t per_row = packs * P;
   const uint32_t total = nrows * per_row;
+  // (the divisor by `packs` was made for strips of full length)
+  const bool full = (int64_t)nx == (g.n0 < (int64_t)sh.tx_elems ? g.n0 : (int64_t)sh.tx_elems);
   for (uint32_t idx0 = threadIdx.x; idx0 < total; idx0 += kThreads * kU) {
     PA va[kU];
     PB vb[kU];
@@ -1023,9 +1070,9 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
 #pragma unroll
     for (uint32_t u = 0; u < kU; ++u) {
       const uint32_t idx = idx0 + u * kThreads;
-      row[u] = rows > 1 ? idx / per_row : 0u;
+      row[u] = rows > 1 ? div_by(idx, sh.by_per_row) : 0u;
       const uint32_t rem = idx - row[u] * per_row;
-      c[u] = rem / packs;
+      c[u] = full ? div_by(rem, sh.by_packs) : rem / packs;
       x[u] = 4 * (rem - c[u] * packs);
       if (idx < total) {
         const int64_t left = (int64_t)nx - x[u];
@@ -1040,16 +1087,9 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
       const uint32_t idx = idx0 + u * kThreads;
       if (idx >= total) continue;
       const int64_t left = (int64_t)nx - x[u];
-      if constexpr (A_D) {
-        const TA *l = sa + row[u] * pitch;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) va[u].v[k] = k < left ? l[(x[u] + k) * P + c[u]] : TA();
-      }
-      if constexpr (NIN == 2 && B_D) {
-        const TB *l = sb + row[u] * pitch;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) vb[u].v[k] = k < left ? l[(x[u] + k) * P + c[u]] : TB();
-      }
+      const uint32_t at = (row[u] * P + c[u]) * xpitch + x[u];  // a multiple of 4 words
+      if constexpr (A_D) va[u] = *reinterpret_cast<const PA *>(sa + at);
+      if constexpr (NIN == 2 && B_D) vb[u] = *reinterpret_cast<const PB *>(sb + at);
       PO o;
 #pragma unroll
       for (int k = 0; k < 4; ++k)
@@ -1534,18 +1574,19 @@ int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool 
       tg.nbatch++;
       batch *= g.shape[d];
     }
-    // strip length: 1024 elements of dimension 0 while the strip fits the LDS array
+    const int64_t lds_words = kDeintLds;
+    // strip length: 1024 elements of dimension 0 while the channels' runs fit the LDS array
     uint32_t tx = 1024;
-    while ((int64_t)tx * P > kDeintLds) tx /= 2;
+    while ((int64_t)P * deint_pitch(tx) > lds_words) tx /= 2;
     const int64_t tiles0 = (tg.n0 + tx - 1) / tx;
     // a short dimension 0 (one strip, a fraction of a block's lanes): a block takes several
     // indices of the first batch dimension, as many strips as fit the LDS array and add up
-    // to about 1024 output elements per channel
+    // to about 2048 output elements per channel
     uint32_t rows = 1;
     int64_t row_tiles = 1;
-    if (tg.n0 < 512 && tg.nbatch >= 1) {
-      const int64_t pitch = (tg.n0 * P + 3) / 4 * 4;
-      int64_t fit = kDeintLds / pitch, want = (2048 + tg.n0 - 1) / tg.n0;
+    if (tg.n0 < 512 && tg.n0 <= (int64_t)tx && tg.nbatch >= 1) {  // (one strip covers dimension 0)
+      const int64_t per_strip = P * (int64_t)deint_pitch((uint32_t)tg.n0);
+      int64_t fit = lds_words / per_strip, want = (2048 + tg.n0 - 1) / tg.n0;
       int64_t k = fit < want ? fit : want;
       if (k > tg.bshape[0]) k = tg.bshape[0];
       if (k >= 2) {
@@ -1559,15 +1600,23 @@ int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool 
     tg.tiles0 = (uint32_t)tiles0;
     tg.tilest = (uint32_t)row_tiles;
     const unsigned grid = (unsigned)(tiles0 * batch);
+    // (with rows > 1 every strip is a whole row of dimension 0: the divisors fit all of them)
+    const uint32_t nx_full = (uint32_t)(tg.n0 < (int64_t)tx ? tg.n0 : (int64_t)tx);
+    const uint32_t packs_full = (nx_full + 3) / 4;
+    const uint32_t words = rows * (uint32_t)P * deint_pitch(nx_full);
+    const DeintShape sh{tx, rows, words, small_div((uint32_t)P), small_div((nx_full * (uint32_t)P + 3u) & ~3u),
+                        small_div(packs_full), small_div(packs_full * (uint32_t)P)};
+    const size_t lds_bytes = (size_t)words * 4 * ((a_d ? 1 : 0) + (NIN == 2 && b_d ? 1 : 0));
+#define TWG_DEINT(AD, BD) \
+  ew_deint<NIN, AD, BD, Op, TO, TA, TB><<<grid, kThreads, lds_bytes, s>>>(out, a, b, tg, sh, op)
     if (a_d && b_d) {
-      if constexpr (NIN == 2)
-        ew_deint<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, rows, op);
+      if constexpr (NIN == 2) TWG_DEINT(true, true);
     } else if (a_d) {
-      ew_deint<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, rows, op);
+      TWG_DEINT(true, false);
     } else {
-      if constexpr (NIN == 2)
-        ew_deint<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, tx, rows, op);
+      if constexpr (NIN == 2) TWG_DEINT(false, true);
     }
+#undef TWG_DEINT
     return (int)hipGetLastError();
   }
 }

@@ -79,6 +79,18 @@ TWG_WALK_FN bool decode_tile(const TileWalk &w, uint32_t bid, uint32_t &t0i, uin
   return true;
 }
 
+// n / d by one multiplication, exact while n * d <= 2^32 (for indices into a block's few
+// thousand elements, where a 32-bit division would cost some thirty instructions per lane).
+struct SmallDiv {
+  uint32_t d, m;
+};
+inline SmallDiv small_div(uint32_t d) {
+  return SmallDiv{d, d <= 1 ? 0u : (uint32_t)(((uint64_t(1) << 32) + d - 1) / d)};
+}
+TWG_WALK_FN uint32_t div_by(uint32_t n, SmallDiv s) {
+  return s.d <= 1 ? n : (uint32_t)(((uint64_t)n * s.m) >> 32);
+}
+
 // Workgroups of a launch over tiles0 x tilest tiles in each of `batch` batch entries; 0 when
 // the counts do not fit the 32-bit decoding above.  xcd_walk asks for the per-XCD order where
 // it can be had (more than one tile along t): *ngroups is then the number of pairs and the
