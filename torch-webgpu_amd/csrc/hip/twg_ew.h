@@ -453,6 +453,9 @@ int launch_flat_nd(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
 struct RowGeom {
   int64_t len;               // extent of dimension 0
   uint32_t chunks_per_row;   // blocks along one row
+  // chunks begin on 128-byte lines of the output rather than at the row's start: the first
+  // chunk of a row that starts inside a line is that much shorter
+  uint32_t line_chunks;
   int32_t nouter;            // remaining dimensions
   int64_t oshape[TWG_MAX_DIMS - 1];
   int64_t ostride[3][TWG_MAX_DIMS - 1];
@@ -536,13 +539,17 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
   if constexpr (A_BC) abc = arow[0];
   if constexpr (NIN == 2 && B_BC) bbc = brow[0];
 
-  const int64_t e0 = (int64_t)chunk * (THREADS * VEC * UNROLL) + (int64_t)threadIdx.x * VEC;
+  // (rows of packs start on pack boundaries, so the shift is a whole number of packs)
+  constexpr uint32_t kLineElems = 128 / sizeof(TO);
+  const uint32_t shift =
+      (!ANY && g.line_chunks) ? (uint32_t)((reinterpret_cast<uintptr_t>(orow) / sizeof(TO)) % kLineElems) : 0u;
+  const int64_t e0 = (int64_t)chunk * (THREADS * VEC * UNROLL) + (int64_t)threadIdx.x * VEC - shift;
   PA va[UNROLL];
   PB vb[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int64_t e = e0 + (int64_t)u * THREADS * VEC;
-    if (e < g.len) {
+    if (e >= 0 && e < g.len) {
       if constexpr (ANY) {
         if constexpr (!A_BC) va[u] = load4_edge<(HINTS & 2) != 0>(arow + e, g.len - e);
         if constexpr (NIN == 2 && !B_BC) vb[u] = load4_edge<(HINTS & 4) != 0>(brow + e, g.len - e);
@@ -557,7 +564,7 @@ __global__ __launch_bounds__(THREADS) void ew_rows(TO *out, const TA *a, const T
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int64_t e = e0 + (int64_t)u * THREADS * VEC;
-    if (e < g.len) {
+    if (e >= 0 && e < g.len) {
       PO r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) {
@@ -1141,7 +1148,10 @@ __global__ __launch_bounds__(kThreads) void ew_generic(TO *out, const TA *a, con
 // slices like x[:, :64], [B, H, T, 64] views.  Dimension 0 of the geometry counts packs.
 // With the nontemporal hints of the dense kernel such shapes run at 79-84% of peak at 2^26
 // elements (70-73% without them, 26-44% one element per lane).
-template <int NIN, int VEC, bool A_BC, bool B_BC, bool STREAM, typename Op, typename TO, typename TA,
+// HINTS as in ew_rows: bit 0 the store, bit 1 operand a, bit 2 operand b carry the nontemporal
+// hint; an operand that is broadcast along an outer dimension and read again and again keeps
+// default caching so that it stays in L2.
+template <int NIN, int VEC, bool A_BC, bool B_BC, int HINTS, typename Op, typename TO, typename TA,
           typename TB>
 __global__ __launch_bounds__(64) void ew_generic_vec(TO *out, const TA *a, const TB *b,
                                                      GenGeom<uint32_t, int32_t> g, Op op) {
@@ -1167,7 +1177,7 @@ __global__ __launch_bounds__(64) void ew_generic_vec(TO *out, const TA *a, const
 #pragma unroll
     for (int k = 0; k < VEC; ++k) va.v[k] = x;
   } else {
-    va = load_pack<STREAM>(reinterpret_cast<const PA *>(a + oa));
+    va = load_pack<(HINTS & 2) != 0>(reinterpret_cast<const PA *>(a + oa));
   }
   if constexpr (NIN == 2) {
     if constexpr (B_BC) {
@@ -1175,14 +1185,14 @@ __global__ __launch_bounds__(64) void ew_generic_vec(TO *out, const TA *a, const
 #pragma unroll
       for (int k = 0; k < VEC; ++k) vb.v[k] = y;
     } else {
-      vb = load_pack<STREAM>(reinterpret_cast<const PB *>(b + ob));
+      vb = load_pack<(HINTS & 4) != 0>(reinterpret_cast<const PB *>(b + ob));
     }
   }
   PO r;
 #pragma unroll
   for (int k = 0; k < VEC; ++k)
     r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
-  store_pack<STREAM && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out + oo), r);
+  store_pack<(HINTS & 1) != 0 && sizeof(PO) >= 8>(reinterpret_cast<PO *>(out + oo), r);
 }
 
 // -------------------------------------------------------------- dispatch
@@ -1230,6 +1240,20 @@ int launch_generic(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipS
   return (int)hipGetLastError();
 }
 
+// Is operand o read again and again (broadcast along an outer dimension) and small enough to
+// stay in the last-level cache (256 MB)?  Such an operand keeps default caching while the
+// streamed ones carry the nontemporal hint.
+template <int NIN>
+bool read_again(const Geom &g, int o, size_t esize) {
+  bool again = false;
+  int64_t footprint = (int64_t)esize * (g.stride[o][0] != 0 ? g.shape[0] : 1);
+  for (int d = 1; d < g.ndim; ++d) {
+    if (g.stride[o][d] == 0) again = again || g.shape[d] > 1;
+    else footprint *= g.shape[d];
+  }
+  return again && footprint <= (int64_t(64) << 20);
+}
+
 // Short unit-stride (or broadcast) rows, packs aligned in every operand: ew_generic_vec.
 // Returns TWG_E_UNSUPPORTED when the geometry is not of that kind.
 template <int NIN, typename Op, typename TO, typename TA, typename TB>
@@ -1240,8 +1264,13 @@ int launch_generic_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, 
   } else {
     const int64_t sa0 = g.stride[1][0], sb0 = NIN == 2 ? g.stride[2][0] : 1;
     if (g.ndim < 2 || g.stride[0][0] != 1 || (sa0 != 0 && sa0 != 1) || (sb0 != 0 && sb0 != 1) ||
-        g.shape[0] % VEC != 0 || g.shape[0] >= 256 || g.numel > INT32_MAX)
+        g.shape[0] % VEC != 0 || g.numel > INT32_MAX)
       return TWG_E_UNSUPPORTED;
+    // Rows of a whole number of 64-lane chunks, and long ones, are for ew_rows; other rows from
+    // 256 elements on come here too: ew_rows leaves the lanes past a row's end idle and cuts
+    // its chunks where the rows start, the flat walk does neither (rows of 1000 floats with a
+    // [16, 1, 1000] operand: 75% -> 80% of peak, [128, 64, 56*56] + [128, 1, 56*56]: 74% -> 77%).
+    if (g.shape[0] >= 256 && (g.shape[0] % (64 * VEC) == 0 || g.shape[0] >= 8192)) return TWG_E_UNSUPPORTED;
     // rows of less than a cache line gain nothing over one element per lane (measured)
     if (g.shape[0] * (int64_t)MaxSize<TO, TA, TB>::value < 128) return TWG_E_UNSUPPORTED;
     if constexpr (NIN == 1) {
@@ -1277,12 +1306,18 @@ int launch_generic_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, 
     const unsigned grid = (unsigned)((gg.numel + 63) / 64);
     const bool stream =
         g.numel * (int64_t)(sizeof(TO) + sizeof(TA) + (NIN == 2 ? sizeof(TB) : 0)) > kStreamBytes;
+    const bool a_again = sa0 == 1 && read_again<NIN>(g, 1, sizeof(TA));
+    const bool b_again = NIN == 2 && sb0 == 1 && read_again<NIN>(g, 2, sizeof(TB));
 #define TWG_GV(ABC, BBC)                                                                          \
   do {                                                                                            \
-    if (stream)                                                                                   \
-      ew_generic_vec<NIN, VEC, ABC, BBC, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
+    if (!stream)                                                                                  \
+      ew_generic_vec<NIN, VEC, ABC, BBC, 0, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
+    else if (!ABC && a_again)                                                                     \
+      ew_generic_vec<NIN, VEC, ABC, BBC, 1 | 4, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
+    else if (!BBC && b_again)                                                                     \
+      ew_generic_vec<NIN, VEC, ABC, BBC, 1 | 2, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
     else                                                                                          \
-      ew_generic_vec<NIN, VEC, ABC, BBC, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
+      ew_generic_vec<NIN, VEC, ABC, BBC, 1 | 2 | 4, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
   } while (0)
     if constexpr (NIN == 2) {
       if (sa0 == 0 && sb0 == 0) TWG_GV(true, true);
@@ -1308,25 +1343,43 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
     rg.oshape[d - 1] = g.shape[d];
     for (int o = 0; o < 3; ++o) rg.ostride[o][d - 1] = g.stride[o][d];
   }
-  // operand k is read again and again (broadcast along an outer dimension) and small enough
-  // to stay in the last-level cache (256 MB): it keeps default caching while the streamed
-  // operands carry the hint
-  bool reused[3] = {false, false, false};
-  for (int o = 1; o <= NIN; ++o) {
-    bool again = false;
-    int64_t footprint = (o == 1 ? sizeof(TA) : sizeof(TB)) * (g.stride[o][0] != 0 ? g.shape[0] : 1);
-    for (int d = 1; d < g.ndim; ++d) {
-      if (g.stride[o][d] == 0) again = again || g.shape[d] > 1;
-      else footprint *= g.shape[d];
-    }
-    reused[o] = again && footprint <= (int64_t(64) << 20);
-  }
+  // an operand that is read again and again keeps default caching while the streamed ones
+  // carry the hint
+  const bool reused[3] = {false, read_again<NIN>(g, 1, sizeof(TA)),
+                          NIN == 2 && read_again<NIN>(g, 2, sizeof(TB))};
   const bool stream = g.numel * (int64_t)(sizeof(TO) + sizeof(TA)) > kStreamBytes;
   const int64_t rows = g.numel / rg.len;
   // Blocks of the grid for packs-per-lane U; 0 if that does not fit a launch.
+  // Rows that do not all start on 128-byte lines of the output (a row pitch of 1000 floats):
+  // chunks cut at the row's start straddle a line each, which the neighbouring chunk, on
+  // another XCD, fetches and writes a second time (69% of peak against 80% for rows of 1024).
+  // From three chunks per row on, the chunks are cut at the output's lines instead; the row
+  // then needs room for the largest shift any row start has, (base + k * gcd) mod line.
+  constexpr int64_t kLineElems = 128 / sizeof(TO);
+  int64_t max_shift = 0;
+  if (!ANY) {
+    int64_t gcd = kLineElems;
+    auto fold = [&](int64_t v) {
+      v = v < 0 ? -v : v;
+      v %= kLineElems;
+      while (v) {
+        const int64_t t = gcd % v;
+        gcd = v;
+        v = t;
+      }
+    };
+    for (int d = 1; d < g.ndim; ++d) fold(g.stride[0][d]);
+    const int64_t base = (int64_t)((reinterpret_cast<uintptr_t>(out) / sizeof(TO)) % kLineElems);
+    if (gcd != kLineElems || base != 0) max_shift = base % gcd + kLineElems - gcd;
+  }
   auto grid_for = [&](int U) -> unsigned {
     const int64_t per_block = (int64_t)kBlock * VEC * U;
-    const int64_t cpr = (rg.len + per_block - 1) / per_block;
+    int64_t cpr = (rg.len + per_block - 1) / per_block;
+    rg.line_chunks = 0;
+    if (max_shift > 0 && cpr >= 3) {
+      rg.line_chunks = 1;
+      cpr = (rg.len + max_shift + per_block - 1) / per_block;
+    }
     if (cpr * rows > INT32_MAX || cpr > UINT32_MAX) return 0u;
     rg.chunks_per_row = (uint32_t)cpr;
     return (unsigned)(cpr * rows);
