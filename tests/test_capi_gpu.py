@@ -293,6 +293,8 @@ def test_add_transposed_operand(twg, rows, cols):
     ((8, 130, 64, 64), (3, 2, 0, 1)), ((3, 40, 9, 64), (3, 2, 0, 1)), ((5, 33, 7, 50), (3, 2, 0, 1)),
     ((4, 64, 10, 96), (2, 3, 0, 1)), ((2, 3, 70, 5, 24), (0, 4, 3, 1, 2)), ((37, 11, 20), (2, 1, 0)),
     ((2, 100, 3, 85), (3, 2, 0, 1)),
+    # a transposed extent of 33..64 elements under a wide dimension 0: one 64-wide tile along it
+    ((64, 5, 8, 64), (1, 2, 3, 0)), ((64, 300), (1, 0)), ((48, 3, 520), (2, 1, 0)),
 ])
 def test_add_permuted_operand_tiles(twg, shape, order):
     # `a` is stored with its dimensions in `order` (outermost first) and viewed in the logical

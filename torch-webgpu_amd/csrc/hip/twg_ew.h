@@ -1555,13 +1555,20 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       }
     }
     if (ok) {
-      if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid)) return TWG_E_UNSUPPORTED;
+      // A transposed extent of 33..64 elements is one 64-wide tile: with 256 x 32 tiles each
+      // 256-byte row of the transposed operand was fetched half by one workgroup, half by
+      // another (`[64,128,64,64]` stored with dimension 0 innermost: 67-73% -> 71-78% of peak).
+      const bool one_t_tile = wide && tg.nt > 32 && tg.nt <= 64;
+      if (!set_tiles(one_t_tile ? 64 : wide ? 256 : mid ? 128 : 64, (wide && !one_t_tile) ? 32 : 64, &grid))
+        return TWG_E_UNSUPPORTED;
       // 256x32 tiles: 512 lanes per tile measured 2-4 points ahead of 256 from 2^22 to 2^26
       // elements (67% -> 71% at 2^24), 1024 lanes another point ahead at 2^28 (77.6%)
       const bool big = g.numel >= (int64_t(1) << 27);
 #define TWG_LAUNCH_TILE_VEC(AT, BT)                                                              \
   do {                                                                                           \
-    if (wide && big)                                                                             \
+    if (one_t_tile)                                                                              \
+      ew_tile_vec<NIN, AT, BT, 64, 64, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);  \
+    else if (wide && big)                                                                             \
       ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 1024><<<grid, 1024, 0, s>>>(out, a, b, tg, op); \
     else if (wide)                                                                               \
       ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
