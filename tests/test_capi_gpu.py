@@ -147,6 +147,46 @@ def test_copy_sizes_around_every_staging_boundary(twg):
         assert bool((back[:3] == 0xEE).all()) and bool((back[3 + nb:3 + nb + 61] == 0xEE).all()), nb
 
 
+def test_uploads_through_the_outbox(twg):
+    # Uploads of 1 KiB..64 KiB are copied into a pinned slot and fetched by a kernel that then
+    # releases the slot: every size class and destination alignment, many more uploads in a row
+    # than there are slots (each to its own place, checked at the end), and uploads queued
+    # behind a long kernel, so that the host has to wait for a slot.
+    L = twg.load()
+    g = torch.Generator().manual_seed(123)
+    raw = torch.randint(0, 256, (1 << 20,), dtype=torch.uint8, generator=g)
+    dev = twg.DeviceBuffer((1 << 20) + 64)
+    back = torch.empty((1 << 20) + 64, dtype=torch.uint8)
+    for nb in (1025, 1040, 2048, 4096, 4099, 16384, 40000, 65535, 65536, 65537):
+        for dst_off in (0, 4, 16, 3):
+            twg.check(L.twg_fill_bytes(dev.ptr, 0xEE, nb + 64, None))
+            twg.check(L.twg_memcpy_h2d(dev.ptr + dst_off, raw.data_ptr() + 5, nb, None))
+            twg.check(L.twg_memcpy_d2h(back.data_ptr(), dev.ptr, nb + 64, None))
+            assert torch.equal(back[dst_off:dst_off + nb], raw[5:5 + nb]), (nb, dst_off)
+            assert bool((back[:dst_off] == 0xEE).all()) and bool((back[dst_off + nb:nb + 64] == 0xEE).all()), (nb, dst_off)
+    # 100 uploads of 8 KiB back to back, the host buffer overwritten right after each call
+    piece = 8192
+    scratch = torch.empty(piece, dtype=torch.uint8)
+    for i in range(100):
+        scratch.copy_(raw[i * piece:(i + 1) * piece])
+        twg.check(L.twg_memcpy_h2d(dev.ptr + i * piece, scratch.data_ptr(), piece, None))
+        scratch.fill_(0)
+    twg.check(L.twg_memcpy_d2h(back.data_ptr(), dev.ptr, 100 * piece, None))
+    assert torch.equal(back[:100 * piece], raw[:100 * piece])
+    # the same behind a kernel that keeps the stream busy for a while
+    n = 1 << 27
+    big_a, big_o = twg.DeviceBuffer(4 * n), twg.DeviceBuffer(4 * n)
+    it = twg.make_iter([n], [1], [1])
+    for _ in range(4):
+        twg.check(L.twg_unary_f32(twg.UNARY_GELU_ERF, big_o.ptr, big_a.ptr, ctypes.byref(it), None))
+    for i in range(40):
+        scratch.copy_(raw[(i + 7) * piece:(i + 8) * piece])
+        twg.check(L.twg_memcpy_h2d(dev.ptr + i * piece, scratch.data_ptr(), piece, None))
+        scratch.fill_(1)
+    twg.check(L.twg_memcpy_d2h(back.data_ptr(), dev.ptr, 40 * piece, None))
+    assert torch.equal(back[:40 * piece], raw[7 * piece:47 * piece])
+
+
 def test_copies_with_a_small_pinned_ring(twg):
     # TWG_STAGE_RING_MIB shrinks the pinned ring (what the library also does by itself when
     # 64 MiB cannot be pinned): every copy size must still round-trip.  The variable is read

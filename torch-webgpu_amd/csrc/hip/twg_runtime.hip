@@ -117,6 +117,8 @@ constexpr int kMailboxSlots = 8;
 constexpr size_t kMailboxStride = kMailboxBytes + 64;       // payload, sequence word, padding
 constexpr size_t kFlowFlagBytes = 128 * sizeof(uint32_t);  // flags of a small download
 constexpr int kMailboxSpins = 200000;                      // then fall back to a stream sync
+constexpr size_t kOutboxSlotBytes = 65536;                 // largest upload served by an outbox slot
+constexpr int kOutboxSlots = 8;
 
 // Bytes a copy of nbytes moves per DMA.  Each hipMemcpyAsync + event record costs ~17 us
 // of host time and a transfer only reaches the link's rate when it is several MiB long,
@@ -162,6 +164,25 @@ struct Staging {
   uint32_t *flow_flags = nullptr;  // coherent pinned: one word per 64 KiB piece of a small download
   void *flow_flags_dev = nullptr;
   uint32_t flow_seq = 0;
+  // Outbox for uploads of up to kOutboxSlotBytes: the host copies the bytes into a slot of
+  // coherent pinned memory and launches a kernel that reads them over the link and then
+  // stores the slot's sequence number into its flag, which says the slot may be refilled.
+  // No DMA and no event: ~5 us of host time against ~12.5 us through the ring.
+  char *outbox = nullptr;  // kOutboxSlots slots, then one flag word per slot (64 bytes apart)
+  void *outbox_dev = nullptr;
+  uint32_t outbox_seq[kOutboxSlots] = {};      // sequence number of the slot's last upload
+  hipStream_t outbox_stream[kOutboxSlots] = {};  // and the stream it went to
+  uint32_t outbox_counter = 0;
+  int outbox_next = 0;
+  char *out_slot(int i) const { return outbox + (size_t)i * kOutboxSlotBytes; }
+  char *out_slot_dev(int i) const { return static_cast<char *>(outbox_dev) + (size_t)i * kOutboxSlotBytes; }
+  uint32_t *out_flag(int i) const {
+    return reinterpret_cast<uint32_t *>(outbox + (size_t)kOutboxSlots * kOutboxSlotBytes + (size_t)i * 64);
+  }
+  uint32_t *out_flag_dev(int i) const {
+    return reinterpret_cast<uint32_t *>(static_cast<char *>(outbox_dev) + (size_t)kOutboxSlots * kOutboxSlotBytes +
+                                        (size_t)i * 64);
+  }
 };
 
 // Copy out of a staging slot into pageable memory.  Large destinations do not fit in
@@ -343,6 +364,10 @@ int staging_prepare_locked(Staging &s) {
                             hipHostMallocCoherent | hipHostMallocMapped));
   TWG_HIP_TRY(hipHostGetDevicePointer(&s.flow_flags_dev, s.flow_flags, 0));
   std::memset(s.flow_flags, 0, kFlowFlagBytes);
+  TWG_HIP_TRY(hipHostMalloc((void **)&s.outbox, kOutboxSlots * (kOutboxSlotBytes + 64),
+                            hipHostMallocCoherent | hipHostMallocMapped));
+  TWG_HIP_TRY(hipHostGetDevicePointer(&s.outbox_dev, s.outbox, 0));
+  std::memset(s.outbox + kOutboxSlots * kOutboxSlotBytes, 0, kOutboxSlots * 64);
   s.ready = true;
   return 0;
 }
@@ -456,6 +481,71 @@ __global__ __launch_bounds__(kFlowLanes) void d2h_flow_kernel(uint8_t *ring, con
     __syncthreads();
     if (t == 0) __hip_atomic_store(flags + p, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
+}
+
+// One workgroup moves an outbox slot into device memory: every lane's loads are issued before
+// the first store, 16 bytes each where the destination allows it.  Once every lane holds its
+// part (its stores have been issued, so its loads have returned) the slot's flag is released.
+constexpr int kOutboxLanes = 1024;
+__global__ __launch_bounds__(kOutboxLanes) void outbox_kernel(uint8_t *dst, const uint8_t *slot, uint32_t n,
+                                                              uint32_t *flag, uint32_t seq) {
+  const uint32_t t = threadIdx.x;
+  uint32_t done = 0;
+  const uint32_t align = (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u);  // the slot is 16-byte aligned
+  if (align == 0) {
+    constexpr uint32_t kPer = (uint32_t)(kOutboxSlotBytes / 16 / kOutboxLanes);  // 4
+    const uint32_t nv = n / 16;
+    uint4 v[kPer];
+#pragma unroll
+    for (uint32_t k = 0; k < kPer; ++k) {
+      const uint32_t i = t + k * kOutboxLanes;
+      if (i < nv) v[k] = reinterpret_cast<const uint4 *>(slot)[i];
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kPer; ++k) {
+      const uint32_t i = t + k * kOutboxLanes;
+      if (i < nv) reinterpret_cast<uint4 *>(dst)[i] = v[k];
+    }
+    done = nv * 16;
+  } else if ((align & 3u) == 0) {
+    const uint32_t nw = n / 4;
+    for (uint32_t i = t; i < nw; i += kOutboxLanes)
+      reinterpret_cast<uint32_t *>(dst)[i] = reinterpret_cast<const uint32_t *>(slot)[i];
+    done = nw * 4;
+  }
+  for (uint32_t i = done + t; i < n; i += kOutboxLanes) dst[i] = slot[i];
+  __syncthreads();
+  if (t == 0) __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+static_assert(kOutboxSlotBytes % (16 * kOutboxLanes) == 0, "whole 16-byte parts per lane");
+
+// Upload n <= kOutboxSlotBytes bytes through the next outbox slot; call with the staging lock held.
+int outbox_upload_locked(Staging &st, void *dst, const void *src, size_t n, hipStream_t s) {
+  const int slot = st.outbox_next;
+  st.outbox_next = (slot + 1) % kOutboxSlots;
+  if (st.outbox_seq[slot] != 0) {  // the kernel that last read this slot must have let go of it
+    const uint32_t *flag = st.out_flag(slot);
+    bool seen = false;
+    for (int i = 0; i < kMailboxSpins && !seen; ++i) {
+      seen = __atomic_load_n(flag, __ATOMIC_ACQUIRE) == st.outbox_seq[slot];
+      if (!seen) _mm_pause();
+    }
+    if (!seen) {  // a long queue ahead of that kernel: wait properly
+      TWG_HIP_TRY(hipStreamSynchronize(st.outbox_stream[slot]));
+      if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != st.outbox_seq[slot]) return (int)hipErrorUnknown;
+    }
+  }
+  std::memcpy(st.out_slot(slot), src, n);
+  uint32_t seq = ++st.outbox_counter;
+  if (seq == 0) seq = ++st.outbox_counter;  // 0 means "never used"
+  outbox_kernel<<<1, kOutboxLanes, 0, s>>>(static_cast<uint8_t *>(dst),
+                                            reinterpret_cast<const uint8_t *>(st.out_slot_dev(slot)), (uint32_t)n,
+                                            st.out_flag_dev(slot), seq);
+  const int rc = (int)hipGetLastError();
+  if (rc) return rc;  // (the slot's old sequence number stands: nothing new will release it)
+  st.outbox_seq[slot] = seq;
+  st.outbox_stream[slot] = s;
+  return 0;
 }
 
 // Uploads of a few bytes (a scalar, a shape) travel as a kernel argument: the launch copies
@@ -670,6 +760,7 @@ int twg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, twg_strea
   Staging &st = staging();
   std::lock_guard<std::mutex> lk(st.mu);
   if ((rc = staging_prepare_locked(st))) return rc;
+  if (nbytes <= kOutboxSlotBytes) return outbox_upload_locked(st, dst_dev, src_host, nbytes, s);
   if ((rc = staging_divide_locked(st, nbytes, true))) return rc;
   const char *src = static_cast<const char *>(src_host);
   char *dst = static_cast<char *>(dst_dev);
