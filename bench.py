@@ -493,8 +493,9 @@ def geometry_families(capi, L):
     """add.Tensor on ~2^25 fp32 elements with (a) the second operand broadcast in every possible
     way over a set of 2- to 4-dimensional shapes, (b) the first operand stored in every
     permutation of its dimensions and (c) one or both operands slices of a larger storage.  Reports algorithmic bytes / time as % of the HBM peak: the
-    slowest patterns and the median of each family.  Median of three batches of 10 launches,
-    each batch between one pair of events on the library's stream."""
+    slowest patterns and the median of each family.  Median of three batches of 12 launches,
+    each batch between one pair of events on the library's stream, consecutive launches on
+    three sets of operands in turn."""
     import itertools
 
     def contig(shape):
@@ -504,28 +505,40 @@ def geometry_families(capi, L):
             acc *= s
         return list(reversed(st))
 
+    # Consecutive launches go to three different sets of operands in turn: at this size one set
+    # is 400 MB, and launched again and again on the same set, a kernel that reads an operand
+    # with default caching finds a good part of it in the 256 MB last-level cache the launch
+    # before left there (a reversed [128,56,56,96] operand: 83% of "HBM peak" on one set, 65%
+    # in rotation; kernels whose loads carry the nontemporal hint read the same either way).
+    kSets = 3
+
+    def median_launch_seconds(run):
+        for i in range(kSets):
+            run(i)
+        capi.sync()
+        batches = []
+        for _ in range(3):  # median of three batches of 12 launches between one event pair
+            e0, e1 = capi.Event(), capi.Event()
+            e0.record()
+            for i in range(12):
+                run(i % kSets)
+            e1.record()
+            capi.sync()
+            batches.append(e0.elapsed_ms(e1) / 12)
+        return statistics.median(batches) / 1e3
+
     def timed(shape, a_st, b_st, nb):
         n = 1
         for s in shape:
             n *= s
-        da, db, do = capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * max(nb, 1)), capi.DeviceBuffer(4 * n)
+        sets = [(capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * max(nb, 1)), capi.DeviceBuffer(4 * n))
+                for _ in range(kSets)]
         it = capi.make_iter(shape, contig(shape), a_st, b_st)
 
-        def run():
+        def run(i):
+            da, db, do = sets[i]
             capi.check(L.twg_add_f32(do.ptr, da.ptr, db.ptr, ctypes.c_float(1.0), ctypes.byref(it), None))
-        for _ in range(3):
-            run()
-        capi.sync()
-        batches = []
-        for _ in range(3):  # median of three batches of 10 launches between one event pair
-            e0, e1 = capi.Event(), capi.Event()
-            e0.record()
-            for _ in range(10):
-                run()
-            e1.record()
-            capi.sync()
-            batches.append(e0.elapsed_ms(e1) / 10)
-        t = statistics.median(batches) / 1e3
+        t = median_launch_seconds(run)
         return round((8 * n + 4 * nb) / t / 1e9 / HBM_PEAK_GBS * 100, 1), round(t * 1e3, 4)
 
     fam = {}
@@ -580,27 +593,16 @@ def geometry_families(capi, L):
         st_storage = contig(storage)
         a_st = [st * k for st, k in zip(st_storage, steps)]
         off = sum(b0 * st for b0, st in zip(starts, st_storage))
-        da, do = capi.DeviceBuffer(4 * ns), capi.DeviceBuffer(4 * n)
-        db = capi.DeviceBuffer(4 * (ns if both else n))
+        sets = [(capi.DeviceBuffer(4 * ns), capi.DeviceBuffer(4 * (ns if both else n)), capi.DeviceBuffer(4 * n))
+                for _ in range(kSets)]
         b_st = a_st if both else contig(shape)
         it = capi.make_iter(shape, contig(shape), a_st, b_st)
-        pa, pb = da.ptr + 4 * off, db.ptr + (4 * off if both else 0)
 
-        def run():
-            capi.check(L.twg_add_f32(do.ptr, pa, pb, ctypes.c_float(1.0), ctypes.byref(it), None))
-        for _ in range(3):
-            run()
-        capi.sync()
-        batches = []
-        for _ in range(3):
-            e0, e1 = capi.Event(), capi.Event()
-            e0.record()
-            for _ in range(10):
-                run()
-            e1.record()
-            capi.sync()
-            batches.append(e0.elapsed_ms(e1) / 10)
-        t = statistics.median(batches) / 1e3
+        def run(i):
+            da, db, do = sets[i]
+            capi.check(L.twg_add_f32(do.ptr, da.ptr + 4 * off, db.ptr + (4 * off if both else 0),
+                                     ctypes.c_float(1.0), ctypes.byref(it), None))
+        t = median_launch_seconds(run)
         return round(12 * n / t / 1e9 / HBM_PEAK_GBS * 100, 1), round(t * 1e3, 4)
 
     rows_ = []
@@ -633,6 +635,7 @@ def geometry_families(capi, L):
     log(f"slice family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
         f"slowest {rows_[0]['pct_hbm_peak']}%")
     return {"geometry_families": fam, "elements_per_pattern": "about 2^25", "op": "add.Tensor fp32",
+            "operand_sets_in_rotation": kSets,
             "bytes": "4 B per element read per full operand + 4 B written; a broadcast operand counts its own size; "
                      "a stepped operand counts the elements used, not the lines touched"}
 
