@@ -115,6 +115,45 @@ int main() {
       for (int64_t e = -2; e <= 2; ++e)
         if (!check(q * d + e) || !check((top / d > q ? top / d - q : 0) * d + e)) return fail("small_div near a multiple", d, (long)q, (long)e, 0);
   }
+  // rows cut at the output's lines: the room reserved for the largest offset of a row start into
+  // its line must cover every row start there is (brute force over small outer extents), and
+  // is exact when the extents are large enough to reach every residue
+  {
+    uint64_t state = 12345;
+    auto rnd = [&](uint32_t n) {
+      state = state * 6364136223846793005ull + 1442695040888963407ull;
+      return (uint32_t)((state >> 33) % n);
+    };
+    for (int iter = 0; iter < 20000; ++iter) {
+      const int64_t line = 32 << rnd(3);  // 32, 64 or 128 elements
+      const int nd = 1 + (int)rnd(3);
+      int64_t stride[3], extent[3];
+      for (int d = 0; d < nd; ++d) {
+        stride[d] = (int64_t)(rnd(4) == 0 ? line * (1 + rnd(5)) : 4 * (1 + rnd(600)));
+        if (rnd(8) == 0) stride[d] = -stride[d];
+        extent[d] = 1 + rnd(nd == 1 ? 200 : 12);
+      }
+      const int64_t base = 4 * (int64_t)rnd(5000);
+      const int64_t bound = twg::max_line_shift(base, stride, nd, line);
+      int64_t worst = 0;
+      int64_t idx[3] = {0, 0, 0};
+      for (;;) {
+        int64_t start = base;
+        for (int d = 0; d < nd; ++d) start += idx[d] * stride[d];
+        const int64_t shift = ((start % line) + line) % line;
+        if (shift > worst) worst = shift;
+        int d = 0;
+        for (; d < nd; ++d) {
+          if (++idx[d] < extent[d]) break;
+          idx[d] = 0;
+        }
+        if (d == nd) break;
+      }
+      if (worst > bound) return fail("a row starts further into its line than the room reserved", line, base, worst, (int)bound);
+      if (bound >= line) return fail("shift bound beyond a line", line, base, bound, 0);
+      if (nd == 1 && extent[0] >= line && worst != bound) return fail("shift bound not attained", line, base, worst, (int)bound);
+    }
+  }
   std::printf("tile walk ok (%d launches)\n", launches);
   return 0;
 }

@@ -1,0 +1,783 @@
+// Elementwise kernels for an operand whose unit stride lies along another dimension than the
+// output's: tiles transposed through LDS (ew_tile, ew_tile_vec, ew_tile_any) and strips
+// deinterleaved through LDS (ew_deint), with their launchers.
+#pragma once
+
+#include "twg_ew_packs.h"
+#include "twg_tile_walk.h"
+
+namespace twg {
+namespace {
+
+// --------------------------------------------------------------- ew_tile
+
+constexpr int kTile = 64;
+
+struct TileGeom : TileWalk {  // tile counts, batch extents and the walk order come from there
+  int64_t n0, nt;          // extents of dimension 0 and of the transposed dimension t
+  int64_t s0[3], st[3];    // strides along those two, per operand
+  // ew_tile_any only: t may be the product of two dimensions, q (outer, extent nt / psplit,
+  // strides st) and p (inner, extent psplit, strides sp), that lie back to back in the
+  // memory of the transposed operands (their offset along t is the index itself) but not in
+  // the other operands.  psplit == 1: t is one dimension.
+  int64_t sp[3];
+  uint32_t psplit;
+  // ew_tile_vec / ew_tile_any: dimension 0 may be the product of two dimensions, the inner one
+  // of extent n0in (strides s0) and the next one (strides s1), that lie back to back in the
+  // memory of the output and of the operands that are not transposed (their offset along
+  // dimension 0 is the index itself) but not in the transposed operands, whose row r sits at
+  // (r % n0in) * s0 + (r / n0in) * s1.  n0in == 0: dimension 0 is one dimension.
+  uint32_t n0in;
+  int64_t s1[3];
+  int64_t bstride[3][TWG_MAX_DIMS - 2];
+};
+
+// Offset of row r (an index along dimension 0) of a transposed operand.
+__device__ __forceinline__ int64_t tile_row_off(const TileGeom &g, int o, int64_t r) {
+  if (g.n0in == 0) return r * g.s0[o];
+  const uint32_t q = (uint32_t)r / g.n0in;
+  const uint32_t rem = (uint32_t)r - q * g.n0in;
+  return (int64_t)rem * g.s0[o] + (int64_t)q * g.s1[o];
+}
+
+// Which tile a workgroup takes (twg_tile_walk.h) and the operand offsets of its batch entry;
+// false for the workgroups that pad the grid.
+template <bool XCD_ORDER, int NIN>
+__device__ __forceinline__ bool tile_of_block(const TileGeom &g, uint32_t bid, uint32_t &t0i,
+                                              uint32_t &tti, int64_t &off_o, int64_t &off_a,
+                                              int64_t &off_b) {
+  off_o = off_a = off_b = 0;
+  return decode_tile<XCD_ORDER>(g, bid, t0i, tti, [&](int d, uint32_t i) {
+    off_o += (int64_t)i * g.bstride[0][d];
+    off_a += (int64_t)i * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += (int64_t)i * g.bstride[2][d];
+  });
+}
+
+// Lane x (0..63) runs along dimension 0, the 4 wavefronts and 16 steps cover 64
+// positions along t.  An operand marked *_T has its unit stride along t: it is
+// read with lane x along t instead, parked in LDS and picked up transposed.
+template <int NIN, bool A_T, bool B_T, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_tile(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                    Op op) {
+  __shared__ TA sa[A_T ? kTile : 1][kTile + 1];
+  __shared__ TB sb[(NIN == 2 && B_T) ? kTile : 1][kTile + 1];
+
+  uint32_t t0i, tti;
+  int64_t off_o, off_a, off_b;
+  tile_of_block<false, NIN>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b);
+  const int x = threadIdx.x & 63;
+  const int y = threadIdx.x >> 6;  // 0..3
+  const int64_t base0 = (int64_t)t0i * kTile;
+  const int64_t baset = (int64_t)tti * kTile;
+
+  if constexpr (A_T) {
+    const int64_t tt = baset + x;
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) {
+      const int64_t d0 = base0 + y + 4 * k;
+      if (tt < g.nt && d0 < g.n0) sa[y + 4 * k][x] = a[off_a + d0 * g.s0[1] + tt * g.st[1]];
+    }
+  }
+  if constexpr (NIN == 2 && B_T) {
+    const int64_t tt = baset + x;
+#pragma unroll
+    for (int k = 0; k < kTile / 4; ++k) {
+      const int64_t d0 = base0 + y + 4 * k;
+      if (tt < g.nt && d0 < g.n0) sb[y + 4 * k][x] = b[off_b + d0 * g.s0[2] + tt * g.st[2]];
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+
+  const int64_t d0 = base0 + x;
+  if (d0 >= g.n0) return;
+#pragma unroll 4
+  for (int k = 0; k < kTile / 4; ++k) {
+    const int tl = y + 4 * k;
+    const int64_t tt = baset + tl;
+    if (tt >= g.nt) break;
+    TA va;
+    TB vb = TB();
+    if constexpr (A_T) {
+      va = sa[x][tl];
+    } else {
+      va = a[off_a + d0 * g.s0[1] + tt * g.st[1]];
+    }
+    if constexpr (NIN == 2) {
+      if constexpr (B_T) {
+        vb = sb[x][tl];
+      } else {
+        vb = b[off_b + d0 * g.s0[2] + tt * g.st[2]];
+      }
+    }
+    out[off_o + d0 * g.s0[0] + tt * g.st[0]] = apply<NIN, Op, TO, TA, TB>(op, va, vb);
+  }
+}
+
+// Same job with 128-bit accesses on both sides of the transpose, for 4-byte
+// elements when extents, strides and pointers are all multiples of 4 elements.
+// Tile = TD0 (dimension 0) x TT (dimension t).  The output and the operands with
+// unit stride along dimension 0 move as float4 runs of TD0 elements; an operand
+// marked *_T is read as float4 runs of TT elements along t, scattered into LDS as
+// st[t][d0] (row pitch TD0 + 4 keeps the float4 reads aligned) and read back along
+// dimension 0.  Wide tiles matter: 256 x 32 reaches 79% of HBM peak on the
+// [32768, 8192] transposed add, 64 x 64 only 66%, one dword per lane 52%.
+//
+// The body of one tile.  FULL: the tile lies inside both extents, so nothing is predicated:
+// loads under a per-lane condition make the compiler wait for every outstanding load at
+// each later use, and a kernel whose tiles are all whole (config 3b: 32768 x 8192 in
+// 256 x 32 tiles) runs 1.2-1.5 points of HBM peak faster without them (77.9% -> 79.3%).
+// The operands that need no transpose are requested first: their loads do not depend on
+// LDS, and ahead of the transposed operand's scatter they are in flight while it waits.
+// SPLIT0: dimension 0 is the product of two dimensions (TileGeom::n0in); kept out of the plain
+// body at compile time, where even a never-taken branch per row cost a point on config 3b.
+template <bool FULL, bool SPLIT0, int NIN, bool A_T, bool B_T, int TD0, int TT, int THREADS,
+          typename Op, typename TO, typename TA, typename TB, typename SA, typename SB>
+__device__ __forceinline__ void tile_vec_body(TO *out, const TA *a, const TB *b, const TileGeom &g,
+                                              const Op &op, int64_t base0, int64_t baset,
+                                              SA &sa, SB &sb) {
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  // everything but the transposed operands: float4 along dimension 0
+  constexpr int kLanes0 = TD0 / 4, kRows0 = THREADS / kLanes0, kPass0 = TT / kRows0;
+  static_assert(TD0 % 4 == 0 && THREADS % kLanes0 == 0 && TT % kRows0 == 0, "tile shape");
+  const int tx0 = threadIdx.x % kLanes0, ty0 = threadIdx.x / kLanes0;
+  const int64_t d0 = base0 + 4 * tx0;
+  PA va[kPass0];
+  PB vb[kPass0];
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int64_t tt = baset + ty0 + kRows0 * p;
+    if (FULL || (d0 < g.n0 && tt < g.nt)) {
+      if constexpr (!A_T) va[p] = load_pack<true>(reinterpret_cast<const PA *>(a + d0 + tt * g.st[1]));
+      if constexpr (NIN == 2 && !B_T)
+        vb[p] = load_pack<true>(reinterpret_cast<const PB *>(b + d0 + tt * g.st[2]));
+    }
+  }
+
+  // transposed operands: float4 along t -> LDS[t][d0]
+  constexpr int kLanesT = TT / 4, kRowsT = THREADS / kLanesT, kPassT = TD0 / kRowsT;
+  static_assert(TT % 4 == 0 && THREADS % kLanesT == 0 && TD0 % kRowsT == 0, "tile shape");
+  {
+    const int tx = threadIdx.x % kLanesT, ty = threadIdx.x / kLanesT;
+    const int64_t tt = baset + 4 * tx;
+    if constexpr (A_T) {
+      PA v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t r0 = base0 + ty + kRowsT * p;
+        if (FULL || (r0 < g.n0 && tt < g.nt))
+          v[p] = load_pack<true>(reinterpret_cast<const PA *>(
+              a + (SPLIT0 ? tile_row_off(g, 1, r0) : r0 * g.s0[1]) + tt));
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (FULL || (base0 + rr < g.n0 && tt < g.nt)) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sa[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+    if constexpr (NIN == 2 && B_T) {
+      PB v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t r0 = base0 + ty + kRowsT * p;
+        if (FULL || (r0 < g.n0 && tt < g.nt))
+          v[p] = load_pack<true>(reinterpret_cast<const PB *>(
+              b + (SPLIT0 ? tile_row_off(g, 2, r0) : r0 * g.s0[2]) + tt));
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (FULL || (base0 + rr < g.n0 && tt < g.nt)) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sb[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int rr = ty0 + kRows0 * p;
+    const int64_t tt = baset + rr;
+    if (FULL || (d0 < g.n0 && tt < g.nt)) {
+      if constexpr (A_T) va[p] = *reinterpret_cast<const PA *>(&sa[rr][4 * tx0]);
+      if constexpr (NIN == 2 && B_T) vb[p] = *reinterpret_cast<const PB *>(&sb[rr][4 * tx0]);
+      PO o;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        o.v[c] = apply<NIN, Op, TO, TA, TB>(op, va[p].v[c], NIN == 2 ? vb[p].v[c] : TB());
+      store_pack<true>(reinterpret_cast<PO *>(out + d0 + tt * g.st[0]), o);
+    }
+  }
+}
+
+template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO, typename TA,
+          typename TB, int THREADS = kThreads>
+__global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, const TB *b,
+                                                        TileGeom g, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  constexpr int kPitch = TD0 + 4;
+  __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
+  __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
+
+  // (this kernel only gets line-aligned pieces, so its tiles are always dealt in plain order)
+  uint32_t t0i, tti;
+  int64_t off_o, off_a, off_b;
+  tile_of_block<false, NIN>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b);
+  const int64_t base0 = (int64_t)t0i * TD0;
+  const int64_t baset = (int64_t)tti * TT;
+  // workgroup-uniform: whole tiles take the unpredicated body
+  const bool whole = base0 + TD0 <= g.n0 && baset + TT <= g.nt;
+#define TWG_TILE_BODY(FULL, SPLIT0)                                                              \
+  tile_vec_body<FULL, SPLIT0, NIN, A_T, B_T, TD0, TT, THREADS>(out + off_o, a + off_a, b + off_b, g, \
+                                                               op, base0, baset, sa, sb)
+  if (g.n0in == 0) {
+    if (whole) TWG_TILE_BODY(true, false); else TWG_TILE_BODY(false, false);
+  } else {
+    if (whole) TWG_TILE_BODY(true, true); else TWG_TILE_BODY(false, true);
+  }
+#undef TWG_TILE_BODY
+}
+
+// The same tile kernel without its alignment conditions.  Wide global loads and stores need
+// only 4-byte alignment on this hardware, so rows whose pitch is not a multiple of 4 elements
+// (a batched [197, 768] transpose) still move as 16-byte packs; extents that are not multiples
+// of 4 end in packs that are handled element by element.  The transposed dimension may be
+// the product of two dimensions (TileGeom::psplit): an operand stored as [.., q, p] with a short
+// innermost extent p (3 channels, 16, 56) is read in unit-stride runs across q and p, while
+// the output rows are addressed by (t / p, t % p).
+template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO, typename TA,
+          typename TB, int THREADS>
+__global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, const TB *b,
+                                                        TileGeom g, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  constexpr int kPitch = TD0 + 4;
+  __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
+  __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
+
+  uint32_t t0i, tti;
+  int64_t off_o, off_a, off_b;
+  if (!tile_of_block<true, NIN>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b)) return;  // workgroup-uniform
+  const int64_t base0 = (int64_t)t0i * TD0;
+  const int64_t baset = (int64_t)tti * TT;
+
+  // transposed operands: 4 elements along t per lane -> LDS[t][d0]
+  constexpr int kLanesT = TT / 4, kRowsT = THREADS / kLanesT, kPassT = TD0 / kRowsT;
+  static_assert(TT % 4 == 0 && THREADS % kLanesT == 0 && TD0 % kRowsT == 0, "tile shape");
+  {
+    const int tx = threadIdx.x % kLanesT, ty = threadIdx.x / kLanesT;
+    const int64_t tt = baset + 4 * tx;
+    const int64_t left = g.nt - tt;  // elements of this lane's pack inside the extent
+    if constexpr (A_T) {
+      PA v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t d0 = base0 + ty + kRowsT * p;
+        // (default caching: a neighbouring tile reads the other part of these lines)
+        if (d0 < g.n0 && left > 0) v[p] = load4_edge<false>(a + off_a + tile_row_off(g, 1, d0) + tt, left);
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (base0 + rr < g.n0 && left > 0) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sa[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+    if constexpr (NIN == 2 && B_T) {
+      PB v[kPassT];
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int64_t d0 = base0 + ty + kRowsT * p;
+        if (d0 < g.n0 && left > 0) v[p] = load4_edge<false>(b + off_b + tile_row_off(g, 2, d0) + tt, left);
+      }
+#pragma unroll
+      for (int p = 0; p < kPassT; ++p) {
+        const int rr = ty + kRowsT * p;
+        if (base0 + rr < g.n0 && left > 0) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sb[4 * tx + c][rr] = v[p].v[c];
+        }
+      }
+    }
+  }
+
+  // everything else: 4 elements along dimension 0 per lane
+  constexpr int kLanes0 = TD0 / 4, kRows0 = THREADS / kLanes0, kPass0 = TT / kRows0;
+  static_assert(TD0 % 4 == 0 && THREADS % kLanes0 == 0 && TT % kRows0 == 0, "tile shape");
+  const int tx = threadIdx.x % kLanes0, ty = threadIdx.x / kLanes0;
+  const int64_t d0 = base0 + 4 * tx;
+  const int64_t left0 = g.n0 - d0;
+  // offset of row tt of operand o: a plain stride, or (tt / p, tt % p) on two of them
+  auto row_off = [&](int64_t tt, int o) -> int64_t {
+    if (g.psplit <= 1) return tt * g.st[o];
+    const uint32_t q = (uint32_t)tt / g.psplit;
+    const uint32_t rem = (uint32_t)tt - q * g.psplit;
+    return (int64_t)q * g.st[o] + (int64_t)rem * g.sp[o];
+  };
+  PA va[kPass0];
+  PB vb[kPass0];
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int64_t tt = baset + ty + kRows0 * p;
+    if (left0 > 0 && tt < g.nt) {
+      if constexpr (!A_T) va[p] = load4_edge(a + off_a + d0 + row_off(tt, 1), left0);
+      if constexpr (NIN == 2 && !B_T) vb[p] = load4_edge(b + off_b + d0 + row_off(tt, 2), left0);
+    }
+  }
+  if constexpr (A_T || (NIN == 2 && B_T)) __syncthreads();
+#pragma unroll
+  for (int p = 0; p < kPass0; ++p) {
+    const int rr = ty + kRows0 * p;
+    const int64_t tt = baset + rr;
+    if (left0 > 0 && tt < g.nt) {
+      if constexpr (A_T) va[p] = *reinterpret_cast<const PA *>(&sa[rr][4 * tx]);
+      if constexpr (NIN == 2 && B_T) vb[p] = *reinterpret_cast<const PB *>(&sb[rr][4 * tx]);
+      PO o;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        o.v[c] = apply<NIN, Op, TO, TA, TB>(op, va[p].v[c], NIN == 2 ? vb[p].v[c] : TB());
+      TO *dst = out + off_o + d0 + row_off(tt, 0);
+      if (left0 >= 4) {
+        store4_any(dst, o);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (c < left0) dst[c] = o.v[c];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------ ew_deint
+// An operand stored as [.., x, c] with a short innermost extent c (3 colour channels, a handful
+// of heads) against an output laid out [.., c, x]: the operand's stride along dimension 0 is the
+// extent of c.  A block reads a strip of TX * c consecutive elements with 16-byte loads and
+// parks it in LDS one run of x per channel, so that the second phase picks up four consecutive
+// x of one channel with one 16-byte LDS read and writes c runs of TX output elements.
+// (Through the gather kernel these layouts ran at 51% of HBM peak.)
+//
+// The transposition happens on the way into LDS, element by element, because that is the side
+// where it can be had without bank conflicts: with the strip parked as it lies in memory, the
+// lanes of a wavefront that pick up x, x+4, x+8.. of one channel are 4*c words apart, which
+// for c = 16 is the same bank for all 64 of them.  A channel's run starts deint_pitch(nx)
+// words after the previous one's, a multiple of 4 (16-byte reads) that is 4 modulo 32: the
+// four words a lane scatters and the words of its neighbours then fall into different banks
+// for every c but multiples of 8 (two lanes per bank).  (Worth 2 points at c = 16.)
+//
+// What sets the rate is how many blocks a CU holds, not how much one block keeps in flight: a
+// block goes through load strip -> LDS -> barrier -> load the straight operands -> store, and
+// only other blocks fill the gaps.  With 36 KiB of LDS per block (4 blocks per CU, 8192
+// elements each) these layouts ran at 65-74% of peak; with 9 KiB (the 8 blocks the CU's
+// wavefront slots allow, ~2000 elements each, two 16-byte loads per lane in flight) at 75-82%.
+// Issuing all of a big block's loads at once was the worst of all (44-50%).
+constexpr int kDeintLds = 2304;  // words of LDS per deinterleaved operand and block at most
+__host__ __device__ constexpr uint32_t deint_pitch(uint32_t nx) { return (nx + 27u) / 32u * 32u + 4u; }
+
+struct DeintShape {
+  uint32_t tx_elems;  // elements of dimension 0 per strip
+  uint32_t rows;      // strips per block (consecutive indices of the first batch dimension)
+  uint32_t lds_words; // words of LDS per deinterleaved operand
+  SmallDiv by_p;      // the channel count
+  SmallDiv by_strip4; // a full strip's length in memory, rounded up to packs
+  SmallDiv by_packs;  // packs of output per channel and full strip
+  SmallDiv by_per_row;  // by_packs.d * P
+};
+
+template <int NIN, bool A_D, bool B_D, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                     DeintShape sh, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  // sh.lds_words words per deinterleaved operand, sized by the launch
+  extern __shared__ __attribute__((aligned(16))) unsigned char deint_lds[];
+  TA *sa = reinterpret_cast<TA *>(deint_lds);
+  TB *sb = reinterpret_cast<TB *>(deint_lds) + (A_D ? sh.lds_words : 0u);
+
+  const uint32_t rows = sh.rows;
+  uint32_t bid = blockIdx.x;
+  const uint32_t t0i = bid % g.tiles0;
+  int64_t r = bid / g.tiles0;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  // rows > 1 (dimension 0 is short): the block takes `rows` consecutive indices of the first
+  // batch dimension, one strip each
+  uint32_t nrows = 1;
+  int d_first = 0;
+  if (rows > 1) {
+    const uint32_t q = (uint32_t)r / g.tilest;
+    const int64_t row0 = (int64_t)((uint32_t)r - q * g.tilest) * rows;
+    r = q;
+    nrows = (uint32_t)(g.bshape[0] - row0 < (int64_t)rows ? g.bshape[0] - row0 : (int64_t)rows);
+    off_o = row0 * g.bstride[0][0];
+    off_a = row0 * g.bstride[1][0];
+    if constexpr (NIN == 2) off_b = row0 * g.bstride[2][0];
+    d_first = 1;
+  }
+  for (int d = d_first; d < g.nbatch; ++d) {
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = (uint32_t)r / extent;  // batch indices fit 32 bits, the grid does
+    const int64_t c = (uint32_t)r - q * extent;
+    r = q;
+    off_o += c * g.bstride[0][d];
+    off_a += c * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += c * g.bstride[2][d];
+  }
+  const uint32_t P = (uint32_t)g.nt;
+  const int64_t x0 = (int64_t)t0i * sh.tx_elems;
+  const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)sh.tx_elems ? g.n0 - x0 : (int64_t)sh.tx_elems);
+  const uint32_t strip = nx * P;  // consecutive elements of a deinterleaved operand
+  // (the last strip along dimension 0 may be shorter than the one the divisors were made for;
+  // then a block takes one strip only and those divisors are not used)
+  const uint32_t strip4 = (strip + 3u) & ~3u;
+  const uint32_t xpitch = deint_pitch(nx);  // words between the runs of two channels in LDS
+  // Loads are issued two at a time before the first of them is used.
+  constexpr uint32_t kU = 2;
+  auto park = [&](auto *lds, const auto *src, int64_t row_stride) {
+    using T = std::remove_cv_t<std::remove_pointer_t<decltype(src)>>;
+    using P4 = Pack<T, 4>;
+    const uint32_t words = nrows * strip4;
+    for (uint32_t i0 = 4 * threadIdx.x; i0 < words; i0 += 4 * kThreads * kU) {
+      P4 v[kU];
+      uint32_t prow[kU], j[kU];
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * 4 * kThreads;
+        prow[u] = rows > 1 ? div_by(i, sh.by_strip4) : 0u;
+        j[u] = i - prow[u] * strip4;
+        if (i < words && j[u] < strip) v[u] = load4_edge(src + prow[u] * row_stride + j[u], (int64_t)strip - j[u]);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * 4 * kThreads;
+        if (i < words && j[u] < strip) {
+          uint32_t px = div_by(j[u], sh.by_p), pc = j[u] - px * P;
+          T *l = lds + prow[u] * P * xpitch;
+#pragma unroll
+          for (uint32_t m = 0; m < 4; ++m) {
+            if (j[u] + m < strip) l[pc * xpitch + px] = v[u].v[m];
+            if (++pc == P) {
+              pc = 0;
+              ++px;
+            }
+          }
+        }
+      }
+    }
+  };
+  if constexpr (A_D) park(sa, a + off_a + x0 * (int64_t)P, g.bstride[1][0]);
+  if constexpr (NIN == 2 && B_D) park(sb, b + off_b + x0 * (int64_t)P, g.bstride[2][0]);
+  __syncthreads();
+  const uint32_t packs = (nx + 3) / 4;  // per channel
+  const uint32_t per_row = packs * P;
+  const uint32_t total = nrows * per_row;
+  // (the divisor by `packs` was made for strips of full length)
+  const bool full = (int64_t)nx == (g.n0 < (int64_t)sh.tx_elems ? g.n0 : (int64_t)sh.tx_elems);
+  for (uint32_t idx0 = threadIdx.x; idx0 < total; idx0 += kThreads * kU) {
+    PA va[kU];
+    PB vb[kU];
+    uint32_t row[kU], c[kU], x[kU];
+    // the operands that come straight from memory first, all kU of them
+#pragma unroll
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t idx = idx0 + u * kThreads;
+      row[u] = rows > 1 ? div_by(idx, sh.by_per_row) : 0u;
+      const uint32_t rem = idx - row[u] * per_row;
+      c[u] = full ? div_by(rem, sh.by_packs) : rem / packs;
+      x[u] = 4 * (rem - c[u] * packs);
+      if (idx < total) {
+        const int64_t left = (int64_t)nx - x[u];
+        if constexpr (!A_D)
+          va[u] = load4_edge(a + off_a + row[u] * g.bstride[1][0] + x0 + x[u] + (int64_t)c[u] * g.st[1], left);
+        if constexpr (NIN == 2 && !B_D)
+          vb[u] = load4_edge(b + off_b + row[u] * g.bstride[2][0] + x0 + x[u] + (int64_t)c[u] * g.st[2], left);
+      }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t idx = idx0 + u * kThreads;
+      if (idx >= total) continue;
+      const int64_t left = (int64_t)nx - x[u];
+      const uint32_t at = (row[u] * P + c[u]) * xpitch + x[u];  // a multiple of 4 words
+      if constexpr (A_D) va[u] = *reinterpret_cast<const PA *>(sa + at);
+      if constexpr (NIN == 2 && B_D) vb[u] = *reinterpret_cast<const PB *>(sb + at);
+      PO o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va[u].v[k], NIN == 2 ? vb[u].v[k] : TB());
+      TO *dst = out + off_o + row[u] * g.bstride[0][0] + x0 + x[u] + (int64_t)c[u] * g.st[0];
+      if (left >= 4) {
+        store4_any(dst, o);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (k < left) dst[k] = o.v[k];
+      }
+    }
+  }
+}
+
+// t: the dimension the transposed operands have their unit stride along; or, with pin >= 1,
+// the outer one of two dimensions (t, pin) that lie back to back in those operands' memory
+// (unit stride along pin, stride shape[pin] along t) and are walked as one.  merge01: the
+// output and the operands that are not transposed are dense across dimensions 0 and 1 (the
+// caller has checked), which are then walked as one dimension of shape[0] * shape[1] elements,
+// so that short rows (64 elements against a 256-wide tile) still move in pieces of 1 KiB.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
+                hipStream_t s, int pin = -1, bool merge01 = false) {
+  TileGeom tg{};
+  tg.n0 = g.shape[0];
+  tg.nt = g.shape[t];
+  tg.psplit = 1;
+  for (int o = 0; o < 3; ++o) {
+    tg.s0[o] = g.stride[o][0];
+    tg.st[o] = g.stride[o][t];
+    tg.sp[o] = 0;
+  }
+  if (merge01) {
+    if (t < 2 || pin >= 0 || g.ndim < 3) return TWG_E_UNSUPPORTED;
+    if (g.shape[0] * g.shape[1] >= (int64_t(1) << 31)) return TWG_E_UNSUPPORTED;
+    tg.n0 = g.shape[0] * g.shape[1];
+    tg.n0in = (uint32_t)g.shape[0];
+    for (int o = 0; o < 3; ++o) tg.s1[o] = g.stride[o][1];
+  }
+  if (pin >= 1) {
+    if (g.shape[t] * g.shape[pin] >= (int64_t(1) << 31)) return TWG_E_UNSUPPORTED;
+    tg.nt = g.shape[t] * g.shape[pin];
+    tg.psplit = (uint32_t)g.shape[pin];
+    for (int o = 0; o < 3; ++o) tg.sp[o] = g.stride[o][pin];
+  }
+  int64_t batch = 1;
+  tg.nbatch = 0;
+  for (int d = 1; d < g.ndim; ++d) {
+    if (d == t || d == pin || (merge01 && d == 1)) continue;
+    tg.bshape[tg.nbatch] = g.shape[d];
+    for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+    tg.nbatch++;
+    batch *= g.shape[d];
+  }
+  // the leading batch dimensions along which the output is denser than along t are walked
+  // before t (decode_tile)
+  tg.nb_inner = 0;
+  {
+    auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+    int64_t along_t = mag(tg.st[0]);
+    if (tg.psplit > 1 && mag(tg.sp[0]) < along_t) along_t = mag(tg.sp[0]);
+    while (tg.nb_inner < tg.nbatch && mag(tg.bstride[0][tg.nb_inner]) < along_t) ++tg.nb_inner;
+  }
+  // Do the pieces of a transposed operand (32 or 64 elements along t) start and end on
+  // 128-byte lines?  If not, tiles that are neighbours along t share lines.
+  auto ragged = [&](int o, const void *base) {
+    bool lines = reinterpret_cast<uintptr_t>(base) % 128 == 0 && tg.s0[o] % 32 == 0 && tg.s1[o] % 32 == 0;
+    for (int d = 0; d < tg.nbatch && lines; ++d) lines = tg.bstride[o][d] % 32 == 0;
+    return !lines;
+  };
+  const bool ragged_t = (a_t && ragged(1, a)) || (NIN == 2 && b_t && ragged(2, b));
+  // xcd_walk: only ew_tile_any decodes the block index that way
+  auto set_tiles = [&](int td0, int tt, unsigned *grid, bool xcd_walk = false) {
+    const int64_t tiles0 = (tg.n0 + td0 - 1) / td0;
+    const int64_t tilest = (tg.nt + tt - 1) / tt;
+    // pieces of a transposed operand that share 128-byte lines with their neighbours along
+    // t: let one XCD walk along t (decode_tile)
+    const int64_t blocks = tile_grid(tiles0, tilest, batch, xcd_walk && ragged_t, &tg.ngroups);
+    if (blocks == 0) return false;
+    tg.tiles0 = (uint32_t)tiles0;
+    tg.tilest = (uint32_t)tilest;
+    *grid = (unsigned)blocks;
+    return true;
+  };
+  unsigned grid = 0;
+
+  // 128-bit path: 4-byte elements, everything a multiple of 4 elements, and every
+  // operand with its unit stride either along dimension 0 or (if marked) along t.
+  if constexpr (sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4) {
+    bool ok = tg.n0 % 4 == 0 && tg.nt % 4 == 0 && tg.s0[0] == 1 && tg.st[0] % 4 == 0 &&
+              aligned_to(out, 16) && aligned_to(a, 16) && (NIN == 1 || aligned_to(b, 16));
+    ok = ok && (a_t ? (tg.st[1] == 1 && tg.s0[1] % 4 == 0 && tg.s1[1] % 4 == 0)
+                    : (tg.s0[1] == 1 && tg.st[1] % 4 == 0));
+    if (NIN == 2)
+      ok = ok && (b_t ? (tg.st[2] == 1 && tg.s0[2] % 4 == 0 && tg.s1[2] % 4 == 0)
+                      : (tg.s0[2] == 1 && tg.st[2] % 4 == 0));
+    for (int d = 0; d < tg.nbatch && ok; ++d)
+      for (int o = 0; o <= NIN; ++o) ok = ok && tg.bstride[o][d] % 4 == 0;
+    // (pieces that share lines with their neighbours go to the kernel below, which reads the
+    // transposed operands with default caching and lets one XCD walk along t)
+    ok = ok && pin < 0 && !ragged_t;
+    // tile shape by the extent of dimension 0: 256 x 32 from 256 on, 128 x 64 where a 128-wide
+    // tile wastes no more lanes than two 64-wide ones (96: 54% -> 6x% of peak), else 64 x 64
+    const bool wide = tg.n0 >= 256;
+    const bool mid = !wide && tg.n0 > 64 && (tg.n0 % 128 == 0 || tg.n0 % 128 > 64);
+    if (!ok) {
+      // The same tiles without the alignment conditions, and with (t, pin) walked as one
+      // dimension: needs the unit strides only.
+      auto unit_t = [&](int o) {
+        return pin >= 1 ? (tg.sp[o] == 1 && tg.st[o] == (int64_t)tg.psplit) : tg.st[o] == 1;
+      };
+      bool any = tg.s0[0] == 1 && (a_t ? unit_t(1) : tg.s0[1] == 1);
+      if (NIN == 2) any = any && (b_t ? unit_t(2) : tg.s0[2] == 1);
+      if (any) {
+        if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid, true)) return TWG_E_UNSUPPORTED;
+        const bool big = g.numel >= (int64_t(1) << 27);
+#define TWG_LAUNCH_TILE_ANY(AT, BT)                                                              \
+  do {                                                                                           \
+    if (wide && big)                                                                             \
+      ew_tile_any<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 1024><<<grid, 1024, 0, s>>>(out, a, b, tg, op); \
+    else if (wide)                                                                               \
+      ew_tile_any<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else if (mid)                                                                                \
+      ew_tile_any<NIN, AT, BT, 128, 64, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else                                                                                         \
+      ew_tile_any<NIN, AT, BT, 64, 64, Op, TO, TA, TB, kThreads><<<grid, kThreads, 0, s>>>(out, a, b, tg, op); \
+  } while (0)
+        if (a_t && b_t) {
+          if constexpr (NIN == 2) TWG_LAUNCH_TILE_ANY(true, true);
+        } else if (a_t) {
+          TWG_LAUNCH_TILE_ANY(true, false);
+        } else {
+          if constexpr (NIN == 2) TWG_LAUNCH_TILE_ANY(false, true);
+        }
+#undef TWG_LAUNCH_TILE_ANY
+        return (int)hipGetLastError();
+      }
+    }
+    if (ok) {
+      // A transposed extent of 33..64 elements is one 64-wide tile: with 256 x 32 tiles each
+      // 256-byte row of the transposed operand was fetched half by one workgroup, half by
+      // another (`[64,128,64,64]` stored with dimension 0 innermost: 67-73% -> 71-78% of peak).
+      const bool one_t_tile = wide && tg.nt > 32 && tg.nt <= 64;
+      if (!set_tiles(one_t_tile ? 64 : wide ? 256 : mid ? 128 : 64, (wide && !one_t_tile) ? 32 : 64, &grid))
+        return TWG_E_UNSUPPORTED;
+      // 256x32 tiles: 512 lanes per tile measured 2-4 points ahead of 256 from 2^22 to 2^26
+      // elements (67% -> 71% at 2^24), 1024 lanes another point ahead at 2^28 (77.6%)
+      const bool big = g.numel >= (int64_t(1) << 27);
+#define TWG_LAUNCH_TILE_VEC(AT, BT)                                                              \
+  do {                                                                                           \
+    if (one_t_tile)                                                                              \
+      ew_tile_vec<NIN, AT, BT, 64, 64, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);  \
+    else if (wide && big)                                                                             \
+      ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 1024><<<grid, 1024, 0, s>>>(out, a, b, tg, op); \
+    else if (wide)                                                                               \
+      ew_tile_vec<NIN, AT, BT, 256, 32, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else if (mid)                                                                                \
+      ew_tile_vec<NIN, AT, BT, 128, 64, Op, TO, TA, TB, 512><<<grid, 512, 0, s>>>(out, a, b, tg, op); \
+    else                                                                                         \
+      ew_tile_vec<NIN, AT, BT, 64, 64, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);  \
+  } while (0)
+      if (a_t && b_t) {
+        if constexpr (NIN == 2) TWG_LAUNCH_TILE_VEC(true, true);
+      } else if (a_t) {
+        TWG_LAUNCH_TILE_VEC(true, false);
+      } else {
+        if constexpr (NIN == 2) TWG_LAUNCH_TILE_VEC(false, true);
+      }
+#undef TWG_LAUNCH_TILE_VEC
+      return (int)hipGetLastError();
+    }
+  }
+
+  if (pin >= 1 || merge01) return TWG_E_UNSUPPORTED;  // the dword kernel walks one dimension only
+  if (!set_tiles(kTile, kTile, &grid)) return TWG_E_UNSUPPORTED;
+  if (a_t && b_t) {
+    if constexpr (NIN == 2)
+      ew_tile<NIN, true, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  } else if (a_t) {
+    ew_tile<NIN, true, false, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  } else {
+    if constexpr (NIN == 2)
+      ew_tile<NIN, false, true, Op, TO, TA, TB><<<grid, kThreads, 0, s>>>(out, a, b, tg, op);
+  }
+  return (int)hipGetLastError();
+}
+
+// Dimension 0 (extent X) and dimension pd (short extent P) form one unit-stride run of X * P
+// elements in the operands marked *_d, while the output and the other operands have their unit
+// stride along dimension 0.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool a_d, bool b_d,
+                 Op op, hipStream_t s) {
+  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    const int64_t P = g.shape[pd];
+    // (from 32 elements on, a run of P is a whole 128-byte line and the tile kernels do better)
+    if (P < 2 || P >= 32 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
+    auto run_of = [&](int o) { return g.stride[o][pd] == 1 && g.stride[o][0] == P; };
+    if (a_d ? !run_of(1) : g.stride[1][0] != 1) return TWG_E_UNSUPPORTED;
+    if (NIN == 2 && (b_d ? !run_of(2) : g.stride[2][0] != 1)) return TWG_E_UNSUPPORTED;
+    TileGeom tg{};
+    tg.n0 = g.shape[0];
+    tg.nt = P;
+    for (int o = 0; o < 3; ++o) {
+      tg.s0[o] = g.stride[o][0];
+      tg.st[o] = g.stride[o][pd];
+    }
+    int64_t batch = 1;
+    tg.nbatch = 0;
+    for (int d = 1; d < g.ndim; ++d) {
+      if (d == pd) continue;
+      tg.bshape[tg.nbatch] = g.shape[d];
+      for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+      tg.nbatch++;
+      batch *= g.shape[d];
+    }
+    const int64_t lds_words = kDeintLds;
+    // strip length: 1024 elements of dimension 0 while the channels' runs fit the LDS array
+    uint32_t tx = 1024;
+    while ((int64_t)P * deint_pitch(tx) > lds_words) tx /= 2;
+    const int64_t tiles0 = (tg.n0 + tx - 1) / tx;
+    // a short dimension 0 (one strip, a fraction of a block's lanes): a block takes several
+    // indices of the first batch dimension, as many strips as fit the LDS array and add up
+    // to about 2048 output elements per channel
+    uint32_t rows = 1;
+    int64_t row_tiles = 1;
+    if (tg.n0 < 512 && tg.n0 <= (int64_t)tx && tg.nbatch >= 1) {  // (one strip covers dimension 0)
+      const int64_t per_strip = P * (int64_t)deint_pitch((uint32_t)tg.n0);
+      int64_t fit = lds_words / per_strip, want = (2048 + tg.n0 - 1) / tg.n0;
+      int64_t k = fit < want ? fit : want;
+      if (k > tg.bshape[0]) k = tg.bshape[0];
+      if (k >= 2) {
+        rows = (uint32_t)k;
+        row_tiles = (tg.bshape[0] + k - 1) / k;
+        batch = batch / tg.bshape[0] * row_tiles;
+      }
+    }
+    if (tg.n0 < 256 && rows < 2) return TWG_E_UNSUPPORTED;  // the gather kernel is as fast
+    if (tiles0 > INT32_MAX || tiles0 * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+    tg.tiles0 = (uint32_t)tiles0;
+    tg.tilest = (uint32_t)row_tiles;
+    const unsigned grid = (unsigned)(tiles0 * batch);
+    // (with rows > 1 every strip is a whole row of dimension 0: the divisors fit all of them)
+    const uint32_t nx_full = (uint32_t)(tg.n0 < (int64_t)tx ? tg.n0 : (int64_t)tx);
+    const uint32_t packs_full = (nx_full + 3) / 4;
+    const uint32_t words = rows * (uint32_t)P * deint_pitch(nx_full);
+    const DeintShape sh{tx, rows, words, small_div((uint32_t)P), small_div((nx_full * (uint32_t)P + 3u) & ~3u),
+                        small_div(packs_full), small_div(packs_full * (uint32_t)P)};
+    const size_t lds_bytes = (size_t)words * 4 * ((a_d ? 1 : 0) + (NIN == 2 && b_d ? 1 : 0));
+#define TWG_DEINT(AD, BD) \
+  ew_deint<NIN, AD, BD, Op, TO, TA, TB><<<grid, kThreads, lds_bytes, s>>>(out, a, b, tg, sh, op)
+    if (a_d && b_d) {
+      if constexpr (NIN == 2) TWG_DEINT(true, true);
+    } else if (a_d) {
+      TWG_DEINT(true, false);
+    } else {
+      if constexpr (NIN == 2) TWG_DEINT(false, true);
+    }
+#undef TWG_DEINT
+    return (int)hipGetLastError();
+  }
+}
+
+
+}  // namespace
+}  // namespace twg

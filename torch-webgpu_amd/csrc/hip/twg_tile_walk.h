@@ -91,6 +91,26 @@ TWG_WALK_FN uint32_t div_by(uint32_t n, SmallDiv s) {
   return s.d <= 1 ? n : (uint32_t)(((uint64_t)n * s.m) >> 32);
 }
 
+// Rows start at base + sum(c_d * stride_d) elements, c_d any index along outer dimension d.
+// How far past the last multiple of `line` elements (a power of two) can a row start lie?  The
+// starts are congruent to base modulo g = gcd(line, strides), so no further than
+// base % g + line - g; 0 when every row starts on a line.
+inline int64_t max_line_shift(int64_t base, const int64_t *stride, int nstrides, int64_t line) {
+  int64_t g = line;
+  for (int d = 0; d < nstrides; ++d) {
+    int64_t v = stride[d] < 0 ? -stride[d] : stride[d];
+    v %= line;
+    while (v) {  // g = gcd(g, v)
+      const int64_t t = g % v;
+      g = v;
+      v = t;
+    }
+  }
+  base %= line;
+  if (g == line && base == 0) return 0;
+  return base % g + line - g;
+}
+
 // Workgroups of a launch over tiles0 x tilest tiles in each of `batch` batch entries; 0 when
 // the counts do not fit the 32-bit decoding above.  xcd_walk asks for the per-XCD order where
 // it can be had (more than one tile along t): *ngroups is then the number of pairs and the
