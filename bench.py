@@ -433,7 +433,46 @@ def dispatcher_lines(args, capi, W, torch, n, rows, cols, K, Wm, time_launches, 
 
     line("masked_select_p0.50", ms_call, W.masked_select_bytes(n, k50),
          c_abi("masked_select_p0.50", "op_ms_with_count_readback"))
+    del src, m
+    res.append(small_call_latency(torch, F))
     return res
+
+
+def small_call_latency(torch, F):
+    """What one call costs the host on tensors too small for the GPU to matter (1024 floats; 4 KiB
+    for the upload): microseconds per call over 2000 calls issued back to back, and the same
+    with the queue drained at the end (equal when the GPU keeps up with the host)."""
+    a = torch.randn(1024).to("webgpu")
+    b = torch.randn(1024).to("webgpu")
+    o = torch.empty_like(a)
+    m = (torch.randn(1024) > 0).to("webgpu")
+    h = torch.randn(1024)
+    one = a[:1]
+
+    def drain():
+        one.cpu()  # a read of four bytes is the sync point
+
+    out = {}
+    for name, fn, reps in (("add", lambda: a + b, 2000), ("add_out", lambda: torch.add(a, b, out=o), 2000),
+                           ("gelu", lambda: F.gelu(a), 2000), ("eq", lambda: torch.eq(a, b), 2000),
+                           ("empty", lambda: torch.empty(1024, device="webgpu"), 2000),
+                           ("as_strided", lambda: a.as_strided((512,), (2,)), 2000),
+                           ("masked_select_with_count", lambda: torch.masked_select(a, m), 500),
+                           ("upload_4KiB", lambda: o.copy_(h), 2000),
+                           ("read_4_bytes", lambda: one.cpu(), 1000), ("item", lambda: one.item(), 1000)):
+        for _ in range(100):
+            fn()
+        drain()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        t1 = time.perf_counter()
+        drain()
+        t2 = time.perf_counter()
+        out[name] = {"host_us": round((t1 - t0) / reps * 1e6, 2), "drained_us": round((t2 - t0) / reps * 1e6, 2)}
+    log("  host microseconds per call on 1024-element tensors: " +
+        ", ".join(f"{k} {v['host_us']}" for k, v in out.items()))
+    return {"op": "small_call_latency", "elements": 1024, "us_per_call": out}
 
 
 def first_launches(capi, L, torch, n, launches=40):
