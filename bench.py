@@ -73,6 +73,10 @@ def main():
                     help="instead of the benchmark: time 40 consecutive gelu launches one by one on buffers "
                          "in different states (fresh from hipMalloc, filled once, recycled by the pool, after "
                          "2 s of idle time) and print the series as one JSON line")
+    ap.add_argument("--chain", action="store_true",
+                    help="instead of the benchmark: time a chain of five dependent elementwise ops "
+                         "(gelu, add, relu, mul, silu) on tensors of 8 to 256 MiB, the inputs taken in turn "
+                         "from four sets and the intermediates recycled, and print one JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this op path is single-GPU (no collectives, nothing to shard in one "
@@ -91,6 +95,9 @@ def main():
         return
     if args.first_launches:
         print(json.dumps(first_launches(capi, L, torch, 1 << args.log2n)), flush=True)
+        return
+    if args.chain:
+        print(json.dumps(op_chain(capi, L)), flush=True)
         return
     dev_name, cus, mem = capi.device_info()
     log(f"device: {dev_name}  CUs={cus}  mem={mem / 2**30:.0f} GiB")
@@ -526,6 +533,49 @@ def first_launches(capi, L, torch, n, launches=40):
         run(f"pass {rep}: input and output fresh, right after the previous series", din, dout)
         dout.free(); din.free()
     return {"first_launches": series, "elements": n, "kernel": "ew_contig<GeluErfOp>", "unit": "us per launch"}
+
+
+def op_chain(capi, L):
+    """t1 = gelu(x); t2 = t1 + y; t3 = relu(t2); t1 = t3 * t2; t2 = silu(t1) on dense fp32 tensors of
+    2^21 .. 2^26 elements: what an op's result being (or not being) in the last-level cache is worth
+    to the op that consumes it.  x and y come in turn from four sets, so only the intermediates
+    can be found cached.  Microseconds per chain over 40 chains between one pair of events."""
+    rows = []
+    for log2n in range(21, 27):
+        n = 1 << log2n
+        it = capi.dense_iter(n)
+        pairs = [(capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * n)) for _ in range(4)]
+        for x, y in pairs:
+            capi.check(L.twg_fill_bytes(x.ptr, 0x3c, 4 * n, None))
+            capi.check(L.twg_fill_bytes(y.ptr, 0x3c, 4 * n, None))
+        t1, t2, t3 = capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * n), capi.DeviceBuffer(4 * n)
+        one = ctypes.c_float(1.0)
+
+        def chain(i):
+            x, y = pairs[i % 4]
+            capi.check(L.twg_unary_f32(capi.UNARY_GELU_ERF, t1.ptr, x.ptr, ctypes.byref(it), None))
+            capi.check(L.twg_add_f32(t2.ptr, t1.ptr, y.ptr, one, ctypes.byref(it), None))
+            capi.check(L.twg_unary_f32(capi.UNARY_RELU, t3.ptr, t2.ptr, ctypes.byref(it), None))
+            capi.check(L.twg_mul_f32(t1.ptr, t3.ptr, t2.ptr, ctypes.byref(it), None))
+            capi.check(L.twg_unary_f32(capi.UNARY_SILU, t2.ptr, t1.ptr, ctypes.byref(it), None))
+        for i in range(4):
+            chain(i)
+        capi.sync()
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for i in range(40):
+            chain(i)
+        e1.record()
+        capi.sync()
+        ms = e0.elapsed_ms(e1) / 40
+        nbytes = (8 + 12 + 8 + 12 + 8) * n
+        rows.append({"log2_elements": log2n, "tensor_MiB": 4 * n >> 20, "chain_us": round(ms * 1e3, 1),
+                     "GBps": round(nbytes / ms / 1e6), "pct_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS * 100, 1)})
+        log(f"  2^{log2n}: {rows[-1]['chain_us']} us per chain, {rows[-1]['pct_hbm_peak']}% of HBM peak on algorithmic bytes")
+        for x, y in pairs:
+            x.free(); y.free()
+        t1.free(); t2.free(); t3.free()
+    return {"op_chain": rows, "ops": "gelu, add, relu, mul, silu", "bytes_per_element": 48}
 
 
 def geometry_families(capi, L):

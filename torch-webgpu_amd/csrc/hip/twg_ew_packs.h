@@ -19,10 +19,14 @@ constexpr int kThreads = 256;  // 4 wavefronts of 64
 #define TWG_ROWS_UNROLL 1
 #endif
 
-// Operands larger than this in total are treated as streaming (touched once, bigger
-// than the caches): loads and stores carry the nontemporal hint.  Smaller problems
-// keep default caching so a following op can hit in L2 / Infinity Cache.
-constexpr int64_t kStreamBytes = int64_t(64) << 20;
+// An op that moves more than this in total is treated as streaming (bigger than the 256 MB
+// last-level cache, every byte touched once): loads and stores carry the nontemporal hint, which
+// keeps them out of that cache.  Smaller ops keep default caching so that the op that consumes
+// the result finds it there: a chain of five dependent elementwise ops on 64 MiB tensors runs in
+// 119 us against 127 us with the hint, on 128 MiB tensors (its unary ops just fit) in 228 us
+// against 244 us; from 256 MiB tensors on nothing fits and the hint is worth 8% (481 against
+// 522 us).
+constexpr int64_t kStreamBytes = int64_t(256) << 20;
 
 inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
