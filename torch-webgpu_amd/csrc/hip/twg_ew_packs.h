@@ -19,14 +19,17 @@ constexpr int kThreads = 256;  // 4 wavefronts of 64
 #define TWG_ROWS_UNROLL 1
 #endif
 
-// An op that moves more than this in total is treated as streaming (bigger than the 256 MB
-// last-level cache, every byte touched once): loads and stores carry the nontemporal hint, which
-// keeps them out of that cache.  Smaller ops keep default caching so that the op that consumes
-// the result finds it there: a chain of five dependent elementwise ops on 64 MiB tensors runs in
-// 119 us against 127 us with the hint, on 128 MiB tensors (its unary ops just fit) in 228 us
-// against 244 us; from 256 MiB tensors on nothing fits and the hint is worth 8% (481 against
-// 522 us).
-constexpr int64_t kStreamBytes = int64_t(256) << 20;
+// An op that moves more than this in total is treated as streaming: loads and stores carry the
+// nontemporal hint, which keeps them out of the 256 MB last-level cache.  Smaller ops keep
+// default caching so that the op that consumes the result can find it there.  The threshold is
+// a trade between the two ways an op meets its operands (microseconds, 32 / 64 / 128 MiB
+// tensors): with 64 MiB, a chain of five dependent ops takes 64 / 127 / 244 and a single add on
+// operands not touched lately 17 / 32 / 61; with 256 MiB (everything that fits the cache stays
+// cacheable) the chain takes 65 / 119 / 228 but the cold add 19 / 36 / 60 and a cold gelu
+// 13 / 23 / 45 instead of 13 / 22 / 41; with 32 MiB the chain takes 69 / 128.  The hint costs a
+// chain 6-7% where its intermediates would have fitted, default caching costs cold operands
+// 7-16%.
+constexpr int64_t kStreamBytes = int64_t(64) << 20;
 
 inline bool aligned_to(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
