@@ -148,16 +148,17 @@ def test_copy_sizes_around_every_staging_boundary(twg):
 
 
 def test_uploads_through_the_outbox(twg):
-    # Uploads of 1 KiB..64 KiB are copied into a pinned slot and fetched by a kernel that then
-    # releases the slot: every size class and destination alignment, many more uploads in a row
+    # Uploads of 1 KiB..2 MiB are copied into pinned slots (up to 16 at a time) and fetched by a
+    # kernel, one workgroup per slot, that then releases them: every size class and destination alignment, many more uploads in a row
     # than there are slots (each to its own place, checked at the end), and uploads queued
     # behind a long kernel, so that the host has to wait for a slot.
     L = twg.load()
     g = torch.Generator().manual_seed(123)
-    raw = torch.randint(0, 256, (1 << 20,), dtype=torch.uint8, generator=g)
-    dev = twg.DeviceBuffer((1 << 20) + 64)
-    back = torch.empty((1 << 20) + 64, dtype=torch.uint8)
-    for nb in (1025, 1040, 2048, 4096, 4099, 16384, 40000, 65535, 65536, 65537):
+    raw = torch.randint(0, 256, ((1 << 21) + 64,), dtype=torch.uint8, generator=g)
+    dev = twg.DeviceBuffer((1 << 21) + 128)
+    back = torch.empty((1 << 21) + 128, dtype=torch.uint8)
+    for nb in (1025, 1040, 2048, 4096, 4099, 16384, 40000, 65535, 65536, 65537, 100000, 262143, 262144, 262145,
+               300001, 524288, 786433, (1 << 20) - 1, 1 << 20, (1 << 20) + 16385, (1 << 21) - 3, 1 << 21, (1 << 21) + 1):
         for dst_off in (0, 4, 16, 3):
             twg.check(L.twg_fill_bytes(dev.ptr, 0xEE, nb + 64, None))
             twg.check(L.twg_memcpy_h2d(dev.ptr + dst_off, raw.data_ptr() + 5, nb, None))
@@ -173,6 +174,18 @@ def test_uploads_through_the_outbox(twg):
         scratch.fill_(0)
     twg.check(L.twg_memcpy_d2h(back.data_ptr(), dev.ptr, 100 * piece, None))
     assert torch.equal(back[:100 * piece], raw[:100 * piece])
+    # small and large uploads interleaved, so that groups of four start at either half
+    sizes = [3000, 200000, 70000, 5000, 5000, 262144, 1500, 400000, 65536, 131073]
+    offs, pos = [], 0
+    for nb in sizes:
+        offs.append(pos)
+        pos += (nb + 63) // 64 * 64
+    for rep in range(3):
+        for nb, o in zip(sizes, offs):
+            twg.check(L.twg_memcpy_h2d(dev.ptr + o, raw.data_ptr() + o + rep, nb, None))
+        twg.check(L.twg_memcpy_d2h(back.data_ptr(), dev.ptr, pos, None))
+        for nb, o in zip(sizes, offs):
+            assert torch.equal(back[o:o + nb], raw[o + rep:o + rep + nb]), (rep, nb)
     # the same behind a kernel that keeps the stream busy for a while
     n = 1 << 27
     big_a, big_o = twg.DeviceBuffer(4 * n), twg.DeviceBuffer(4 * n)
