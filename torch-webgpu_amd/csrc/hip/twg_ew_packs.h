@@ -15,10 +15,6 @@ namespace {
 
 constexpr int kThreads = 256;  // 4 wavefronts of 64
 
-#ifndef TWG_ROWS_UNROLL
-#define TWG_ROWS_UNROLL 1
-#endif
-
 // An op that moves more than this in total is treated as streaming: loads and stores carry the
 // nontemporal hint, which keeps them out of the 256 MB last-level cache.  Smaller ops keep
 // default caching so that the op that consumes the result can find it there.  The threshold is

@@ -391,7 +391,7 @@ int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipSt
     TWG_LAUNCH_ROWS(4, 1);
     return (int)hipGetLastError();
   }
-  constexpr int U = TWG_ROWS_UNROLL;
+  constexpr int U = 1;  // packs per lane where an input is streamed (2 and 4 were slower)
   const unsigned grid = grid_for(U);
   if (grid == 0) return TWG_E_UNSUPPORTED;
   if (!stream)
