@@ -470,6 +470,52 @@ def _random_view(g, shape, rng):
     return t[tuple(slice(None, None, steps[d]) for d in range(nd))]
 
 
+def test_random_strips_and_ragged_rows(twg):
+    # Seeded shapes aimed at two launch paths whose index arithmetic depends on the extents:
+    # an operand stored [.., x, c] with 2..31 channels against a [.., c, x] output (strips
+    # through LDS: one strip per block, several strips of short rows per block, last strips that
+    # are shorter, channel counts that do and do not divide the LDS pitch), and rows whose
+    # starts fall anywhere into the output's 128-byte lines (chunks cut at those lines).
+    import random
+    rng = random.Random(4321)
+    g = torch.Generator().manual_seed(99)
+    for case in range(48):
+        c = rng.choice((2, 3, 4, 5, 7, 8, 12, 16, 17, 24, 31))
+        x = rng.choice((32, 40, 96, 100, 224, 256, 260, 513, 1024, 1500, 4099))
+        outer = rng.choice(((2,), (3,), (2, 3), (5, 2)))
+        while torch.Size(outer).numel() * c * x > (1 << 19):
+            x = max(32, x // 2)
+        off = rng.choice((0, 0, 1, 4))
+        stored = torch.randn(off + torch.Size(outer).numel() * x * c, generator=g)[off:].view(*outer, x, c)
+        a = stored.transpose(-1, -2)                     # logical [.., c, x], unit stride along c
+        b = torch.randn(*outer, c, x, generator=g)
+        _say(f"strip case {case}: {tuple(a.shape)} stored {tuple(stored.shape)} offset {off}")
+        assert bit_equal(H.add(a, b, alpha=0.5), oracle.add(a, b, alpha=0.5))
+        assert bit_equal(H.add(b, a), oracle.add(b, a))
+        stored2 = torch.randn(*outer, x, c, generator=g)
+        assert bit_equal(H.add(a, stored2.transpose(-1, -2)), oracle.add(a, stored2.transpose(-1, -2)))
+    for case in range(32):
+        rows = rng.choice((3, 17, 64, 200))
+        # three chunks and more; from 8192 elements on the row kernel takes them, below that the pack walk
+        length = 4 * rng.choice((193, 250, 251, 300, 511, 1000, 2047, 2050, 2051, 2251, 3073))
+        lead = rng.choice((0, 4, 8, 20, 28))                                    # row 0 starts here
+        pitch = length + 4 * rng.choice((0, 1, 2, 3, 5, 8))
+        big_o = torch.zeros(lead + rows * pitch)
+        out = big_o[lead:].as_strided((rows, length), (pitch, 1))
+        big_a = torch.randn(lead + rows * pitch, generator=g)
+        a = big_a[lead:].as_strided((rows, length), (pitch, 1))
+        colv = torch.randn(rows, 1, generator=g)
+        full = torch.randn(rows, length, generator=g)
+        _say(f"ragged rows {case}: {rows} x {length}, pitch {pitch}, lead {lead}")
+        assert bit_equal(H.add(a, colv, out=out), oracle.add(a, colv))
+        assert bool((big_o[:lead] == 0).all())
+        if pitch > length:
+            gaps = big_o[lead:].as_strided((rows - 1, pitch - length), (pitch, 1), length)
+            assert bool((gaps == 0).all()), "wrote between the rows"
+        assert bit_equal(H.add(full, colv), oracle.add(full, colv))
+        assert bit_equal(H.add(a, full), oracle.add(a, full))
+
+
 def test_random_geometries(twg):
     # 120 seeded layouts: every dispatch path of the elementwise launcher (contiguous,
     # rows with broadcast operands, LDS tiles, 128-bit tiles, div/mod) and the strided
