@@ -449,9 +449,11 @@ __global__ __launch_bounds__(kMailboxLanes) void mailbox_kernel(uint8_t *box, co
 // against 18 us.  One workgroup pushes ~8 GB/s over the link, eight ~31 GB/s; more of them
 // finish their pieces too far out of order for the host to overlap (32: 26 GB/s).  From
 // 16 MiB on the DMA path with its helper threads is faster.
-constexpr uint32_t kFlowPiece = 65536;
+constexpr uint32_t kFlowPieceLarge = 65536;
+constexpr uint32_t kFlowPieceSmall = 16384;          // up to kFlowSmallBytes: more workgroups at work
+constexpr size_t kFlowSmallBytes = size_t(512) << 10;
 constexpr size_t kFlowMaxBytes = size_t(8) << 20;
-constexpr uint32_t kFlowMaxPieces = (uint32_t)(kFlowMaxBytes / kFlowPiece);
+constexpr uint32_t kFlowMaxPieces = (uint32_t)(kFlowMaxBytes / kFlowPieceLarge);
 constexpr int kFlowBlocks = 8;
 constexpr int kFlowLanes = 1024;
 static_assert(kFlowMaxPieces * sizeof(uint32_t) <= kFlowFlagBytes, "one flag per piece");
@@ -467,7 +469,7 @@ __device__ __forceinline__ uint32_t flow_copy(uint8_t *dst, const uint8_t *src, 
 
 __global__ __launch_bounds__(kFlowLanes) void d2h_flow_kernel(uint8_t *ring, const uint8_t *src,
                                                                size_t n, uint32_t *flags,
-                                                               uint32_t seq) {
+                                                               uint32_t seq, uint32_t kFlowPiece) {
   const uint32_t t = threadIdx.x;
   const uint32_t npieces = (uint32_t)((n + kFlowPiece - 1) / kFlowPiece);
   const uint32_t align = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);  // pieces keep it
@@ -867,11 +869,12 @@ int twg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, twg_strea
   if ((rc = staging_drain_locked(st))) return rc;  // uploads may still read the ring's slots
   if (nbytes <= kFlowMaxBytes && nbytes <= st.ring_bytes) {
     const uint32_t seq = ++st.flow_seq;
+    const uint32_t kFlowPiece = nbytes <= kFlowSmallBytes ? kFlowPieceSmall : kFlowPieceLarge;
     const uint32_t npieces = (uint32_t)((nbytes + kFlowPiece - 1) / kFlowPiece);
     const int blocks = npieces < (uint32_t)kFlowBlocks ? (int)npieces : kFlowBlocks;
     d2h_flow_kernel<<<blocks, kFlowLanes, 0, s>>>(static_cast<uint8_t *>(st.base_dev),
                                                   reinterpret_cast<const uint8_t *>(src), nbytes,
-                                                  static_cast<uint32_t *>(st.flow_flags_dev), seq);
+                                                  static_cast<uint32_t *>(st.flow_flags_dev), seq, kFlowPiece);
     TWG_HIP_TRY(hipGetLastError());
     bool synced = false;
     for (uint32_t p = 0; p < npieces; ++p) {
