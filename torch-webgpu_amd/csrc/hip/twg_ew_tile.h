@@ -655,7 +655,9 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       // A transposed extent of 33..64 elements is one 64-wide tile: with 256 x 32 tiles each
       // 256-byte row of the transposed operand was fetched half by one workgroup, half by
       // another (`[64,128,64,64]` stored with dimension 0 innermost: 67-73% -> 71-78% of peak).
-      const bool one_t_tile = wide && tg.nt > 32 && tg.nt <= 64;
+      // From 2^27 elements on the 1024-lane 256 x 32 tiles win again (`[64,256,128,128]` reversed:
+      // 74.6% against 67.4%).
+      const bool one_t_tile = wide && tg.nt > 32 && tg.nt <= 64 && g.numel < (int64_t(1) << 27);
       if (!set_tiles(one_t_tile ? 64 : wide ? 256 : mid ? 128 : 64, (wide && !one_t_tile) ? 32 : 64, &grid))
         return TWG_E_UNSUPPORTED;
       // 256x32 tiles: 512 lanes per tile measured 2-4 points ahead of 256 from 2^22 to 2^26
