@@ -336,6 +336,14 @@ def test_add_transposed_operand(twg, rows, cols):
     ((4, 4, 1027), (0, 2, 1)), ((2, 16, 700), (0, 2, 1)), ((2, 32, 301), (0, 2, 1)),
     ((2, 33, 300), (0, 2, 1)), ((7, 2, 5000), (0, 2, 1)), ((3, 5, 255), (0, 2, 1)),
     ((2, 8, 3001), (0, 2, 1)), ((3, 16, 1100), (0, 2, 1)), ((2, 24, 777), (0, 2, 1)),
+    # the mirror image: the output [.., x, c] with a short c, the operand stored planar [.., c, x]
+    # (NCHW -> NHWC with few channels): strips interleaved through LDS
+    ((4, 30, 40, 3), (0, 3, 1, 2)), ((2, 1000, 3), (0, 2, 1)), ((1027, 4), (1, 0)), ((3, 700, 16), (0, 2, 1)),
+    ((2, 301, 31), (0, 2, 1)), ((5000, 2), (1, 0)), ((3, 2051, 7), (0, 2, 1)), ((2, 4099, 24), (0, 2, 1)),
+    ((2, 3, 255, 5), (0, 1, 3, 2)), ((2, 2, 260, 8), (1, 0, 3, 2)), ((300, 32), (1, 0)),
+    # a short x: several strips per block (groups of the next dimension, the last group shorter)
+    ((7, 5, 40, 3), (0, 1, 3, 2)), ((3, 11, 100, 2), (0, 1, 3, 2)), ((2, 9, 33, 31), (0, 1, 3, 2)),
+    ((2, 23, 56, 3), (1, 0, 3, 2)), ((40, 112, 3), (0, 2, 1)), ((1, 3, 32, 4), (0, 1, 3, 2)),
     # the same with fewer than 256 elements per strip: several strips per block
     ((4, 3, 23, 100), (2, 0, 3, 1)), ((3, 5, 9, 33), (0, 2, 3, 1)), ((2, 2, 7, 250), (2, 0, 3, 1)),
     ((6, 3, 224), (0, 2, 1)), ((2, 31, 40), (0, 2, 1)), ((16, 3, 224, 96), (2, 0, 3, 1)),
@@ -474,7 +482,8 @@ def test_random_strips_and_ragged_rows(twg):
     # Seeded shapes aimed at two launch paths whose index arithmetic depends on the extents:
     # an operand stored [.., x, c] with 2..31 channels against a [.., c, x] output (strips
     # through LDS: one strip per block, several strips of short rows per block, last strips that
-    # are shorter, channel counts that do and do not divide the LDS pitch), and rows whose
+    # are shorter, channel counts that do and do not divide the LDS pitch), the mirror image of
+    # that (planar operand, [.., x, c] output), and rows whose
     # starts fall anywhere into the output's 128-byte lines (chunks cut at those lines).
     import random
     rng = random.Random(4321)
@@ -494,6 +503,13 @@ def test_random_strips_and_ragged_rows(twg):
         assert bit_equal(H.add(b, a), oracle.add(b, a))
         stored2 = torch.randn(*outer, x, c, generator=g)
         assert bit_equal(H.add(a, stored2.transpose(-1, -2)), oracle.add(a, stored2.transpose(-1, -2)))
+        # the mirror image: output [.., x, c], operand stored planar [.., c, x]
+        planar = torch.randn(off + torch.Size(outer).numel() * x * c, generator=g)[off:].view(*outer, c, x)
+        pa = planar.transpose(-1, -2)                    # logical [.., x, c], unit stride along x
+        assert bit_equal(H.add(pa, stored2, alpha=0.25), oracle.add(pa, stored2, alpha=0.25))
+        assert bit_equal(H.add(stored2, pa), oracle.add(stored2, pa))
+        assert bit_equal(H.add(pa, b.transpose(-1, -2)), oracle.add(pa, b.transpose(-1, -2)))
+        assert bit_equal(H.unary("twg_unary_f32", pa, pre=(ctypes.c_int(1),)), torch.relu(pa))
     for case in range(32):
         rows = rng.choice((3, 17, 64, 200))
         # three chunks and more; from 8192 elements on the row kernel takes them, below that the pack walk

@@ -107,6 +107,14 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
       const int r = try_deint();
       if (r != TWG_E_UNSUPPORTED) return r;
     }
+    // The mirror image: the output stored [.., x, c] with a short c and an input stored planar.
+    if (g.ndim >= 2 && g.shape[0] < 32 && g.stride[0][0] == 1) {
+      const bool a_p = g.stride[1][0] != 1, b_p = NIN == 2 && g.stride[2][0] != 1;
+      if (a_p || b_p) {
+        const int r = launch_inter<NIN, Op, TO, TA, TB>(out, a, b, g, a_p, b_p, op, s);
+        if (r != TWG_E_UNSUPPORTED) return r;
+      }
+    }
     // (i-c) rows too short or too ragged for one block per 256-element row chunk: if the
     // output and one input are dense, walk them flat and gather the other input
     if constexpr (NIN == 2) {
@@ -175,7 +183,7 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
       // across dimensions 0 and 1 (and t is a later one): the two are walked as one, so that
       // a tile covers 256 consecutive output elements however short the rows are, and
       // consecutive workgroups write consecutive memory across the rows
-      if (g.ndim >= 3 && g.shape[0] >= 4 && g.shape[0] * g.shape[1] >= 128) {
+      if (g.ndim >= 3 && g.shape[0] >= 2 && g.shape[0] * g.shape[1] >= 128) {
         int t = -1;
         for (int d = 2; d < g.ndim && t < 0; ++d) {
           if (g.shape[d] < 16) continue;

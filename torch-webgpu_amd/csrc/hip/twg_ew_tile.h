@@ -781,5 +781,232 @@ int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool 
 }
 
 
+// ------------------------------------------------------------ ew_inter
+// The mirror of ew_deint: the OUTPUT is laid out [.., x, c] with a short innermost extent c
+// (dimension 0, 2..31 elements; x is dimension 1, output stride c) and an input is stored
+// planar, [.., c, x] (unit stride along x): NCHW -> NHWC with a few channels, coordinate arrays
+// stacked into points.  A block takes a strip of TX values of x: it reads the planar operands'
+// c runs of TX elements with 16-byte loads straight into LDS (one run per channel, the pitch
+// of ew_deint), then walks the strip as it lies in the output, TX * c consecutive elements in
+// 16-byte packs, picking each pack's four values out of LDS.  Inputs laid out like the output
+// are read in the same packs.  (One element per lane, which these layouts took before, ran at
+// 40% of HBM peak for c = 3, 4, 8.)
+struct InterShape {
+  uint32_t tx_elems;   // values of x per strip
+  uint32_t rows;       // strips per block (consecutive indices of the first batch dimension)
+  uint32_t lds_words;  // words of LDS per planar operand
+  SmallDiv by_p;       // the channel count
+  SmallDiv by_packs;   // packs of a full strip's run per channel
+  SmallDiv by_run_packs;    // by_packs.d * P: packs of all the runs of a strip
+  SmallDiv by_strip_packs;  // packs of a full strip as it lies in the output
+};
+
+template <int NIN, bool A_P, bool B_P, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_inter(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                     InterShape sh, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char inter_lds[];
+  TA *sa = reinterpret_cast<TA *>(inter_lds);
+  TB *sb = reinterpret_cast<TB *>(inter_lds) + (A_P ? sh.lds_words : 0u);
+
+  // g.n0 / g.s0: extent and strides of x; g.nt / g.st: of c; tiles0 strips along x
+  const uint32_t rows = sh.rows;
+  uint32_t rem = blockIdx.x / g.tiles0;
+  const uint32_t t0i = blockIdx.x - rem * g.tiles0;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  // rows > 1 (x is short, one strip covers it): the block takes `rows` consecutive indices of
+  // the first batch dimension, one strip each; g.tilest counts those groups
+  uint32_t nrows = 1;
+  int d_first = 0;
+  if (rows > 1) {
+    const uint32_t q = rem / g.tilest;
+    const int64_t row0 = (int64_t)(rem - q * g.tilest) * rows;
+    rem = q;
+    nrows = (uint32_t)(g.bshape[0] - row0 < (int64_t)rows ? g.bshape[0] - row0 : (int64_t)rows);
+    off_o = row0 * g.bstride[0][0];
+    off_a = row0 * g.bstride[1][0];
+    if constexpr (NIN == 2) off_b = row0 * g.bstride[2][0];
+    d_first = 1;
+  }
+  for (int d = d_first; d < g.nbatch; ++d) {
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = rem / extent;  // batch indices fit 32 bits, the grid does
+    const int64_t i = rem - q * extent;
+    rem = q;
+    off_o += i * g.bstride[0][d];
+    off_a += i * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += i * g.bstride[2][d];
+  }
+  const uint32_t P = (uint32_t)g.nt;
+  const int64_t x0 = (int64_t)t0i * sh.tx_elems;
+  const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)sh.tx_elems ? g.n0 - x0 : (int64_t)sh.tx_elems);
+  const uint32_t xpitch = deint_pitch(nx);  // words between the runs of two channels in LDS
+  constexpr uint32_t kU = 2;                // loads issued before the first of them is used
+  // (the divisors were made for strips of full length; with rows > 1 every strip is one)
+  const bool full = (int64_t)nx == (g.n0 < (int64_t)sh.tx_elems ? g.n0 : (int64_t)sh.tx_elems);
+
+  // the planar operands' runs, as they lie in memory: lane -> (strip, channel, pack of the run)
+  const uint32_t packs = (nx + 3) / 4;
+  const uint32_t run_packs = packs * P;
+  auto park = [&](auto *lds, const auto *src, int64_t c_stride, int64_t row_stride) {
+    using T = std::remove_cv_t<std::remove_pointer_t<decltype(src)>>;
+    using P4 = Pack<T, 4>;
+    const uint32_t total = nrows * run_packs;
+    for (uint32_t i0 = threadIdx.x; i0 < total; i0 += kThreads * kU) {
+      P4 v[kU];
+      uint32_t at[kU];
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * kThreads;
+        const uint32_t row = rows > 1 ? div_by(i, sh.by_run_packs) : 0u;
+        const uint32_t k = i - row * run_packs;
+        const uint32_t c = full ? div_by(k, sh.by_packs) : k / packs;
+        const uint32_t x = 4 * (k - c * packs);
+        at[u] = (row * P + c) * xpitch + x;
+        if (i < total) v[u] = load4_edge(src + row * row_stride + (int64_t)c * c_stride + x, (int64_t)nx - x);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * kThreads;
+        if (i < total) *reinterpret_cast<P4 *>(lds + at[u]) = v[u];
+      }
+    }
+  };
+  if constexpr (A_P) park(sa, a + off_a + x0 * g.s0[1], g.st[1], g.bstride[1][0]);
+  if constexpr (NIN == 2 && B_P) park(sb, b + off_b + x0 * g.s0[2], g.st[2], g.bstride[2][0]);
+  __syncthreads();
+
+  // each strip as it lies in the output: nx * P consecutive elements, in packs
+  const uint32_t strip = nx * P;
+  const uint32_t strip_packs = (strip + 3) / 4;
+  const uint32_t total = nrows * strip_packs;
+  for (uint32_t q0 = threadIdx.x; q0 < total; q0 += kThreads * kU) {
+    PA va[kU];
+    PB vb[kU];
+    uint32_t row[kU], j[kU];
+#pragma unroll
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t q = q0 + u * kThreads;
+      row[u] = rows > 1 ? div_by(q, sh.by_strip_packs) : 0u;
+      j[u] = 4 * (q - row[u] * strip_packs);
+      if (q < total) {
+        if constexpr (!A_P)
+          va[u] = load4_edge(a + off_a + row[u] * g.bstride[1][0] + x0 * (int64_t)P + j[u], (int64_t)strip - j[u]);
+        if constexpr (NIN == 2 && !B_P)
+          vb[u] = load4_edge(b + off_b + row[u] * g.bstride[2][0] + x0 * (int64_t)P + j[u], (int64_t)strip - j[u]);
+      }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t q = q0 + u * kThreads;
+      if (q >= total) continue;
+      const uint32_t left = strip - j[u];
+      uint32_t x = div_by(j[u], sh.by_p), c = j[u] - x * P;
+      const uint32_t base = row[u] * P * xpitch;
+#pragma unroll
+      for (uint32_t m = 0; m < 4; ++m) {
+        if (m < left) {
+          if constexpr (A_P) va[u].v[m] = sa[base + c * xpitch + x];
+          if constexpr (NIN == 2 && B_P) vb[u].v[m] = sb[base + c * xpitch + x];
+        }
+        if (++c == P) {
+          c = 0;
+          ++x;
+        }
+      }
+      PO o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va[u].v[k], NIN == 2 ? vb[u].v[k] : TB());
+      TO *dst = out + off_o + row[u] * g.bstride[0][0] + x0 * (int64_t)P + j[u];
+      if (left >= 4) {
+        store4_any(dst, o);
+      } else {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k)
+          if (k < left) dst[k] = o.v[k];
+      }
+    }
+  }
+}
+
+// Dimension 0 is the short extent c, dimension 1 is x with output stride c; *_p marks the inputs
+// stored planar (unit stride along x), the others lie like the output.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_inter(TO *out, const TA *a, const TB *b, const Geom &g, bool a_p, bool b_p, Op op,
+                 hipStream_t s) {
+  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    if (g.ndim < 2) return TWG_E_UNSUPPORTED;
+    const int64_t P = g.shape[0];
+    if (P < 2 || P >= 32 || g.stride[0][0] != 1 || g.stride[0][1] != P) return TWG_E_UNSUPPORTED;
+    auto like_out = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == P; };
+    auto planar = [&](int o) { return g.stride[o][1] == 1 && g.stride[o][0] != 0; };
+    if (a_p ? !planar(1) : !like_out(1)) return TWG_E_UNSUPPORTED;
+    if (NIN == 2 && (b_p ? !planar(2) : !like_out(2))) return TWG_E_UNSUPPORTED;
+    TileGeom tg{};
+    tg.n0 = g.shape[1];
+    tg.nt = P;
+    for (int o = 0; o < 3; ++o) {
+      tg.s0[o] = g.stride[o][1];
+      tg.st[o] = g.stride[o][0];
+    }
+    int64_t batch = 1;
+    for (int d = 2; d < g.ndim; ++d) {
+      tg.bshape[tg.nbatch] = g.shape[d];
+      for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+      tg.nbatch++;
+      batch *= g.shape[d];
+    }
+    // strip length: as in ew_deint, what keeps 8 blocks on a CU
+    uint32_t tx = 1024;
+    while ((int64_t)P * deint_pitch(tx) > kDeintLds) tx /= 2;
+    const int64_t tiles0 = (tg.n0 + tx - 1) / tx;
+    // a short x (one strip, a fraction of a block's lanes): a block takes several indices of
+    // the first batch dimension, as many strips as fit the LDS array and add up to about 2048
+    // elements
+    uint32_t rows = 1;
+    int64_t row_tiles = 1;
+    if (tg.n0 <= (int64_t)tx && tg.n0 * P < 1024 && tg.nbatch >= 1) {
+      const int64_t per_strip = P * (int64_t)deint_pitch((uint32_t)tg.n0);
+      int64_t fit = kDeintLds / per_strip, want = (2048 + tg.n0 * P - 1) / (tg.n0 * P);
+      int64_t k = fit < want ? fit : want;
+      if (k > tg.bshape[0]) k = tg.bshape[0];
+      if (k >= 2) {
+        rows = (uint32_t)k;
+        row_tiles = (tg.bshape[0] + k - 1) / k;
+        batch = batch / tg.bshape[0] * row_tiles;
+      }
+    }
+    // (too little per run or per block to beat the gather)
+    if (tg.n0 < 32 || (tg.n0 * P < 512 && rows < 2)) return TWG_E_UNSUPPORTED;
+    if (tiles0 > INT32_MAX || batch > INT32_MAX || tiles0 * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+    tg.tiles0 = (uint32_t)tiles0;
+    tg.tilest = (uint32_t)row_tiles;
+    const unsigned grid = (unsigned)(tiles0 * batch);
+    const uint32_t nx_full = (uint32_t)(tg.n0 < (int64_t)tx ? tg.n0 : (int64_t)tx);
+    const uint32_t packs_full = (nx_full + 3) / 4;
+    const uint32_t words = rows * (uint32_t)P * deint_pitch(nx_full);
+    const InterShape sh{tx, rows, words, small_div((uint32_t)P), small_div(packs_full),
+                        small_div(packs_full * (uint32_t)P), small_div((nx_full * (uint32_t)P + 3) / 4)};
+    const size_t lds_bytes = (size_t)words * 4 * ((a_p ? 1 : 0) + (NIN == 2 && b_p ? 1 : 0));
+#define TWG_INTER(AP, BP) \
+  ew_inter<NIN, AP, BP, Op, TO, TA, TB><<<grid, kThreads, lds_bytes, s>>>(out, a, b, tg, sh, op)
+    if (a_p && b_p) {
+      if constexpr (NIN == 2) TWG_INTER(true, true);
+    } else if (a_p) {
+      TWG_INTER(true, false);
+    } else {
+      if constexpr (NIN == 2) TWG_INTER(false, true);
+    }
+#undef TWG_INTER
+    return (int)hipGetLastError();
+  }
+}
+
 }  // namespace
 }  // namespace twg
