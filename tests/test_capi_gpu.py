@@ -344,6 +344,13 @@ def test_add_transposed_operand(twg, rows, cols):
     # a short x: several strips per block (groups of the next dimension, the last group shorter)
     ((7, 5, 40, 3), (0, 1, 3, 2)), ((3, 11, 100, 2), (0, 1, 3, 2)), ((2, 9, 33, 31), (0, 1, 3, 2)),
     ((2, 23, 56, 3), (1, 0, 3, 2)), ((40, 112, 3), (0, 2, 1)), ((1, 3, 32, 4), (0, 1, 3, 2)),
+    # channels-last pixels with two outer dimensions swapped: tiles of pixels through LDS (full
+    # and ragged tiles, channel counts that do and do not divide a pack, the transposed
+    # dimension next to x or further out)
+    ((4, 30, 40, 3), (0, 2, 1, 3)), ((5, 33, 35, 4), (0, 2, 1, 3)), ((37, 9, 45, 2), (2, 1, 0, 3)),
+    ((3, 70, 65, 7), (0, 2, 1, 3)), ((2, 19, 23, 16), (0, 2, 1, 3)), ((2, 40, 17, 31), (0, 2, 1, 3)),
+    ((12, 13, 14, 5), (1, 2, 0, 3)), ((9, 8, 8, 24), (2, 0, 1, 3)), ((64, 65, 3), (1, 0, 2)),
+    ((2, 3, 32, 64, 8), (0, 1, 3, 2, 4)), ((2, 100, 8, 3), (0, 2, 1, 3)),
     # the same with fewer than 256 elements per strip: several strips per block
     ((4, 3, 23, 100), (2, 0, 3, 1)), ((3, 5, 9, 33), (0, 2, 3, 1)), ((2, 2, 7, 250), (2, 0, 3, 1)),
     ((6, 3, 224), (0, 2, 1)), ((2, 31, 40), (0, 2, 1)), ((16, 3, 224, 96), (2, 0, 3, 1)),

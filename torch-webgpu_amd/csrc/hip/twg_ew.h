@@ -115,6 +115,23 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
         if (r != TWG_E_UNSUPPORTED) return r;
       }
     }
+    // Channels-last pixels (2..31 channels, unit stride in every operand) with two outer
+    // dimensions swapped between the output and an input: tiles of pixels through LDS.
+    if (g.ndim >= 3 && g.shape[0] >= 2 && g.shape[0] < 32 && g.stride[0][0] == 1 &&
+        g.stride[0][1] == g.shape[0] && g.stride[1][0] == 1 && (NIN == 1 || g.stride[2][0] == 1)) {
+      const int64_t C = g.shape[0];
+      auto y_of = [&](int o) {
+        if (g.stride[o][1] == C) return 0;  // stored like the output
+        for (int d = 2; d < g.ndim; ++d)
+          if (g.stride[o][d] == C) return d;
+        return -1;
+      };
+      const int ta = y_of(1), tb = NIN == 2 ? y_of(2) : 0;
+      if (ta >= 0 && tb >= 0 && (ta > 0 || tb > 0) && (ta == 0 || tb == 0 || ta == tb)) {
+        const int r = launch_pix<NIN, Op, TO, TA, TB>(out, a, b, g, ta > 0 ? ta : tb, ta > 0, tb > 0, op, s);
+        if (r != TWG_E_UNSUPPORTED) return r;
+      }
+    }
     // (i-c) rows too short or too ragged for one block per 256-element row chunk: if the
     // output and one input are dense, walk them flat and gather the other input
     if constexpr (NIN == 2) {

@@ -1008,5 +1008,199 @@ int launch_inter(TO *out, const TA *a, const TB *b, const Geom &g, bool a_p, boo
   }
 }
 
+// Transposes of pixels.  Every operand keeps a short innermost extent c (2..31 elements, unit
+// stride: the channels of a channels-last image), the output is stored [.., y, x, c] and an
+// input [.., x, y, c]: no operand has runs longer than c elements in the other's order.  A
+// block takes a tile of t0 x tt pixels: it parks the transposed input's runs (tt * c
+// consecutive elements for each x) in LDS as they lie in memory, then writes the output's runs
+// (t0 * c consecutive elements for each y) in 16-byte packs, gathering from LDS.
+struct PixShape {
+  uint32_t t0, tt;        // pixels of a tile along x and along y
+  uint32_t pitch;         // words of LDS between two x
+  uint32_t lds_words;     // words of LDS per transposed operand
+  SmallDiv by_c;          // the channel count
+  SmallDiv by_in_packs;   // packs of a full tile's input run
+  SmallDiv by_out_packs;  // packs of a full tile's output run
+};
+
+template <int NIN, bool A_T, bool B_T, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(kThreads) void ew_pix(TO *out, const TA *a, const TB *b, TileGeom g,
+                                                   PixShape sh, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char pix_lds[];
+  TA *sa = reinterpret_cast<TA *>(pix_lds);
+  TB *sb = reinterpret_cast<TB *>(pix_lds) + (A_T ? sh.lds_words : 0u);
+
+  // g.n0 / g.s0: extent and strides of x; g.nt / g.st: of y.  Tiles along x are dealt first
+  // (they are neighbours in the output's memory), then those along y, then the batch.
+  uint32_t rem = blockIdx.x / g.tiles0;
+  const uint32_t t0i = blockIdx.x - rem * g.tiles0;
+  const uint32_t tti = rem % g.tilest;
+  rem /= g.tilest;
+  int64_t off_o = 0, off_a = 0, off_b = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = rem / extent;  // batch indices fit 32 bits, the grid does
+    const int64_t i = rem - q * extent;
+    rem = q;
+    off_o += i * g.bstride[0][d];
+    off_a += i * g.bstride[1][d];
+    if constexpr (NIN == 2) off_b += i * g.bstride[2][d];
+  }
+  const uint32_t C = sh.by_c.d;
+  const int64_t x0 = (int64_t)t0i * sh.t0, y0 = (int64_t)tti * sh.tt;
+  const uint32_t nx = (uint32_t)(g.n0 - x0 < (int64_t)sh.t0 ? g.n0 - x0 : (int64_t)sh.t0);
+  const uint32_t ny = (uint32_t)(g.nt - y0 < (int64_t)sh.tt ? g.nt - y0 : (int64_t)sh.tt);
+  const bool full = nx == sh.t0 && ny == sh.tt;  // the divisors were made for full tiles
+  constexpr uint32_t kU = 2;                     // loads issued before the first of them is used
+
+  // the transposed operands' runs, as they lie in memory: lane -> (x, pack of the run)
+  const uint32_t in_run = ny * C, in_packs = (in_run + 3) / 4;
+  auto park = [&](auto *lds, const auto *src, int64_t x_stride) {
+    using T = std::remove_cv_t<std::remove_pointer_t<decltype(src)>>;
+    using P4 = Pack<T, 4>;
+    const uint32_t total = nx * in_packs;
+    for (uint32_t i0 = threadIdx.x; i0 < total; i0 += kThreads * kU) {
+      P4 v[kU];
+      uint32_t at[kU];
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * kThreads;
+        const uint32_t x = full ? div_by(i, sh.by_in_packs) : i / in_packs;
+        const uint32_t k = 4 * (i - x * in_packs);
+        at[u] = x * sh.pitch + k;
+        if (i < total) v[u] = load4_edge(src + (int64_t)x * x_stride + k, (int64_t)in_run - k);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kU; ++u) {
+        const uint32_t i = i0 + u * kThreads;
+        if (i < total) *reinterpret_cast<P4 *>(lds + at[u]) = v[u];
+      }
+    }
+  };
+  if constexpr (A_T) park(sa, a + off_a + x0 * g.s0[1] + y0 * (int64_t)C, g.s0[1]);
+  if constexpr (NIN == 2 && B_T) park(sb, b + off_b + x0 * g.s0[2] + y0 * (int64_t)C, g.s0[2]);
+  __syncthreads();
+
+  // the output's runs: lane -> (y, pack of the run)
+  const uint32_t out_run = nx * C, out_packs = (out_run + 3) / 4;
+  const uint32_t total = ny * out_packs;
+  for (uint32_t q0 = threadIdx.x; q0 < total; q0 += kThreads * kU) {
+    PA va[kU];
+    PB vb[kU];
+    uint32_t y[kU], j[kU];
+#pragma unroll
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t q = q0 + u * kThreads;
+      y[u] = full ? div_by(q, sh.by_out_packs) : q / out_packs;
+      j[u] = 4 * (q - y[u] * out_packs);
+      if (q < total) {
+        if constexpr (!A_T)
+          va[u] = load4_edge(a + off_a + (y0 + y[u]) * g.st[1] + x0 * (int64_t)C + j[u], (int64_t)out_run - j[u]);
+        if constexpr (NIN == 2 && !B_T)
+          vb[u] = load4_edge(b + off_b + (y0 + y[u]) * g.st[2] + x0 * (int64_t)C + j[u], (int64_t)out_run - j[u]);
+      }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kU; ++u) {
+      const uint32_t q = q0 + u * kThreads;
+      if (q >= total) continue;
+      const uint32_t left = out_run - j[u];
+      uint32_t x = div_by(j[u], sh.by_c), c = j[u] - x * C;
+      const uint32_t base = y[u] * C;
+#pragma unroll
+      for (uint32_t m = 0; m < 4; ++m) {
+        if (m < left) {
+          if constexpr (A_T) va[u].v[m] = sa[x * sh.pitch + base + c];
+          if constexpr (NIN == 2 && B_T) vb[u].v[m] = sb[x * sh.pitch + base + c];
+        }
+        if (++c == C) {
+          c = 0;
+          ++x;
+        }
+      }
+      PO o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        o.v[k] = apply<NIN, Op, TO, TA, TB>(op, va[u].v[k], NIN == 2 ? vb[u].v[k] : TB());
+      TO *dst = out + off_o + (y0 + y[u]) * g.st[0] + x0 * (int64_t)C + j[u];
+      if (left >= 4) {
+        store4_any(dst, o);
+      } else {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k)
+          if (k < left) dst[k] = o.v[k];
+      }
+    }
+  }
+}
+
+// Dimension 0 is the short extent c (unit stride in every operand), dimension 1 is x with output
+// stride c, dimension t is y, with stride c in the transposed inputs; *_t marks those.  The
+// other inputs are stored like the output along dimensions 0 and 1.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_pix(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
+               hipStream_t s) {
+  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    if (g.ndim < 3 || t < 2 || t >= g.ndim || !(a_t || b_t)) return TWG_E_UNSUPPORTED;
+    const int64_t C = g.shape[0];
+    if (C < 2 || C >= 32 || g.stride[0][0] != 1 || g.stride[0][1] != C) return TWG_E_UNSUPPORTED;
+    auto like_out = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == C; };
+    auto transposed = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][t] == C; };
+    if (a_t ? !transposed(1) : !like_out(1)) return TWG_E_UNSUPPORTED;
+    if (NIN == 2 && (b_t ? !transposed(2) : !like_out(2))) return TWG_E_UNSUPPORTED;
+    if (g.shape[1] < 8 || g.shape[t] < 8) return TWG_E_UNSUPPORTED;  // (runs too short to gain)
+    TileGeom tg{};
+    tg.n0 = g.shape[1];
+    tg.nt = g.shape[t];
+    for (int o = 0; o < 3; ++o) {
+      tg.s0[o] = g.stride[o][1];
+      tg.st[o] = g.stride[o][t];
+    }
+    int64_t batch = 1;
+    for (int d = 2; d < g.ndim; ++d) {
+      if (d == t) continue;
+      tg.bshape[tg.nbatch] = g.shape[d];
+      for (int o = 0; o < 3; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+      tg.nbatch++;
+      batch *= g.shape[d];
+    }
+    // runs of about 128 elements either way, one to three thousand elements per block (3
+    // channels: 32 x 32 pixels 71% of peak, 64 x 32 or 16 x 16 57-61%, 8 x 8 24%; 8 channels:
+    // 16 x 16 75%, 32 x 32 67%; 16 channels: 8 x 8 or 16 x 8 71%, 32 x 32 48%)
+    uint32_t t0 = C <= 4 ? 32 : C <= 8 ? 16 : 8, tt = t0;
+    if (t0 * tt * C > 3072) tt /= 2;
+    if (t0 * tt * C < 1024) t0 *= 2;
+    const uint32_t pitch = deint_pitch(tt * (uint32_t)C);
+    const int64_t tiles0 = (tg.n0 + t0 - 1) / t0, tilest = (tg.nt + tt - 1) / tt;
+    if (tiles0 > INT32_MAX || tilest > INT32_MAX || batch > INT32_MAX ||
+        tiles0 * tilest > INT32_MAX || tiles0 * tilest * batch > INT32_MAX)
+      return TWG_E_UNSUPPORTED;
+    tg.tiles0 = (uint32_t)tiles0;
+    tg.tilest = (uint32_t)tilest;
+    const unsigned grid = (unsigned)(tiles0 * tilest * batch);
+    const uint32_t words = t0 * pitch;
+    const PixShape sh{t0, tt, pitch, words, small_div((uint32_t)C),
+                      small_div((tt * (uint32_t)C + 3) / 4), small_div((t0 * (uint32_t)C + 3) / 4)};
+    const size_t lds_bytes = (size_t)words * 4 * ((a_t ? 1 : 0) + (NIN == 2 && b_t ? 1 : 0));
+#define TWG_PIX(AT, BT) \
+  ew_pix<NIN, AT, BT, Op, TO, TA, TB><<<grid, kThreads, lds_bytes, s>>>(out, a, b, tg, sh, op)
+    if (a_t && b_t) {
+      if constexpr (NIN == 2) TWG_PIX(true, true);
+    } else if (a_t) {
+      TWG_PIX(true, false);
+    } else {
+      if constexpr (NIN == 2) TWG_PIX(false, true);
+    }
+#undef TWG_PIX
+    return (int)hipGetLastError();
+  }
+}
+
 }  // namespace
 }  // namespace twg
