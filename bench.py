@@ -633,7 +633,8 @@ def geometry_families(capi, L):
     fam = {}
     rows_ = []
     for shape in ([2048, 256, 7, 7], [512, 256, 14, 14], [128, 64, 56, 56], [32, 16, 1024, 64],
-                  [32, 16, 256, 256], [16, 2048, 1000], [256, 197, 768], [5792, 5792], [512, 768, 3, 27]):
+                  [32, 16, 256, 256], [16, 2048, 1000], [256, 197, 768], [5792, 5792], [512, 768, 3, 27],
+                  [256, 224, 224, 3]):
         for keep in itertools.product((True, False), repeat=len(shape)):
             if all(keep) or not any(keep):
                 continue
@@ -650,7 +651,8 @@ def geometry_families(capi, L):
     log(f"broadcast family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
         f"slowest {rows_[0]['pct_hbm_peak']}%")
     rows_ = []
-    for shape in ([32, 16, 1024, 64], [64, 128, 64, 64], [256, 197, 768], [512, 3, 224, 96], [128, 56, 56, 96]):
+    for shape in ([32, 16, 1024, 64], [64, 128, 64, 64], [256, 197, 768], [512, 3, 224, 96], [128, 56, 56, 96],
+                  [256, 224, 224, 3]):
         nd = len(shape)
         n = 1
         for s in shape:

@@ -122,6 +122,9 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
       const int64_t C = g.shape[0];
       auto y_of = [&](int o) {
         if (g.stride[o][1] == C) return 0;  // stored like the output
+        // (an operand broadcast along x is better off gathered: [256,224,224,3] + [256,1,1,3]
+        // 79% of peak against 65% through the tiles)
+        if (g.stride[o][1] == 0) return -1;
         for (int d = 2; d < g.ndim; ++d)
           if (g.stride[o][d] == C) return d;
         return -1;
