@@ -387,6 +387,46 @@ def test_add_permuted_operand_tiles(twg, shape, order):
         assert bit_equal(r, torch.relu(a))
 
 
+@pytest.mark.parametrize("rows,cols", [(8, 64), (37, 128), (5, 4096), (16, 36), (3, 260), (64, 32), (2, 12288)])
+def test_rows_stepped_by_two_and_three(twg, rows, cols):
+    # x[:, ::2]: a lane fetches the two aligned packs that hold its four elements and keeps
+    # every second value (x[:, ::3] stays with the gather and is checked beside it).  One or both inputs stepped, different steps, either
+    # slot, rows that merge into one run, three dimensions, an activation over the view, views
+    # that end with the storage's last element, and starts that break the 16-byte alignment
+    # (those take the gather).
+    g = torch.Generator().manual_seed(rows * 7 + cols)
+    x2 = torch.randn(rows, 2 * cols, generator=g)
+    x3 = torch.randn(rows, 3 * cols, generator=g)
+    d = torch.randn(rows, cols, generator=g)
+    a2, a3 = x2[:, ::2], x3[:, ::3]
+    _say(f"stepped rows {rows} x {cols}")
+    assert bit_equal(H.add(a2, d, alpha=0.5), oracle.add(a2, d, alpha=0.5))
+    assert bit_equal(H.add(d, a2), oracle.add(d, a2))
+    assert bit_equal(H.add(a3, d, alpha=-2.0), oracle.add(a3, d, alpha=-2.0))
+    assert bit_equal(H.add(d, a3), oracle.add(d, a3))
+    assert bit_equal(H.add(a2, x2[:, 1::2]), oracle.add(a2, x2[:, 1::2]))         # second input unaligned
+    assert bit_equal(H.add(a2, a3, alpha=0.25), oracle.add(a2, a3, alpha=0.25))
+    assert bit_equal(H.add(a3, a2), oracle.add(a3, a2))
+    assert bit_equal(H.add(a2, a2), oracle.add(a2, a2))
+    assert bit_equal(H.add(a3, x3[:, 2::3]), oracle.add(a3, x3[:, 2::3]))         # ends with the storage
+    assert bit_equal(H.binary("twg_mul_f32", a3, d), a3 * d)
+    assert bit_equal(H.unary("twg_unary_f32", a2, pre=(ctypes.c_int(1),)), torch.relu(a2))
+    assert bit_equal(H.unary("twg_unary_f32", a3, pre=(ctypes.c_int(0),)), a3.contiguous())
+    # rows that do not merge (a narrower view of the stepped rows), and three dimensions
+    w = cols - 4
+    assert bit_equal(H.add(a2[:, :w], d[:, :w]), oracle.add(a2[:, :w], d[:, :w]))
+    assert bit_equal(H.add(a3[:, 4:], d[:, 4:]), oracle.add(a3[:, 4:], d[:, 4:]))
+    y = torch.randn(3, rows, 2 * cols, generator=g)
+    e = torch.randn(3, rows, cols, generator=g)
+    assert bit_equal(H.add(y[..., ::2], e), oracle.add(y[..., ::2], e))
+    assert bit_equal(H.add(y[1:, :, ::2], e[0]), oracle.add(y[1:, :, ::2], e[0]))  # e read again
+    assert bit_equal(H.add(y.transpose(0, 1)[..., ::2], e.transpose(0, 1)),
+                     oracle.add(y.transpose(0, 1)[..., ::2], e.transpose(0, 1)))
+    # output stepped as well stays with the general walk
+    o = torch.zeros(rows, 2 * cols)[:, ::2]
+    assert bit_equal(H.add(a2, d, out=o), oracle.add(a2, d))
+
+
 @pytest.mark.parametrize("rows,cols,pad,start", [
     (37, 1000, 1, 1), (37, 1000, 5, 0), (50, 1001, 3, 2), (9, 4099, 1, 1), (300, 256, 2, 1),
     (3, 70001, 7, 3), (64, 999, 0, 0), (130, 66, 1, 1)])

@@ -84,6 +84,11 @@ int launch_ew(TO *out, const TA *a, const TB *b, const twg_iter_t *it, Op op, tw
       const int r = launch_generic_vec<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
       if (r != TWG_E_UNSUPPORTED) return r;
     }
+    // (i-b2) the same walk for inputs stepped by 2 elements along their rows
+    {
+      const int r = launch_stepped_vec<NIN, Op, TO, TA, TB>(out, a, b, g, op, s);
+      if (r != TWG_E_UNSUPPORTED) return r;
+    }
     // An input stored [.., x, c] with a short c against an output stored [.., c, x]: strips
     // through LDS (a single strip of fewer than 256 output elements per channel runs no
     // faster than a gather; with another dimension to take several strips from, 32 are enough).

@@ -336,6 +336,126 @@ int launch_generic_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, 
   }
 }
 
+// Rows whose inputs are stepped by 2 elements along dimension 0 (x[:, ::2]): the pack walk of
+// ew_generic_vec, where a lane fetches the two aligned packs that hold its four elements of a
+// stepped input and keeps every second value ([4096, 8192][:, ::2] + dense: 50% -> 62% of peak
+// in algorithmic bytes, which is 82% in lines moved; both inputs stepped: 42% -> 46%).  Both
+// packs hold an element of the operand, so what is read past the last one stays inside its
+// aligned 16 bytes.  A step of 3 the same way (three packs, 48 bytes from lane to lane) ran
+// slower than the gather, 39% against 43%, and stays with it.
+// SA / SB: step of input a / b (1: unit stride).
+template <int S, bool STREAM, typename T>
+__device__ __forceinline__ Pack<T, 4> load_stepped(const T *p) {
+  using P4 = Pack<T, 4>;
+  const P4 *q = reinterpret_cast<const P4 *>(p);
+  if constexpr (S == 1) {
+    return load_pack<STREAM>(q);
+  } else {
+    static_assert(S == 2, "steps of 1 and 2 elements");
+    const P4 p0 = load_pack<STREAM>(q), p1 = load_pack<STREAM>(q + 1);
+    P4 r;
+    r.v[0] = p0.v[0];
+    r.v[1] = p0.v[2];
+    r.v[2] = p1.v[0];
+    r.v[3] = p1.v[2];
+    return r;
+  }
+}
+
+template <int NIN, int SA, int SB, bool STREAM, typename Op, typename TO, typename TA, typename TB>
+__global__ __launch_bounds__(64) void ew_stepped_vec(TO *out, const TA *a, const TB *b,
+                                                     GenGeom<uint32_t, int32_t> g, Op op) {
+  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  using PO = Pack<TO, 4>;
+  using PA = Pack<TA, 4>;
+  using PB = Pack<TB, 4>;
+  const uint32_t i = blockIdx.x * 64u + threadIdx.x;
+  if (i >= g.numel) return;
+  uint32_t rem = i;
+  int32_t oo = 0, oa = 0, ob = 0;
+  for (int d = 0; d < g.ndim; ++d) {
+    const uint32_t q = rem / g.shape[d];
+    const int32_t c = (int32_t)(rem - q * g.shape[d]);
+    rem = q;
+    oo += c * g.stride[0][d];
+    oa += c * g.stride[1][d];
+    if constexpr (NIN == 2) ob += c * g.stride[2][d];
+  }
+  const PA va = load_stepped<SA, STREAM>(a + oa);
+  PB vb;
+  if constexpr (NIN == 2) vb = load_stepped<SB, STREAM>(b + ob);
+  PO r;
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    r.v[k] = apply<NIN, Op, TO, TA, TB>(op, va.v[k], NIN == 2 ? vb.v[k] : TB());
+  store_pack<STREAM>(reinterpret_cast<PO *>(out + oo), r);
+}
+
+// Unit-stride output rows of a whole number of packs, inputs with a step of 1 or 2 along
+// dimension 0 (at least one of them stepped), every pack aligned.  Returns TWG_E_UNSUPPORTED
+// when the geometry is not of that kind.
+template <int NIN, typename Op, typename TO, typename TA, typename TB>
+int launch_stepped_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
+  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+    return TWG_E_UNSUPPORTED;
+  } else {
+    const int64_t sa0 = g.stride[1][0], sb0 = NIN == 2 ? g.stride[2][0] : 1;
+    if (g.ndim < 1 || g.stride[0][0] != 1 || sa0 < 1 || sa0 > 2 || sb0 < 1 || sb0 > 2 ||
+        (sa0 == 1 && sb0 == 1) || g.shape[0] % 4 != 0 || g.shape[0] < 32 || g.numel > INT32_MAX)
+      return TWG_E_UNSUPPORTED;
+    auto packs_aligned = [&](int o, const void *p) {
+      if (!aligned_to(p, 16)) return false;
+      for (int d = 1; d < g.ndim; ++d)
+        if (g.stride[o][d] % 4 != 0) return false;
+      return true;
+    };
+    if (!packs_aligned(0, out) || !packs_aligned(1, a) || (NIN == 2 && !packs_aligned(2, b)))
+      return TWG_E_UNSUPPORTED;
+    // an input that is read again and again (broadcast along an outer dimension) is better
+    // off with the kernels that keep it in cache
+    if (read_again<NIN>(g, 1, sizeof(TA)) || (NIN == 2 && read_again<NIN>(g, 2, sizeof(TB))))
+      return TWG_E_UNSUPPORTED;
+    GenGeom<uint32_t, int32_t> gg{};
+    gg.ndim = g.ndim;
+    gg.numel = (uint32_t)(g.numel / 4);
+    for (int o = 0; o <= NIN; ++o) {
+      int64_t span = 0;
+      for (int d = 0; d < g.ndim; ++d) {
+        const int64_t st = g.stride[o][d] < 0 ? -g.stride[o][d] : g.stride[o][d];
+        span += st * (g.shape[d] - 1);
+      }
+      if (span > INT32_MAX - 16) return TWG_E_UNSUPPORTED;
+    }
+    for (int d = 0; d < TWG_MAX_DIMS; ++d) {
+      gg.shape[d] = (uint32_t)g.shape[d];
+      for (int o = 0; o < 3; ++o) gg.stride[o][d] = (int32_t)g.stride[o][d];
+    }
+    gg.shape[0] = (uint32_t)(g.shape[0] / 4);  // dimension 0 counts packs of the output
+    for (int o = 0; o < 3; ++o) gg.stride[o][0] = (int32_t)(g.stride[o][0] * 4);
+    const unsigned grid = (unsigned)((gg.numel + 63) / 64);
+    const bool stream = g.numel * (int64_t)(4 * (1 + sa0 + (NIN == 2 ? sb0 : 0))) > kStreamBytes;
+#define TWG_SV(SA, SB)                                                                          \
+  do {                                                                                          \
+    if (stream)                                                                                 \
+      ew_stepped_vec<NIN, SA, SB, true, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
+    else                                                                                        \
+      ew_stepped_vec<NIN, SA, SB, false, Op, TO, TA, TB><<<grid, 64, 0, s>>>(out, a, b, gg, op); \
+  } while (0)
+    if (sa0 == 2 && sb0 == 1) {
+      TWG_SV(2, 1);
+    } else {
+      if constexpr (NIN == 2) {
+        if (sa0 == 1) TWG_SV(1, 2);
+        else TWG_SV(2, 2);
+      } else {
+        return TWG_E_UNSUPPORTED;
+      }
+    }
+#undef TWG_SV
+    return (int)hipGetLastError();
+  }
+}
+
 template <int NIN, int VEC, bool A_BC, bool B_BC, typename Op, typename TO, typename TA,
           typename TB, bool ANY = false>
 int launch_rows_v(TO *out, const TA *a, const TB *b, const Geom &g, Op op, hipStream_t s) {
