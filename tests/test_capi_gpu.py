@@ -385,6 +385,13 @@ def test_add_permuted_operand_tiles(twg, shape, order):
         assert bit_equal(H.add(a, b, out=out), oracle.add(a, b))
         r = H.unary("twg_unary_f32", a, pre=(ctypes.c_int(1),))          # relu, contiguous output
         assert bit_equal(r, torch.relu(a))
+        if off != 3:
+            # a compare over the same layouts (its bools leave the tiles four to a dword); values
+            # rounded to halves so that both outcomes occur
+            ar, br = (a * 2).round(), (b * 2).round()
+            assert ar.stride() == a.stride()
+            assert torch.equal(H.binary("twg_eq_f32", ar, br, out_dtype=torch.bool), torch.eq(ar, br))
+            assert torch.equal(H.binary("twg_eq_f32", br, ar, out_dtype=torch.bool), torch.eq(br, ar))
 
 
 @pytest.mark.parametrize("rows,cols", [(8, 64), (37, 128), (5, 4096), (16, 36), (3, 260), (64, 32), (2, 12288)])

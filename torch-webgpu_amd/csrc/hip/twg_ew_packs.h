@@ -125,12 +125,16 @@ __device__ __forceinline__ Pack<T, 4> load4_any(const T *p) {
 }
 template <bool NT = true, typename T>
 __device__ __forceinline__ void store4_any(T *p, const Pack<T, 4> &x) {
-  U32x4A4 r;
-  __builtin_memcpy(&r, &x, 16);
-  if constexpr (NT) {
-    __builtin_nontemporal_store(r, reinterpret_cast<U32x4A4 *>(p));
+  if constexpr (sizeof(T) == 1) {  // four bools: one dword, which the caller keeps 4-byte aligned
+    store_pack<NT>(reinterpret_cast<Pack<T, 4> *>(p), x);
   } else {
-    *reinterpret_cast<U32x4A4 *>(p) = r;
+    U32x4A4 r;
+    __builtin_memcpy(&r, &x, 16);
+    if constexpr (NT) {
+      __builtin_nontemporal_store(r, reinterpret_cast<U32x4A4 *>(p));
+    } else {
+      *reinterpret_cast<U32x4A4 *>(p) = r;
+    }
   }
 }
 // up to 4 elements from p, `valid` of them inside the extent

@@ -220,7 +220,8 @@ template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO
           typename TB, int THREADS = kThreads>
 __global__ __launch_bounds__(THREADS) void ew_tile_vec(TO *out, const TA *a, const TB *b,
                                                         TileGeom g, Op op) {
-  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  static_assert((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4,
+                "4-byte inputs, 4-byte or 1-byte (compare) output");
   constexpr int kPitch = TD0 + 4;
   __shared__ __attribute__((aligned(16))) TA sa[A_T ? TT : 1][A_T ? kPitch : 4];
   __shared__ __attribute__((aligned(16))) TB sb[(NIN == 2 && B_T) ? TT : 1][(NIN == 2 && B_T) ? kPitch : 4];
@@ -255,7 +256,8 @@ template <int NIN, bool A_T, bool B_T, int TD0, int TT, typename Op, typename TO
           typename TB, int THREADS>
 __global__ __launch_bounds__(THREADS) void ew_tile_any(TO *out, const TA *a, const TB *b,
                                                         TileGeom g, Op op) {
-  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  static_assert((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4,
+                "4-byte inputs, 4-byte or 1-byte (compare) output");
   using PO = Pack<TO, 4>;
   using PA = Pack<TA, 4>;
   using PB = Pack<TB, 4>;
@@ -396,7 +398,8 @@ struct DeintShape {
 template <int NIN, bool A_D, bool B_D, typename Op, typename TO, typename TA, typename TB>
 __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const TB *b, TileGeom g,
                                                      DeintShape sh, Op op) {
-  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  static_assert((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4,
+                "4-byte inputs, 4-byte or 1-byte (compare) output");
   using PO = Pack<TO, 4>;
   using PA = Pack<TA, 4>;
   using PB = Pack<TB, 4>;
@@ -527,6 +530,18 @@ __global__ __launch_bounds__(kThreads) void ew_deint(TO *out, const TA *a, const
   }
 }
 
+// A 1-byte output (the bools of a compare) leaves the strip and pixel kernels as dwords of four
+// elements: the pointer and every output stride from dimension `from` on must be multiples of
+// 4 (the kernels' own offsets along the dimensions before that are).
+template <typename TO>
+bool out_packs_aligned(const TO *out, const Geom &g, int from) {
+  if (sizeof(TO) != 1) return true;
+  if (!aligned_to(out, 4)) return false;
+  for (int d = from; d < g.ndim; ++d)
+    if (g.stride[0][d] % 4 != 0) return false;
+  return true;
+}
+
 // t: the dimension the transposed operands have their unit stride along; or, with pin >= 1,
 // the outer one of two dimensions (t, pin) that lie back to back in those operands' memory
 // (unit stride along pin, stride shape[pin] along t) and are walked as one.  merge01: the
@@ -601,9 +616,10 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
 
   // 128-bit path: 4-byte elements, everything a multiple of 4 elements, and every
   // operand with its unit stride either along dimension 0 or (if marked) along t.
-  if constexpr (sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4) {
+  // (a compare's output of bools moves as one dword per lane)
+  if constexpr ((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4) {
     bool ok = tg.n0 % 4 == 0 && tg.nt % 4 == 0 && tg.s0[0] == 1 && tg.st[0] % 4 == 0 &&
-              aligned_to(out, 16) && aligned_to(a, 16) && (NIN == 1 || aligned_to(b, 16));
+              aligned_to(out, 4 * sizeof(TO)) && aligned_to(a, 16) && (NIN == 1 || aligned_to(b, 16));
     ok = ok && (a_t ? (tg.st[1] == 1 && tg.s0[1] % 4 == 0 && tg.s1[1] % 4 == 0)
                     : (tg.s0[1] == 1 && tg.st[1] % 4 == 0));
     if (NIN == 2)
@@ -626,6 +642,11 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
       };
       bool any = tg.s0[0] == 1 && (a_t ? unit_t(1) : tg.s0[1] == 1);
       if (NIN == 2) any = any && (b_t ? unit_t(2) : tg.s0[2] == 1);
+      if (sizeof(TO) == 1) {  // the dwords of four bools must be aligned
+        any = any && aligned_to(out, 4) && tg.st[0] % 4 == 0 && (tg.psplit <= 1 || tg.sp[0] % 4 == 0) &&
+              (tg.n0in == 0 || tg.n0in % 4 == 0);
+        for (int d = 0; d < tg.nbatch && any; ++d) any = tg.bstride[0][d] % 4 == 0;
+      }
       if (any) {
         if (!set_tiles(wide ? 256 : mid ? 128 : 64, wide ? 32 : 64, &grid, true)) return TWG_E_UNSUPPORTED;
         const bool big = g.numel >= (int64_t(1) << 27);
@@ -708,9 +729,10 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
 template <int NIN, typename Op, typename TO, typename TA, typename TB>
 int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool a_d, bool b_d,
                  Op op, hipStream_t s) {
-  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+  if constexpr ((sizeof(TO) != 4 && sizeof(TO) != 1) || sizeof(TA) != 4 || sizeof(TB) != 4) {
     return TWG_E_UNSUPPORTED;
   } else {
+    if (!out_packs_aligned(out, g, 1)) return TWG_E_UNSUPPORTED;
     const int64_t P = g.shape[pd];
     // (from 32 elements on, a run of P is a whole 128-byte line and the tile kernels do better)
     if (P < 2 || P >= 32 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
@@ -804,7 +826,8 @@ struct InterShape {
 template <int NIN, bool A_P, bool B_P, typename Op, typename TO, typename TA, typename TB>
 __global__ __launch_bounds__(kThreads) void ew_inter(TO *out, const TA *a, const TB *b, TileGeom g,
                                                      InterShape sh, Op op) {
-  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  static_assert((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4,
+                "4-byte inputs, 4-byte or 1-byte (compare) output");
   using PO = Pack<TO, 4>;
   using PA = Pack<TA, 4>;
   using PB = Pack<TB, 4>;
@@ -938,9 +961,10 @@ __global__ __launch_bounds__(kThreads) void ew_inter(TO *out, const TA *a, const
 template <int NIN, typename Op, typename TO, typename TA, typename TB>
 int launch_inter(TO *out, const TA *a, const TB *b, const Geom &g, bool a_p, bool b_p, Op op,
                  hipStream_t s) {
-  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+  if constexpr ((sizeof(TO) != 4 && sizeof(TO) != 1) || sizeof(TA) != 4 || sizeof(TB) != 4) {
     return TWG_E_UNSUPPORTED;
   } else {
+    if (!out_packs_aligned(out, g, 2)) return TWG_E_UNSUPPORTED;
     if (g.ndim < 2) return TWG_E_UNSUPPORTED;
     const int64_t P = g.shape[0];
     if (P < 2 || P >= 32 || g.stride[0][0] != 1 || g.stride[0][1] != P) return TWG_E_UNSUPPORTED;
@@ -1026,7 +1050,8 @@ struct PixShape {
 template <int NIN, bool A_T, bool B_T, typename Op, typename TO, typename TA, typename TB>
 __global__ __launch_bounds__(kThreads) void ew_pix(TO *out, const TA *a, const TB *b, TileGeom g,
                                                    PixShape sh, Op op) {
-  static_assert(sizeof(TO) == 4 && sizeof(TA) == 4 && sizeof(TB) == 4, "4-byte elements only");
+  static_assert((sizeof(TO) == 4 || sizeof(TO) == 1) && sizeof(TA) == 4 && sizeof(TB) == 4,
+                "4-byte inputs, 4-byte or 1-byte (compare) output");
   using PO = Pack<TO, 4>;
   using PA = Pack<TA, 4>;
   using PB = Pack<TB, 4>;
@@ -1144,9 +1169,10 @@ __global__ __launch_bounds__(kThreads) void ew_pix(TO *out, const TA *a, const T
 template <int NIN, typename Op, typename TO, typename TA, typename TB>
 int launch_pix(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t, bool b_t, Op op,
                hipStream_t s) {
-  if constexpr (sizeof(TO) != 4 || sizeof(TA) != 4 || sizeof(TB) != 4) {
+  if constexpr ((sizeof(TO) != 4 && sizeof(TO) != 1) || sizeof(TA) != 4 || sizeof(TB) != 4) {
     return TWG_E_UNSUPPORTED;
   } else {
+    if (!out_packs_aligned(out, g, 2)) return TWG_E_UNSUPPORTED;
     if (g.ndim < 3 || t < 2 || t >= g.ndim || !(a_t || b_t)) return TWG_E_UNSUPPORTED;
     const int64_t C = g.shape[0];
     if (C < 2 || C >= 32 || g.stride[0][0] != 1 || g.stride[0][1] != C) return TWG_E_UNSUPPORTED;
