@@ -260,6 +260,12 @@ size_t twg_masked_select_scratch_bytes(int64_t numel);
  * addresses mask, stride[TWG_OUT] is ignored; dim 0 fastest, so logical index i
  * is the row-major index of the broadcast shape reversed.  Asynchronous: read
  * *d_count with twg_memcpy_d2h (or call twg_masked_select_count, below).
+ * A source or mask that is not dense in logical order (or is off its alignment: four
+ * elements for the source, 4 bytes for the mask) is first copied dense on the device, from
+ * 2^16 elements on, into a block of the library's allocator (numel elements for the source,
+ * numel bytes for the mask; returned to the allocator before the call returns, reusable once
+ * the stream has passed it); if the allocator has no room, or the stream is being captured,
+ * such operands are gathered element by element instead, 3-5 times slower.
  * The scratch must belong to this call alone until its kernels have finished: it holds a
  * ticket counter and one status word per tile.  No wait inside the kernels is unbounded:
  * if the scratch is shared by two launches in flight, or overwritten under a running one,

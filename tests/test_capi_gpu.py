@@ -1246,6 +1246,38 @@ def test_masked_select_misaligned_broadcast_strided(twg):
     assert bit_equal(v, torch.masked_select(xs, ms))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.uint8, torch.int16, torch.int64])
+def test_masked_select_layouts_that_are_copied_dense_first(twg, dtype):
+    # From 2^16 elements on, a source or mask that is not dense in logical order (transposed,
+    # sliced, broadcast along rows or columns, off its alignment) is written out dense before the
+    # vectorised kernels run: same values, same order, nothing written past the k results.
+    g = torch.Generator().manual_seed(77)
+    rows, cols = 640, 1000
+    x = (torch.randn(rows, cols, generator=g) * 1000).to(dtype)
+    m = torch.rand(rows, cols, generator=g) < 0.45
+    xt = (torch.randn(cols, rows, generator=g) * 1000).to(dtype).t()
+    mt = (torch.rand(cols, rows, generator=g) < 0.6).t()
+    wide = (torch.randn(rows, 2 * cols + 3, generator=g) * 1000).to(dtype)
+    cases = [
+        ("source transposed", xt, m),
+        ("mask transposed", x, mt),
+        ("both transposed", xt, mt),
+        ("one mask row for all rows", x, m[3]),
+        ("one mask value per row", x, m[:, 5:6]),
+        ("one source row under a full mask", x[7], m),
+        ("source stepped by 2", wide[:, 1:2 * cols:2], m),
+        ("source and mask off their alignment", x.flatten()[1:-3], m.flatten()[3:-1]),
+        ("three dimensions, the middle one broadcast", x.view(rows, 1, cols).expand(rows, 2, cols)[:400], m[:400].view(400, 1, cols)),
+    ]
+    for name, xs, ms in cases:
+        _say(f"masked_select {dtype} {name}")
+        vals, k = H.masked_select(xs, ms, check_guard=True)
+        ref = torch.masked_select(xs, ms)
+        assert k == ref.numel() and bit_equal(vals, ref), (dtype, name)
+        if dtype == torch.float32:
+            assert bit_equal(vals, oracle.masked_select(xs, ms)), name
+
+
 def test_masked_select_rejects_small_scratch(twg):
     x = torch.rand(100000)
     m = x > 0.5

@@ -25,8 +25,9 @@ int ensure_init();
 
 // The compaction behind the masked_select entry points: elements of 1, 2, 4 or 8
 // bytes, count written to *d_count (device memory, or host memory the device can
-// address).  Dense 16-byte-aligned sources of 4-byte elements take the vectorised
-// kernels, everything else the one-element-per-lane kernel.
+// address).  Dense, aligned sources and masks take the vectorised kernels; other layouts
+// are first copied dense into blocks of the caching allocator (allow_alloc, from 2^16
+// elements on) or take the one-element-per-lane kernel.
 // `wait` is only ever set by the test hook: the ticket counter's first value (0..255; tiles
 // below it are never compacted or published) and the number of polling rounds after which
 // a look-back gives up (0 = the library's limit).
@@ -36,7 +37,8 @@ struct MsWait {
 };
 int masked_select_launch(void *out, int64_t *d_count, const void *src, int elem_size,
                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                         size_t scratch_bytes, twg_stream_t stream, MsWait wait = MsWait());
+                         size_t scratch_bytes, twg_stream_t stream, MsWait wait = MsWait(),
+                         bool allow_alloc = true);
 
 
 // Look up the address the current device gives the masked_select scratch array that is

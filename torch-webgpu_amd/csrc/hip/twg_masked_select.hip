@@ -103,7 +103,7 @@ namespace twg {
 
 int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int elem_size,
                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                         size_t scratch_bytes, twg_stream_t stream, MsWait wait) {
+                         size_t scratch_bytes, twg_stream_t stream, MsWait wait, bool allow_alloc) {
   if (wait.max_rounds == 0) wait.max_rounds = kMsMaxPollRounds;
   if (wait.first_ticket > 255) return TWG_E_INVALID_ARG;
   int rc = ensure_init();
@@ -140,6 +140,72 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
       case 4: return launch_fast<float>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
       default: return launch_fast<uint64_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
     }
+  }
+
+  // Anything else (a transposed or sliced source, a mask that is broadcast along rows,
+  // pointers off their alignment), from 2^16 elements on: the operand that is not dense is
+  // first written out dense, in logical order, by the elementwise copy kernels into a block
+  // of the caching allocator, and the fast variants run on that.  At 2^25 elements and
+  // p = 0.5 the one-element-per-lane kernel below takes 0.15-0.26 ms for such layouts, the
+  // dense path 0.05 ms and the copies 0.01-0.05 ms.  Callers that must not allocate
+  // (allow_alloc false, a stream under graph capture) and inputs the allocator has no room
+  // for stay with the kernel below.
+  // (a stream that is being captured must not meet an allocation either)
+  if (allow_alloc) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    TWG_HIP_TRY(hipStreamIsCapturing(s, &cap));
+    if (cap != hipStreamCaptureStatusNone) allow_alloc = false;
+  }
+  if (allow_alloc && g.numel >= (int64_t(1) << 16)) {
+    auto is_dense = [&](int o) {
+      int64_t want = 1;
+      for (int d = 0; d < g.ndim; ++d) {
+        if (g.stride[o][d] != want) return false;
+        want *= g.shape[d];
+      }
+      return true;
+    };
+    const bool copy_src = !is_dense(TWG_A) || reinterpret_cast<uintptr_t>(src_v) % src_align != 0;
+    const bool copy_mask = !is_dense(TWG_B) || reinterpret_cast<uintptr_t>(mask) % 4 != 0;
+    void *tmp_src = nullptr, *tmp_mask = nullptr;
+    bool have = true;
+    if (copy_src) have = twg_malloc(&tmp_src, (size_t)g.numel * elem_size) == 0 && tmp_src;
+    if (have && copy_mask) have = twg_malloc(&tmp_mask, (size_t)g.numel) == 0 && tmp_mask;
+    if (have) {
+      twg_iter_t ci{};
+      ci.ndim = g.ndim;
+      ci.numel = g.numel;
+      int64_t acc = 1;
+      for (int d = 0; d < g.ndim; ++d) {
+        ci.shape[d] = g.shape[d];
+        ci.stride[TWG_OUT][d] = acc;
+        acc *= g.shape[d];
+      }
+      if (copy_src) {
+        for (int d = 0; d < g.ndim; ++d) ci.stride[TWG_A][d] = g.stride[TWG_A][d];
+        rc = twg_record_stream(tmp_src, stream);
+        if (!rc) rc = twg_copy_strided(tmp_src, src_v, elem_size, &ci, stream);
+      }
+      if (!rc && copy_mask) {
+        for (int d = 0; d < g.ndim; ++d) ci.stride[TWG_A][d] = g.stride[TWG_B][d];
+        rc = twg_record_stream(tmp_mask, stream);
+        if (!rc) rc = twg_copy_strided(tmp_mask, mask, 1, &ci, stream);
+      }
+      if (!rc) {
+        const void *fs = copy_src ? tmp_src : src_v;
+        const uint8_t *fm = copy_mask ? static_cast<const uint8_t *>(tmp_mask) : mask;
+        switch (elem_size) {
+          case 1: rc = launch_fast<uint8_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
+          case 2: rc = launch_fast<uint16_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
+          case 4: rc = launch_fast<float>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
+          default: rc = launch_fast<uint64_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
+        }
+      }
+    }
+    // (freed blocks wait for the work queued on the caller's stream: twg_record_stream above)
+    if (tmp_src) twg_free(tmp_src);
+    if (tmp_mask) twg_free(tmp_mask);
+    if (have) return rc;
   }
 
   // scratch: [0] ticket, [256...] one status word per tile
@@ -255,7 +321,8 @@ int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
     if (q == hipErrorNotReady) return TWG_E_BUSY;
     if (q != hipSuccess) return (int)q;
   }
-  rc = masked_select_launch(out, d_count, src, 4, mask, it, ptr, kStaticScratchBytes, stream);
+  rc = masked_select_launch(out, d_count, src, 4, mask, it, ptr, kStaticScratchBytes, stream, MsWait(),
+                            /*allow_alloc=*/false);
   if (rc == 0 && !capturing) {
     TWG_HIP_TRY(hipEventRecord(use.done, s));
     use.last = s;

@@ -339,14 +339,8 @@ at::Tensor masked_select_impl(const at::Tensor &self, const at::Tensor &mask, at
     }
     return at::empty({0}, self.options());
   }
-  // The compaction kernels stream dense operands 3-5x faster than they gather strided or
-  // broadcast ones element by element (2^26 elements: 0.09 ms against 0.31-0.47 ms), and a
-  // strided copy runs near the dense rate, so from 2^16 elements on anything that is not
-  // dense is laid out densely first (a broadcast mask: +0.02 ms, a strided source: +0.08 ms).
-  if (n >= (int64_t(1) << 16)) {
-    if (!me.is_contiguous()) me = me.contiguous();
-    if (!se.is_contiguous()) se = se.contiguous();
-  }
+  // (operands that are not dense in logical order are laid out densely inside the library,
+  // from 2^16 elements on, before its streaming kernels run)
 
   twg_iter_t it;
   fill_iter_logical(se, me, &it);
