@@ -217,11 +217,12 @@ def main():
 
     def run_ms(mask_buf=None):
         """The op as the dispatcher runs it: compaction with the count handed to the host
-        (the call returns once the count is known; the output is stream ordered)."""
+        (the call returns once the count is known; the output is stream ordered), tickets
+        and status words in the array the library keeps for this (no scratch passed)."""
         note_ms("masked_select_p0.50")
         capi.check(L.twg_masked_select_count(d_out.ptr, ctypes.byref(k_host), d_src.ptr, 4,
                                              (mask_buf or d_m).ptr, ctypes.byref(it),
-                                             d_scratch.ptr, scratch_bytes, None))
+                                             None, 0, None))
         return k_host.value
 
     bytes_add = W.BYTES_PER_ELEM["add"] * n

@@ -286,8 +286,11 @@ int twg_masked_select_f32(float *out, int64_t *d_count, const float *src,
  * reference.  The call allocates nothing and frees nothing once the library is
  * initialised (call twg_init() first: initialisation itself creates the stream).
  * it->numel may be at most TWG_MS_STATIC_MAX_NUMEL; larger inputs return TWG_E_TOO_LARGE.
- * All calls on one GPU share the one array.  Calls on one stream are ordered and each clears
- * what it needs; a call on another stream while the previous call's kernels are still
+ * All calls on one GPU share the one array.  Calls on one stream are ordered; nothing is
+ * cleared between them (each launch marks its status words with its own epoch and counts
+ * its tiles from where the ticket counter stands; the array is cleared before the first
+ * call, when the 2^20 epochs run out, after a launch that failed, and by every call from
+ * the first one under graph capture on).  A call on another stream while the previous call's kernels are still
  * running is refused with TWG_E_BUSY (the library records an event behind every call and
  * queries it; the event is created by twg_init).  Under graph capture that check cannot be
  * made and is skipped: a capturing caller orders its own uses of the array. */
@@ -320,7 +323,11 @@ int twg_masked_select_f32_wait_probe(float *out, int64_t *d_count, const float *
  * it needs K to shape the result.  `out` and `src` must be aligned to elem_size; every
  * element size takes the kernels of twg_masked_select_f32, instantiated for it (dense
  * operands with `src` aligned to four elements, 16 bytes for 8-byte elements; anything
- * else runs the one-element-per-lane variant). */
+ * else is copied dense first, see twg_masked_select_f32).
+ * scratch == NULL with scratch_bytes == 0 selects the array the library keeps for
+ * twg_masked_select_f32_static, with that entry point's limit (TWG_E_TOO_LARGE beyond
+ * TWG_MS_STATIC_MAX_NUMEL elements) and its rule for streams (TWG_E_BUSY); the launch that
+ * clears a caller's scratch then falls away (13 -> 9 us per call up to 2^19 elements). */
 int twg_masked_select_count(void *out, int64_t *count_host, const void *src,
                             int32_t elem_size, const uint8_t *mask, const twg_iter_t *it,
                             void *scratch, size_t scratch_bytes, twg_stream_t stream);

@@ -161,6 +161,27 @@ def masked_select(x, mask, scratch_bytes=None, out_offset=0, check_guard=False):
     return vals, k
 
 
+def masked_select_on_library_array(x, mask):
+    """twg_masked_select_count without a scratch of the caller's (the library's own array).
+    Returns (values, count)."""
+    L = capi.load()
+    shape = torch.broadcast_shapes(x.shape, mask.shape)
+    xe, me = _expanded(shape, x, mask)
+    n = 1
+    for s in shape:
+        n *= s
+    es = x.element_size()
+    ux, um = Uploaded(x), Uploaded(mask)
+    out = capi.DeviceBuffer(max(es * n, es) + 256)
+    it = _iter_for(shape, None, (xe, me), sort_by_out=False)
+    kh = ctypes.c_int64(-7)
+    capi.check(L.twg_masked_select_count(out.ptr, ctypes.byref(kh), ux.ptr, es, um.ptr, ctypes.byref(it),
+                                         None, 0, None))
+    k = kh.value
+    vals = out.download((k,), x.dtype) if k else torch.empty(0, dtype=x.dtype)
+    return vals, k
+
+
 def compare_eq(a, b):
     """twg_eq on two CPU tensors of one dtype (broadcast together); returns a bool tensor."""
     L = capi.load()

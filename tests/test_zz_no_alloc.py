@@ -78,6 +78,47 @@ def test_static_scratch_matches_allocated_scratch(twg):
     _both(twg, L, 40000, 0.6, 5, shift=3)
 
 
+def test_static_scratch_is_not_cleared_between_calls(twg):
+    # Calls in a row on the library's array, which no launch clears in between: each launch
+    # tells its status words from its predecessors' by their epoch and counts its tiles from
+    # where the ticket counter stands.  Sizes that take the streaming kernel (thousands of
+    # status words), the small-tile kernel, a single tile (no ticket drawn) and the
+    # one-element-per-lane kernel, growing and shrinking, every density; also through the entry
+    # point that hands the count to the host, for other element sizes and with layouts that are
+    # copied dense first.
+    L = twg.load()
+    g = torch.Generator().manual_seed(2024)
+    sizes = [(1 << 21) + 5, 70001, (1 << 23) + 999, 8192, 300000, (1 << 22), 1000, 65536 * 3 + 1,
+             (1 << 21) + 5, 100, 40000, (1 << 24) + 17, 20000]
+    for i, n in enumerate(sizes):
+        p = (0.02, 0.5, 0.97, 0.3)[i % 4]
+        shift = 1 if i % 5 == 4 else 0
+        print(f"static call {i}: n={n} p={p} shift={shift}", flush=True)
+        src_all = torch.rand(n + shift, generator=g)
+        src, mask = src_all[shift:], torch.rand(n, generator=g) < p
+        d_src, d_mask = twg.to_device(src_all), twg.to_device(mask)
+        out, cnt = twg.DeviceBuffer(4 * n + 256), twg.DeviceBuffer(8)
+        it = twg.dense_iter(n)
+        if i % 3 == 2:
+            kh = ctypes.c_int64(-7)
+            twg.check(L.twg_masked_select_count(out.ptr, ctypes.byref(kh), d_src.at(4 * shift), 4, d_mask.ptr,
+                                                ctypes.byref(it), None, 0, None))
+            k = kh.value
+        else:
+            twg.check(L.twg_masked_select_f32_static(out.ptr, cnt.ptr, d_src.at(4 * shift), d_mask.ptr,
+                                                     ctypes.byref(it), None))
+            k = int(cnt.download((1,), torch.int64)[0])
+        assert k == int(mask.sum()), (i, n, k)
+        assert torch.equal(out.download((k,), torch.float32), src[mask]), (i, n)
+    # other element sizes and a transposed source through the count entry point
+    import capi_helpers as H
+    for dtype in (torch.int64, torch.uint8, torch.int16, torch.float32):
+        x = (torch.randn(700, 500, generator=g) * 100).to(dtype).t()
+        m = torch.rand(500, 700, generator=g) < 0.4
+        vals, k = H.masked_select_on_library_array(x, m)
+        assert k == int(m.sum()) and torch.equal(vals, torch.masked_select(x, m)), dtype
+
+
 def test_static_scratch_is_refused_to_a_second_stream_while_in_use(twg):
     # One array per GPU: a call on another stream while the previous call's kernels may still
     # be running must be refused (TWG_E_BUSY), not left to corrupt the tickets; once that work
@@ -133,3 +174,61 @@ def test_static_scratch_limits(twg):
     twg.check(L.twg_fill_bytes(cnt.ptr, 0xFF, 8, None))
     twg.check(L.twg_masked_select_f32_static(None, cnt.ptr, None, None, ctypes.byref(it0), None))
     assert int(cnt.download((1,), torch.int64)[0]) == 0
+
+
+def test_static_scratch_under_graph_capture_then_eager(twg):
+    # A graph that holds a launch on the library's array replays it with the arguments of its
+    # capture, so from the first call under capture on every call clears what it needs again.
+    # Eager calls, a captured call replayed with new contents, eager calls again: all exact.
+    hip = ctypes.CDLL("libamdhip64.so")
+    L = twg.load()
+    g = torch.Generator().manual_seed(555)
+
+    def eager(n, p):
+        src, mask = torch.rand(n, generator=g), torch.rand(n, generator=g) < p
+        d_src, d_mask = twg.to_device(src), twg.to_device(mask)
+        out, cnt = twg.DeviceBuffer(4 * n + 256), twg.DeviceBuffer(8)
+        it = twg.dense_iter(n)
+        twg.check(L.twg_masked_select_f32_static(out.ptr, cnt.ptr, d_src.ptr, d_mask.ptr, ctypes.byref(it), None))
+        k = int(cnt.download((1,), torch.int64)[0])
+        assert k == int(mask.sum()) and torch.equal(out.download((k,), torch.float32), src[mask]), (n, p)
+
+    eager((1 << 21) + 77, 0.5)
+    eager(90000, 0.2)
+    stream = ctypes.c_void_p()
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(stream), 1) == 0  # hipStreamNonBlocking
+    n = (1 << 21) + 4096 + 13
+    src, mask = torch.rand(n, generator=g), torch.rand(n, generator=g) < 0.37
+    d_src, d_mask = twg.to_device(src), twg.to_device(mask)
+    out, cnt = twg.DeviceBuffer(4 * n + 256), twg.DeviceBuffer(8)
+    it = twg.dense_iter(n)
+    twg.sync()
+    assert hip.hipStreamBeginCapture(stream, 1) == 0  # hipStreamCaptureModeThreadLocal
+    try:
+        rc = L.twg_masked_select_f32_static(out.ptr, cnt.ptr, d_src.ptr, d_mask.ptr, ctypes.byref(it), stream)
+    finally:
+        graph = ctypes.c_void_p()
+        rc_end = hip.hipStreamEndCapture(stream, ctypes.byref(graph))
+    assert rc == 0 and rc_end == 0, (rc, rc_end)
+    graph_exec = ctypes.c_void_p()
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)) == 0
+    try:
+        for rep in range(3):
+            print(f"static masked_select: graph replay {rep}", flush=True)
+            if rep:
+                src, mask = torch.rand(n, generator=g), torch.rand(n, generator=g) < (0.1 + 0.4 * rep)
+                d_src.upload(src)
+                d_mask.upload(mask)
+                eager(50000 * rep + 3, 0.6)   # eager work on the array between the replays
+            twg.sync()
+            assert hip.hipGraphLaunch(graph_exec, stream) == 0
+            assert hip.hipStreamSynchronize(stream) == 0
+            k = int(cnt.download((1,), torch.int64)[0])
+            assert k == int(mask.sum()), (rep, k)
+            assert torch.equal(out.download((k,), torch.float32), src[mask]), rep
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
+        hip.hipStreamDestroy(stream)
+    eager((1 << 22) + 5, 0.9)
+    eager(70001, 0.4)

@@ -34,11 +34,13 @@ struct MsLaunch {
   void *scratch;
   twg_stream_t stream;
   MsWait wait;
+  uint32_t *drawn;  // receives the number of tickets the launch draws
 };
 
 // Clear the header and `words` status words; a first ticket other than 0 (the test hook)
 // goes into the low byte of the ticket counter.
 int clear_scratch(void *scratch, size_t words, const MsWait &wait, twg_stream_t stream) {
+  if (wait.keep_scratch) return 0;  // the library's own array: told apart by epochs instead
   int rc = twg_fill_bytes(scratch, 0, kMsHeaderBytes + sizeof(uint64_t) * words, stream);
   if (rc == 0 && wait.first_ticket) rc = twg_fill_bytes(scratch, (int)wait.first_ticket, 1, stream);
   return rc;
@@ -54,9 +56,10 @@ int launch_stream(const MsLaunch<T> &m) {
   const size_t words = (size_t)ntiles * kStreamStatusStride;
   int rc = clear_scratch(m.scratch, words, m.wait, m.stream);
   if (rc) return rc;
+  *m.drawn = (uint32_t)ntiles;
   ms_compact_stream<WAVES, GROUPS, T><<<(unsigned)ntiles, WAVES * 64, 0, resolve_stream(m.stream)>>>(
       m.out, m.d_count, m.src, m.mask, m.numel, (uint32_t)ntiles, m.ticket, m.status,
-      m.wait.max_rounds);
+      MsRun{m.wait.max_rounds, m.wait.epoch, m.wait.ticket_base});
   return (int)hipGetLastError();
 }
 
@@ -64,14 +67,14 @@ int launch_stream(const MsLaunch<T> &m) {
 // variant below that.
 template <typename T>
 int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t *mask, int64_t numel,
-                void *scratch, twg_stream_t stream, const MsWait &wait) {
+                void *scratch, twg_stream_t stream, const MsWait &wait, uint32_t *drawn) {
   // scratch: [0] ticket, [256...] the tiles' status words
   uint32_t *ticket = static_cast<uint32_t *>(scratch);
   uint64_t *status = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kMsHeaderBytes);
   T *out = static_cast<T *>(out_v);
   const T *src = static_cast<const T *>(src_v);
   if (numel >= kStreamMinElems) {
-    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, status, scratch, stream, wait};
+    const MsLaunch<T> m{out, d_count, src, mask, numel, ticket, status, scratch, stream, wait, drawn};
     if (numel >= (int64_t(1) << 25)) return launch_stream<16, 4>(m);
     if (numel >= (int64_t(1) << 23)) return launch_stream<16, 2>(m);
     return launch_stream<8, 1>(m);
@@ -81,8 +84,10 @@ int launch_fast(void *out_v, int64_t *d_count, const void *src_v, const uint8_t 
   int rc = 0;
   // one tile takes no ticket and looks back at nothing: the scratch may hold anything
   if (ntiles > 1 && (rc = clear_scratch(scratch, ntiles, wait, stream))) return rc;
+  *drawn = ntiles > 1 ? ntiles : 0u;
   ms_compact_vec<kSmallWaves, T><<<ntiles, kSmallWaves * 64, 0, resolve_stream(stream)>>>(
-      out, d_count, src, mask, numel, ntiles, ticket, status, wait.max_rounds);
+      out, d_count, src, mask, numel, ntiles, ticket, status,
+      MsRun{wait.max_rounds, wait.epoch, wait.ticket_base});
   return (int)hipGetLastError();
 }
 
@@ -103,7 +108,11 @@ namespace twg {
 
 int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int elem_size,
                          const uint8_t *mask, const twg_iter_t *it, void *scratch,
-                         size_t scratch_bytes, twg_stream_t stream, MsWait wait, bool allow_alloc) {
+                         size_t scratch_bytes, twg_stream_t stream, MsWait wait, bool allow_alloc,
+                         uint32_t *tickets_drawn) {
+  uint32_t drawn_here = 0;
+  uint32_t *drawn = tickets_drawn ? tickets_drawn : &drawn_here;
+  *drawn = 0;
   if (wait.max_rounds == 0) wait.max_rounds = kMsMaxPollRounds;
   if (wait.first_ticket > 255) return TWG_E_INVALID_ARG;
   int rc = ensure_init();
@@ -118,6 +127,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
   Geom g;
   if ((rc = canonicalize(&local, 3, &g, false))) return rc;
   if (g.numel == 0) return twg_fill_bytes(d_count, 0, sizeof(int64_t), stream);
+  if (g.numel > kMsMaxNumel) return TWG_E_UNSUPPORTED;  // counts must fit a status word's value field
   if (!out_v || !src_v || !mask || !scratch) return TWG_E_INVALID_ARG;
   if (reinterpret_cast<uintptr_t>(out_v) % elem_size || reinterpret_cast<uintptr_t>(src_v) % elem_size)
     return TWG_E_INVALID_ARG;
@@ -135,10 +145,10 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
                     reinterpret_cast<uintptr_t>(mask) % 4 == 0;
   if (fast) {
     switch (elem_size) {
-      case 1: return launch_fast<uint8_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
-      case 2: return launch_fast<uint16_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
-      case 4: return launch_fast<float>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
-      default: return launch_fast<uint64_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait);
+      case 1: return launch_fast<uint8_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait, drawn);
+      case 2: return launch_fast<uint16_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait, drawn);
+      case 4: return launch_fast<float>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait, drawn);
+      default: return launch_fast<uint64_t>(out_v, d_count, src_v, mask, g.numel, scratch, stream, wait, drawn);
     }
   }
 
@@ -195,10 +205,10 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
         const void *fs = copy_src ? tmp_src : src_v;
         const uint8_t *fm = copy_mask ? static_cast<const uint8_t *>(tmp_mask) : mask;
         switch (elem_size) {
-          case 1: rc = launch_fast<uint8_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
-          case 2: rc = launch_fast<uint16_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
-          case 4: rc = launch_fast<float>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
-          default: rc = launch_fast<uint64_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait); break;
+          case 1: rc = launch_fast<uint8_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait, drawn); break;
+          case 2: rc = launch_fast<uint16_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait, drawn); break;
+          case 4: rc = launch_fast<float>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait, drawn); break;
+          default: rc = launch_fast<uint64_t>(out_v, d_count, fs, fm, g.numel, scratch, stream, wait, drawn); break;
         }
       }
     }
@@ -216,6 +226,7 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
   const uint32_t ntiles = (uint32_t)ntiles64;
   // one tile takes no ticket and looks back at nothing: the scratch may hold anything
   if (ntiles > 1 && (rc = clear_scratch(scratch, ntiles, wait, stream))) return rc;
+  *drawn = ntiles > 1 ? ntiles : 0u;
 
   {
     MsGeom mg{};
@@ -230,11 +241,11 @@ int masked_select_launch(void *out_v, int64_t *d_count, const void *src_v, int e
       if (dense)
         ms_compact_scalar<false, T><<<ntiles, kScalarWaves * 64, 0, s>>>(
             static_cast<T *>(out_v), d_count, static_cast<const T *>(src_v), mask, g.numel, ntiles,
-            ticket, status, wait.max_rounds, mg);
+            ticket, status, MsRun{wait.max_rounds, wait.epoch, wait.ticket_base}, mg);
       else
         ms_compact_scalar<true, T><<<ntiles, kScalarWaves * 64, 0, s>>>(
             static_cast<T *>(out_v), d_count, static_cast<const T *>(src_v), mask, g.numel, ntiles,
-            ticket, status, wait.max_rounds, mg);
+            ticket, status, MsRun{wait.max_rounds, wait.epoch, wait.ticket_base}, mg);
     };
     switch (elem_size) {
       case 1: scalar(uint8_t{}); break;
@@ -271,6 +282,19 @@ struct StaticUse {
   hipEvent_t done = nullptr;
   hipStream_t last = nullptr;
   bool used = false;
+  bool recorded = false;  // `done` stands behind the last call's kernels (a caller's stream)
+  // Only this library's launches write the array, so it is not cleared between them: each
+  // launch marks its status words with the next epoch and counts its tiles from where the
+  // ticket counter stands (MsWait::keep_scratch).  `trusted` says that the counters below
+  // describe the array (false before the first use and after a launch that failed: the array
+  // is then cleared once); when the epochs run out it is cleared as well.  A graph that holds
+  // a launch replays it with the arguments of its capture, which no counter here can follow:
+  // from the first call under capture on, every call clears what it needs as it does for a
+  // caller's scratch.
+  bool trusted = false;
+  bool captured_once = false;
+  uint32_t epoch = 0;
+  uint32_t ticket_next = 0;
 };
 StaticUse g_static_use[kMaxDevices];
 }  // namespace
@@ -289,17 +313,11 @@ int static_scratch_setup() {
 }
 }  // namespace twg
 
-extern "C" {
+namespace twg {
 
-int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const uint8_t *mask,
-                          const twg_iter_t *it, void *scratch, size_t scratch_bytes,
-                          twg_stream_t stream) {
-  return masked_select_launch(out, d_count, src, 4, mask, it, scratch, scratch_bytes, stream);
-}
-
-int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
-                                 const uint8_t *mask, const twg_iter_t *it,
-                                 twg_stream_t stream) {
+int masked_select_on_own_array(void *out, int64_t *d_count, const void *src, int elem_size,
+                               const uint8_t *mask, const twg_iter_t *it, twg_stream_t stream,
+                               bool allow_alloc) {
   int rc = ensure_init();
   if (rc) return rc;
   if (!it) return TWG_E_INVALID_ARG;
@@ -316,19 +334,61 @@ int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   TWG_HIP_TRY(hipStreamIsCapturing(s, &cap));
   const bool capturing = cap != hipStreamCaptureStatusNone;
+  if (capturing) use.captured_once = true;
   if (!capturing && use.used && use.last != s) {
-    const hipError_t q = hipEventQuery(use.done);
+    // (behind a call on the library's own stream no event is recorded: a marker behind every
+    // call cost the stream more than the clear that the epochs save, 1-2 us per call.  That
+    // stream outlives every caller and is asked itself: busy while anything on it is pending.)
+    const hipError_t q = use.recorded ? hipEventQuery(use.done) : hipStreamQuery(use.last);
     if (q == hipErrorNotReady) return TWG_E_BUSY;
     if (q != hipSuccess) return (int)q;
   }
-  rc = masked_select_launch(out, d_count, src, 4, mask, it, ptr, kStaticScratchBytes, stream, MsWait(),
-                            /*allow_alloc=*/false);
+  MsWait wait;
+  const bool keep = !use.captured_once;
+  if (keep) {
+    if (!use.trusted || use.epoch + 1 >= kEpochLimit) {
+      if ((rc = twg_fill_bytes(ptr, 0, kStaticScratchBytes, stream))) return rc;
+      use.epoch = 0;
+      use.ticket_next = 0;
+      use.trusted = true;
+    }
+    wait.keep_scratch = true;
+    wait.epoch = ++use.epoch;
+    wait.ticket_base = use.ticket_next;
+  }
+  uint32_t drawn = 0;
+  rc = masked_select_launch(out, d_count, src, elem_size, mask, it, ptr, kStaticScratchBytes, stream,
+                            wait, allow_alloc, &drawn);
+  if (keep) {
+    if (rc == 0) use.ticket_next += drawn;
+    else use.trusted = false;
+  }
   if (rc == 0 && !capturing) {
-    TWG_HIP_TRY(hipEventRecord(use.done, s));
+    use.recorded = false;
+    if (s != resolve_stream(nullptr)) {  // a caller's stream may be gone by the next call
+      TWG_HIP_TRY(hipEventRecord(use.done, s));
+      use.recorded = true;
+    }
     use.last = s;
     use.used = true;
   }
   return rc;
+}
+
+}  // namespace twg
+
+extern "C" {
+
+int twg_masked_select_f32(float *out, int64_t *d_count, const float *src, const uint8_t *mask,
+                          const twg_iter_t *it, void *scratch, size_t scratch_bytes,
+                          twg_stream_t stream) {
+  return masked_select_launch(out, d_count, src, 4, mask, it, scratch, scratch_bytes, stream);
+}
+
+int twg_masked_select_f32_static(float *out, int64_t *d_count, const float *src,
+                                 const uint8_t *mask, const twg_iter_t *it,
+                                 twg_stream_t stream) {
+  return masked_select_on_own_array(out, d_count, src, 4, mask, it, stream, /*allow_alloc=*/false);
 }
 
 int twg_masked_select_f32_wait_probe(float *out, int64_t *d_count, const float *src,

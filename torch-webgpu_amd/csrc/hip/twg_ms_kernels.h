@@ -21,7 +21,7 @@
 //     three 64-wide ballots of the lane counts plus mbcnt give each lane its offset, the
 //     values are compacted in LDS at the phase they will have in memory and written
 //     as aligned float4s.
-// A status word packs {flag:2, value:62} so one relaxed agent-scope 64-bit
+// A status word packs {flag:2, epoch:20, value:42} so one relaxed agent-scope 64-bit
 // load/store carries everything; no fences are needed because no other memory
 // is communicated between tiles.
 //
@@ -97,7 +97,24 @@ constexpr uint64_t kFlagShift = 62;
 constexpr uint64_t kFlagAggregate = 1ull << kFlagShift;
 constexpr uint64_t kFlagInclusive = 2ull << kFlagShift;
 constexpr uint64_t kFlagBroken = 3ull << kFlagShift;  // inclusive, but the value is not to be used
-constexpr uint64_t kValueMask = (1ull << kFlagShift) - 1;
+// Below the flag, 20 bits name the launch the word belongs to (its epoch) and 42 bits hold the
+// value.  A word of another epoch reads as not yet published, so a scratch that only this
+// library's launches write (the array behind twg_masked_select_f32_static) needs no clearing
+// between launches: each launch gets the next epoch, and its tiles are counted from the value
+// the ticket counter had when it started (MsRun::ticket_base).  A scratch of the caller's is
+// cleared by every launch and runs at epoch 0, ticket base 0.
+constexpr uint64_t kEpochShift = 42;
+constexpr uint32_t kEpochLimit = 1u << 20;  // epochs are 1 .. kEpochLimit - 1, then the array is cleared
+constexpr uint64_t kEpochMask = (uint64_t)(kEpochLimit - 1) << kEpochShift;
+constexpr uint64_t kValueMask = (1ull << kEpochShift) - 1;
+constexpr int64_t kMsMaxNumel = (int64_t)1 << 41;  // counts must fit the value field
+
+// What a launch knows about its scratch and its waits.
+struct MsRun {
+  uint32_t max_rounds;   // polling rounds after which a look-back gives up
+  uint32_t epoch;        // 0 with a cleared scratch
+  uint32_t ticket_base;  // value of the ticket counter when the launch starts
+};
 
 struct MsGeom {
   int32_t ndim;
@@ -155,7 +172,7 @@ __device__ __forceinline__ void wave_offsets(uint32_t c, uint32_t &below, uint32
 // inclusive word is marked BROKEN.
 template <int LPL, int STRIDE>
 __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t tile, int lane,
-                                             uint32_t max_rounds) {
+                                             uint32_t max_rounds, uint64_t ep) {
   int64_t exclusive = 0;
   int64_t look = (int64_t)tile - 1 - lane;  // lane's nearest candidate
   uint32_t rounds = 0;
@@ -167,8 +184,9 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
       for (int q = 0; q < LPL; ++q) {
         const int64_t idx = look - 64 * q;
         // slots before tile 0 behave like an inclusive prefix of 0
-        st[q] = (idx >= 0) ? status_load(status + idx * STRIDE) : kFlagInclusive;
-        pending |= (st[q] >> kFlagShift) == 0;
+        st[q] = (idx >= 0) ? status_load(status + idx * STRIDE) : (kFlagInclusive | ep);
+        // (a word left by an earlier launch on this scratch has not been published yet)
+        pending |= (st[q] >> kFlagShift) == 0 || (st[q] & kEpochMask) != ep;
       }
       if (__ballot(pending) == 0) break;
       if (++rounds >= max_rounds) return -1;  // wavefront-uniform
@@ -206,22 +224,23 @@ __device__ __forceinline__ int64_t look_back(const uint64_t *status, uint32_t ti
 template <int LPL = kLookPerLane, int STRIDE = 1>
 __device__ __forceinline__ int64_t tile_prefix(uint64_t *status, uint32_t *hdr, uint32_t tile,
                                                uint32_t ntiles, uint32_t tile_total, int64_t room,
-                                               uint32_t max_rounds, int64_t *d_count,
+                                               const MsRun &run, int64_t *d_count,
                                                int64_t *s_slot) {
   const int lane = threadIdx.x & 63;
+  const uint64_t ep = (uint64_t)run.epoch << kEpochShift;
   if (threadIdx.x < 64) {  // wave 0
     uint64_t *mine = status + (size_t)tile * STRIDE;
     if (lane == 0)
-      status_store(mine, (tile == 0 ? kFlagInclusive : kFlagAggregate) | (uint64_t)tile_total);
+      status_store(mine, (tile == 0 ? kFlagInclusive : kFlagAggregate) | ep | (uint64_t)tile_total);
     int64_t exclusive = 0;
     if (tile != 0) {
-      exclusive = look_back<LPL, STRIDE>(status, tile, lane, max_rounds);
+      exclusive = look_back<LPL, STRIDE>(status, tile, lane, run.max_rounds, ep);
       if (exclusive >= 0 && exclusive + (int64_t)tile_total > room) exclusive = -1;
       if (lane == 0) {
         if (exclusive >= 0) {
-          status_store(mine, kFlagInclusive | (uint64_t)(exclusive + tile_total));
+          status_store(mine, kFlagInclusive | ep | (uint64_t)(exclusive + tile_total));
         } else {
-          status_store(mine, kFlagBroken);
+          status_store(mine, kFlagBroken | ep);
           __hip_atomic_store(hdr + kMsErrorWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
@@ -347,8 +366,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
                                                                 const T *src,
                                                                 const uint8_t *mask, int64_t n,
                                                                 uint32_t ntiles, uint32_t *ticket,
-                                                                uint64_t *status,
-                                                                uint32_t max_rounds) {
+                                                                uint64_t *status, MsRun launch) {
   constexpr uint32_t kWaveSpan = 256u * 8u * GROUPS;
   constexpr int64_t kTileElems = (int64_t)kWaveSpan * WAVES;
   constexpr uint32_t kLine = 128u / sizeof(T);  // elements per 128-byte line
@@ -359,7 +377,8 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
   if (threadIdx.x == 0)
-    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh.tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
+              launch.ticket_base;
   __syncthreads();
   const uint32_t tile = sh.tile;
   if (tile >= ntiles) return;  // workgroup-uniform; only with a ticket counter that is not ours alone
@@ -435,7 +454,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_stream(T *out, int64_t 
     for (int k = 0; k < kDepth; ++k) vals[k] = fetch((b_cur >> (4 * k)) & 0xFu, k);
   }
   const int64_t base = tile_prefix<kStreamLookPerLane, kStreamStatusStride>(
-      status, ticket, tile, ntiles, tile_total, n, max_rounds, d_count, &sh.base);
+      status, ticket, tile, ntiles, tile_total, n, launch, d_count, &sh.base);
   if (base < 0) return;  // workgroup-uniform: the look-back was abandoned
 
   // ---- 3a. a wavefront with few selected elements gathers them one element per lane:
@@ -560,7 +579,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
                                                              const T *src,
                                                              const uint8_t *mask, int64_t n,
                                                              uint32_t ntiles, uint32_t *ticket,
-                                                             uint64_t *status, uint32_t max_rounds) {
+                                                             uint64_t *status, MsRun launch) {
   constexpr int64_t kTileElems = (int64_t)kWaveElems * WAVES;
   constexpr uint32_t kSlot = 16u / sizeof(T);  // elements per 16-byte store
   __shared__ MsShared<WAVES, T> sh;
@@ -570,7 +589,8 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
   if (threadIdx.x == 0)
     sh.tile = ntiles == 1
                   ? 0u
-                  : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                  : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
+                        launch.ticket_base;
   __syncthreads();
   const uint32_t tile = sh.tile;
   if (tile >= ntiles) return;  // workgroup-uniform; only with a ticket counter that is not ours alone
@@ -622,7 +642,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
       }
     }
   }
-  const int64_t base = tile_prefix(status, ticket, tile, ntiles, tile_total, n, max_rounds, d_count,
+  const int64_t base = tile_prefix(status, ticket, tile, ntiles, tile_total, n, launch, d_count,
                                    &sh.base);
   if (base < 0) return;  // workgroup-uniform: the look-back was abandoned
 
@@ -674,7 +694,7 @@ __global__ __launch_bounds__(WAVES * 64) void ms_compact_vec(T *out, int64_t *d_
 template <bool STRIDED, typename T>
 __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
     T *out, int64_t *d_count, const T *src, const uint8_t *mask, int64_t n,
-    uint32_t ntiles, uint32_t *ticket, uint64_t *status, uint32_t max_rounds, MsGeom g) {
+    uint32_t ntiles, uint32_t *ticket, uint64_t *status, MsRun launch, MsGeom g) {
   constexpr int kWaveSpan = 64 * kScalarSteps;
   constexpr int kTileElems = kWaveSpan * kScalarWaves;
 
@@ -687,7 +707,8 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
   if (threadIdx.x == 0)
     s_tile = ntiles == 1
                  ? 0u
-                 : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                 : __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
+                       launch.ticket_base;
   __syncthreads();
   const uint32_t tile = s_tile;
   if (tile >= ntiles) return;  // workgroup-uniform; only with a ticket counter that is not ours alone
@@ -736,7 +757,7 @@ __global__ __launch_bounds__(kScalarWaves * 64) void ms_compact_scalar(
 #pragma unroll
   for (int k = 0; k < kScalarSteps; ++k)
     if (sel[k]) vals[k] = src[soff[k]];
-  const int64_t base = tile_prefix(status, ticket, tile, ntiles, tile_total, n, max_rounds, d_count,
+  const int64_t base = tile_prefix(status, ticket, tile, ntiles, tile_total, n, launch, d_count,
                                    &s_base);
   if (base < 0) return;  // workgroup-uniform: the look-back was abandoned
   const int64_t wpos = base + wave_base;

@@ -958,8 +958,13 @@ int twg_masked_select_count(void *out, int64_t *count_host, const void *src, int
   constexpr int64_t kPending = INT64_MIN;
   int64_t *slot = reinterpret_cast<int64_t *>(st.box(mb));
   __atomic_store_n(slot, kPending, __ATOMIC_RELEASE);
-  rc = masked_select_launch(out, reinterpret_cast<int64_t *>(st.box_dev(mb)), src, elem_size, mask,
-                            it, scratch, scratch_bytes, stream);
+  // no scratch of the caller's: the array the library keeps for this
+  if (!scratch && scratch_bytes == 0)
+    rc = masked_select_on_own_array(out, reinterpret_cast<int64_t *>(st.box_dev(mb)), src, elem_size,
+                                    mask, it, stream, /*allow_alloc=*/true);
+  else
+    rc = masked_select_launch(out, reinterpret_cast<int64_t *>(st.box_dev(mb)), src, elem_size, mask,
+                              it, scratch, scratch_bytes, stream);
   int64_t k = kPending;
   if (rc == 0 && it->numel != 0) {  // an empty input clears the count bytewise: wait for the stream
     for (int i = 0; i < kMailboxSpins && k == kPending; ++i) {

@@ -344,16 +344,27 @@ at::Tensor masked_select_impl(const at::Tensor &self, const at::Tensor &mask, at
 
   twg_iter_t it;
   fill_iter_logical(se, me, &it);
-  const size_t scratch_bytes = twg_masked_select_scratch_bytes(n);
-  at::Tensor work = at::empty({(int64_t)scratch_bytes}, self.options().dtype(at::kByte));
   const bool direct = into.defined() && into.is_contiguous() && into.numel() >= n;
   at::Tensor out = direct ? into : at::empty({n}, self.options());
   // The output shape depends on the data: waiting for the count is the op's one sync
   // point.  The kernel hands it over through pinned memory as soon as it is known.
+  // Tickets and status words live in the array the library keeps for this (no scratch to
+  // allocate, none to clear); an input beyond its limit, or a call while another stream's
+  // launch still uses it, brings its own scratch.
   int64_t k = 0;
-  TWG_CHECK(twg_masked_select_count(out.data_ptr(), &k, se.const_data_ptr(), (int32_t)esize,
-                                    static_cast<const uint8_t *>(me.const_data_ptr()), &it,
-                                    work.data_ptr(), scratch_bytes, nullptr));
+  int rc = n <= TWG_MS_STATIC_MAX_NUMEL
+               ? twg_masked_select_count(out.data_ptr(), &k, se.const_data_ptr(), (int32_t)esize,
+                                         static_cast<const uint8_t *>(me.const_data_ptr()), &it,
+                                         nullptr, 0, nullptr)
+               : TWG_E_TOO_LARGE;
+  if (rc == TWG_E_TOO_LARGE || rc == TWG_E_BUSY) {
+    const size_t scratch_bytes = twg_masked_select_scratch_bytes(n);
+    at::Tensor work = at::empty({(int64_t)scratch_bytes}, self.options().dtype(at::kByte));
+    rc = twg_masked_select_count(out.data_ptr(), &k, se.const_data_ptr(), (int32_t)esize,
+                                 static_cast<const uint8_t *>(me.const_data_ptr()), &it,
+                                 work.data_ptr(), scratch_bytes, nullptr);
+  }
+  TWG_CHECK(rc);
   TORCH_CHECK(k >= 0 && k <= n, "webgpu masked_select: implausible count ", k);
   if (direct) {
     out.resize_({k});  // shrinking keeps the storage
