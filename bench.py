@@ -602,7 +602,10 @@ def geometry_families(capi, L):
     # in rotation; kernels whose loads carry the nontemporal hint read the same either way).
     kSets = 3
 
+    launches = [0]  # patterns timed so far: a kernel trace of this sweep tells them apart by it
+
     def median_launch_seconds(run):
+        launches[0] += 1
         for i in range(kSets):
             run(i)
         capi.sync()
@@ -645,7 +648,7 @@ def geometry_families(capi, L):
             for s in bshape:
                 nb *= s
             pct, ms = timed(shape, contig(shape), b_st, nb)
-            rows_.append({"pct_hbm_peak": pct, "ms": ms, "a": shape, "b": bshape})
+            rows_.append({"pct_hbm_peak": pct, "ms": ms, "a": shape, "b": bshape, "launch_order": launches[0]})
     rows_.sort(key=lambda r: r["pct_hbm_peak"])
     fam["broadcast_second_operand"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
                                        "slowest": rows_[:5], "all": rows_}
@@ -666,7 +669,8 @@ def geometry_families(capi, L):
             for pos, p in enumerate(perm):
                 a_st[p] = phys[pos]
             pct, ms = timed(shape, a_st, contig(shape), n)
-            rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "a_memory_order": list(perm)})
+            rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "a_memory_order": list(perm),
+                          "launch_order": launches[0]})
     rows_.sort(key=lambda r: r["pct_hbm_peak"])
     fam["permuted_first_operand"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
                                      "slowest": rows_[:5], "all": rows_}
@@ -720,7 +724,7 @@ def geometry_families(capi, L):
             for both in (False, True):
                 pct, ms = timed_view(shape, storage, starts, steps, both)
                 rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "slice": what,
-                              "operands_sliced": "both" if both else "first"})
+                              "operands_sliced": "both" if both else "first", "launch_order": launches[0]})
     rows_.sort(key=lambda r: r["pct_hbm_peak"])
     fam["sliced_operands"] = {"patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"],
                               "slowest": rows_[:5], "all": rows_}
@@ -728,6 +732,7 @@ def geometry_families(capi, L):
         f"slowest {rows_[0]['pct_hbm_peak']}%")
     return {"geometry_families": fam, "elements_per_pattern": "about 2^25", "op": "add.Tensor fp32",
             "operand_sets_in_rotation": kSets,
+            "launches_per_pattern": kSets + 3 * 12,
             "bytes": "4 B per element read per full operand + 4 B written; a broadcast operand counts its own size; "
                      "a stepped operand counts the elements used, not the lines touched"}
 
