@@ -119,6 +119,40 @@ def test_static_scratch_is_not_cleared_between_calls(twg):
         assert k == int(m.sum()) and torch.equal(vals, torch.masked_select(x, m)), dtype
 
 
+def test_library_array_from_two_host_threads(twg):
+    # Two host threads call into the array at once (ctypes drops the GIL for the call): the
+    # epoch and ticket bookkeeping is taken under the array's lock together with the launch, so
+    # every call still sees its own count and values.
+    import threading
+    L = twg.load()
+    errors = []
+
+    def worker(seed):
+        try:
+            g = torch.Generator().manual_seed(seed)
+            for i in range(12):
+                n = (70001, (1 << 21) + 3, 9000, 300000)[i % 4] + seed
+                src, mask = torch.rand(n, generator=g), torch.rand(n, generator=g) < (0.2 + 0.05 * i)
+                d_src, d_mask = twg.to_device(src), twg.to_device(mask)
+                out = twg.DeviceBuffer(4 * n + 256)
+                it = twg.dense_iter(n)
+                kh = ctypes.c_int64(-7)
+                twg.check(L.twg_masked_select_count(out.ptr, ctypes.byref(kh), d_src.ptr, 4, d_mask.ptr,
+                                                    ctypes.byref(it), None, 0, None))
+                if kh.value != int(mask.sum()) or not torch.equal(out.download((kh.value,), torch.float32), src[mask]):
+                    errors.append((seed, i, n, kh.value))
+        except Exception as e:  # noqa: BLE001 - reported below, in the test's thread
+            errors.append((seed, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in (1, 2)]
+    print("library array: two host threads", flush=True)
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_static_scratch_is_refused_to_a_second_stream_while_in_use(twg):
     # One array per GPU: a call on another stream while the previous call's kernels may still
     # be running must be refused (TWG_E_BUSY), not left to corrupt the tickets; once that work
