@@ -394,6 +394,26 @@ def test_add_permuted_operand_tiles(twg, shape, order):
             assert torch.equal(H.binary("twg_eq_f32", br, ar, out_dtype=torch.bool), torch.eq(br, ar))
 
 
+def test_fill_bytes_every_size_class(twg):
+    # twg_fill_bytes: an unaligned head, a body of 16-byte packs and a tail.  From 16 MiB on the
+    # body goes out in whole blocks of 4 KiB without a test per store, and what the last
+    # whole block leaves over goes to the kernel for small fills: sizes on both sides of the
+    # switch, at odd offsets, must set exactly their bytes.
+    L = twg.load()
+    mib = 1 << 20
+    buf = twg.DeviceBuffer(49 * mib + 64)
+    for nb in (0, 1, 15, 16, 17, 4097, 16 * mib - 1, 16 * mib, 16 * mib + 1, 16 * mib + 15,
+               16 * mib + 4096 + 5, 16 * mib + 4080, 48 * mib + 1234567):
+        for off in (0, 1, 7, 16):
+            _say(f"fill {nb} bytes at offset {off}")
+            twg.check(L.twg_fill_bytes(buf.ptr, 0xEE, buf.nbytes, None))
+            twg.check(L.twg_fill_bytes(buf.ptr + off, 0x5A, nb, None))
+            raw = buf.download((buf.nbytes,), torch.uint8)
+            assert bool((raw[:off] == 0xEE).all()), (nb, off)
+            assert bool((raw[off:off + nb] == 0x5A).all()), (nb, off)
+            assert bool((raw[off + nb:] == 0xEE).all()), (nb, off)
+
+
 @pytest.mark.parametrize("rows,cols", [(8, 64), (37, 128), (5, 4096), (16, 36), (3, 260), (64, 32), (2, 12288)])
 def test_rows_stepped_by_two_and_three(twg, rows, cols):
     # x[:, ::2]: a lane fetches the two aligned packs that hold its four elements and keeps
