@@ -1065,6 +1065,44 @@ def test_compare_ieee_cases_and_layouts(twg):
                              extra=(ctypes.c_int32(1),)), M.t().contiguous())
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.float32, torch.int64, torch.float64])
+def test_copy_strided_every_element_size_and_layout(twg, dtype):
+    # twg_copy_strided moves elements of 1, 2, 4 and 8 bytes without looking at them.  8-byte
+    # elements travel as pairs of 4-byte words (one more innermost dimension) through the same
+    # kernels as float32, so every layout class is checked for every size: transposed, permuted
+    # with short and long innermost extents, channels-last pixels, sliced and stepped rows,
+    # broadcast, sliced outputs, and an 8-dimensional view that leaves no room for the extra
+    # dimension.
+    g = torch.Generator().manual_seed(42 + dtype.itemsize)
+    es = ctypes.c_int32(dtype.itemsize)
+
+    def rnd(*shape):
+        return (torch.randn(*shape, generator=g) * 1000).to(dtype)
+
+    def check(view, out=None, what=""):
+        _say(f"copy_strided {dtype} {what} {tuple(view.shape)} strides {view.stride()}")
+        got = H.unary("twg_copy_strided", view, out=out, out_dtype=dtype, extra=(es,))
+        assert torch.equal(got, view.contiguous() if out is None else view), (dtype, what)
+
+    check(rnd(300, 200).t(), what="transposed")
+    check(rnd(1027, 260).t(), what="transposed, ragged")
+    check(rnd(4, 30, 40, 3).permute(0, 3, 1, 2), what="NHWC viewed as NCHW")
+    check(rnd(4, 3, 30, 40).permute(0, 2, 3, 1), what="NCHW viewed as NHWC")
+    check(rnd(5, 33, 35, 4).permute(0, 2, 1, 3), what="pixels, h and w swapped")
+    check(rnd(6, 17, 64, 70).permute(3, 1, 0, 2), what="permuted")
+    check(rnd(2, 96, 56, 56).permute(0, 2, 3, 1), what="permuted, 96 channels")
+    check(rnd(37, 1001)[:, 1:], what="rows from 1 on")
+    check(rnd(50, 2048)[:, ::2], what="stepped rows")
+    check(rnd(1, 700).expand(90, 700), what="broadcast rows")
+    check(rnd(90, 1).expand(90, 700), what="one value per row")
+    check(rnd(64, 128), out=torch.zeros(128, 64, dtype=dtype).t(), what="transposed output")
+    check(rnd(40, 300), out=torch.zeros(40, 601, dtype=dtype)[:, 1::2], what="stepped output")
+    x8 = rnd(2, 3, 2, 2, 3, 2, 2, 6)[:, ::2, :, :, ::2]
+    check(x8.permute(7, 6, 5, 4, 3, 2, 1, 0), what="8 dimensions, reversed")
+    check(rnd(70001)[1:], what="one dimension from 1 on")
+    check(rnd((1 << 20) + 3), what="dense")
+
+
 # ----------------------------------------------------------- masked_select
 
 @pytest.mark.parametrize("p", [0.0, 0.01, 0.5, 0.99, 1.0])
