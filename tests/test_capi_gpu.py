@@ -1085,6 +1085,17 @@ def test_copy_strided_every_element_size_and_layout(twg, dtype):
         assert torch.equal(got, view.contiguous() if out is None else view), (dtype, what)
 
     check(rnd(300, 200).t(), what="transposed")
+    # extents and strides that are multiples of 16 elements: 1- and 2-byte elements take the tile
+    # kernel with 16-byte packs on both sides (whole tiles, ragged tiles, a batch, an offset
+    # that keeps the alignment and one that breaks it)
+    check(rnd(320, 256).t(), what="transposed, whole packs")
+    check(rnd(1088, 544).t(), what="transposed, ragged tiles")
+    check(rnd(3, 160, 96).transpose(1, 2), what="batched transposes")
+    check(rnd(4, 32, 48, 64).permute(0, 3, 1, 2), what="NHWC viewed as NCHW, whole packs")
+    check(rnd(2, 64, 48, 32).permute(3, 1, 0, 2), what="permuted, whole packs")
+    check(rnd(16 + 320 * 256)[16:].view(320, 256).t(), what="transposed, storage offset of 16")
+    check(rnd(3 + 320 * 256)[3:].view(320, 256).t(), what="transposed, storage offset of 3")
+    check(rnd(256, 512).t(), out=torch.zeros(512, 512, dtype=dtype)[:, :256], what="transposed into a wider output")
     check(rnd(1027, 260).t(), what="transposed, ragged")
     check(rnd(4, 30, 40, 3).permute(0, 3, 1, 2), what="NHWC viewed as NCHW")
     check(rnd(4, 3, 30, 40).permute(0, 2, 3, 1), what="NCHW viewed as NHWC")

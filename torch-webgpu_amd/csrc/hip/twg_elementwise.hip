@@ -126,6 +126,17 @@ int twg_unary_f32(int op, float *out, const float *in, const twg_iter_t *it, twg
 
 int twg_copy_strided(void *out, const void *in, int32_t elem_size, const twg_iter_t *it,
                      twg_stream_t stream) {
+  // transposing copies of 1- and 2-byte elements have a tile kernel of their own
+  if ((elem_size == 1 || elem_size == 2) && out && in) {
+    Geom g;
+    int rc = ensure_init();
+    if (rc) return rc;
+    if ((rc = canonicalize(it, 2, &g))) return rc;
+    if (g.numel >= 4096) {
+      rc = launch_tile_narrow(out, in, elem_size, g, resolve_stream(stream));
+      if (rc != TWG_E_UNSUPPORTED) return rc;
+    }
+  }
   switch (elem_size) {
     case 1:
       return launch_ew<1, CopyOp<uint8_t>, uint8_t, uint8_t, uint8_t>(

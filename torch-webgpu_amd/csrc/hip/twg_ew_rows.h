@@ -275,8 +275,13 @@ int launch_generic_vec(TO *out, const TA *a, const TB *b, const Geom &g, Op op, 
     // its chunks where the rows start, the flat walk does neither (rows of 1000 floats with a
     // [16, 1, 1000] operand: 75% -> 80% of peak, [128, 64, 56*56] + [128, 1, 56*56]: 74% -> 77%).
     if (g.shape[0] >= 256 && (g.shape[0] % (64 * VEC) == 0 || g.shape[0] >= 8192)) return TWG_E_UNSUPPORTED;
-    // rows of less than a cache line gain nothing over one element per lane (measured)
-    if (g.shape[0] * (int64_t)MaxSize<TO, TA, TB>::value < 128) return TWG_E_UNSUPPORTED;
+    // rows of less than a cache line gain nothing over one element per lane (measured with
+    // 4-byte elements; 1- and 2-byte elements, where a lane would move as little as a byte, gain
+    // from one pack per row on: 64-byte rows of bools 6% -> 54% of peak, 32-byte rows 32%)
+    {
+      constexpr int64_t kSize = MaxSize<TO, TA, TB>::value;
+      if (g.shape[0] * kSize < (kSize >= 4 ? 128 : 16)) return TWG_E_UNSUPPORTED;
+    }
     if constexpr (NIN == 1) {
       if (sa0 == 0) return TWG_E_UNSUPPORTED;
     }

@@ -1228,5 +1228,135 @@ int launch_pix(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t
   }
 }
 
+// ------------------------------------------------------- ew_tile_narrow
+// Transposing copies of 1- and 2-byte elements (bool masks, half and bfloat16 tensors) with
+// 16-byte accesses on both sides.  One element per lane and instruction (ew_tile) moves as
+// many elements per second as the float32 tile kernel moves, which for these widths is a
+// quarter or half of its bytes.  Here a tile of TD0 x TT elements is read as 16-byte packs
+// along t, the input's unit-stride dimension, and parked in LDS as it lies in memory; each
+// lane then gathers the 8 or 16 elements of one output pack (consecutive along dimension 0,
+// one LDS row apart) with narrow LDS reads and stores 16 bytes.  The 64 lanes of a store cover
+// 8 output rows x 128 bytes, whole lines.  A row pitch of an odd number of words keeps the
+// gathers free of bank conflicts for 2-byte elements (two lanes per bank for 1-byte ones).
+// Offsets and strides are in elements.  Every pack must be aligned: the launcher checks.
+template <int ES, int TD0, int TT>
+__global__ __launch_bounds__(kThreads) void ew_tile_narrow(unsigned char *out, const unsigned char *in,
+                                                           TileGeom g) {
+  static_assert(ES == 1 || ES == 2, "1- and 2-byte elements");
+  constexpr int EPP = 16 / ES;             // elements per pack
+  constexpr int kRowWords = TT * ES / 4;   // a tile row of the input, in words
+  constexpr int kPitch = kRowWords + 1;    // odd
+  constexpr int kPacksT = TT / EPP, kPacks0 = TD0 / EPP;
+  static_assert(kRowWords % 4 == 0 && TT % 8 == 0 && TD0 % EPP == 0 && kPacks0 >= 8, "tile shape");
+  typedef uint32_t Words __attribute__((ext_vector_type(4)));
+  using Elem = typename std::conditional<ES == 1, uint8_t, uint16_t>::type;
+  __shared__ uint32_t lds[TD0 * kPitch];
+
+  uint32_t t0i, tti;
+  int64_t off_o, off_a, off_b;
+  tile_of_block<false, 1>(g, blockIdx.x, t0i, tti, off_o, off_a, off_b);
+  const int64_t base0 = (int64_t)t0i * TD0, baset = (int64_t)tti * TT;
+
+  // the input's rows (one per index of dimension 0), packs along t
+  constexpr int kIn = TD0 * kPacksT / kThreads;
+  static_assert(TD0 * kPacksT % kThreads == 0, "tile shape");
+  Words v[kIn];
+#pragma unroll
+  for (int u = 0; u < kIn; ++u) {
+    const int i = threadIdx.x + u * kThreads;
+    const int r = i / kPacksT, p = i - r * kPacksT;
+    const int64_t d0 = base0 + r, tt = baset + (int64_t)p * EPP;
+    if (d0 < g.n0 && tt < g.nt)
+      v[u] = __builtin_nontemporal_load(
+          reinterpret_cast<const Words *>(in + (off_a + d0 * g.s0[1] + tt) * ES));
+  }
+#pragma unroll
+  for (int u = 0; u < kIn; ++u) {
+    const int i = threadIdx.x + u * kThreads;
+    const int r = i / kPacksT, p = i - r * kPacksT;
+    uint32_t *dst = lds + r * kPitch + p * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) dst[c] = v[u][c];  // (rows and packs outside the extents are never read)
+  }
+  __syncthreads();
+
+  // the output's rows (one per index of t), packs along dimension 0: lane -> (row within a
+  // group of 8, pack), so that a store instruction writes 8 rows x 8 packs
+  const Elem *cells = reinterpret_cast<const Elem *>(lds);
+  constexpr int kCellPitch = kPitch * 4 / ES;  // elements between two LDS rows
+  constexpr int kOut = TT * kPacks0 / kThreads;
+  static_assert(TT * kPacks0 % kThreads == 0, "tile shape");
+#pragma unroll
+  for (int u = 0; u < kOut; ++u) {
+    const int i = threadIdx.x + u * kThreads;
+    const int ts = i & 7, dpk = (i >> 3) % kPacks0, trow = (i >> 3) / kPacks0 * 8 + ts;
+    const int64_t d0 = base0 + (int64_t)dpk * EPP, tt = baset + trow;
+    if (d0 >= g.n0 || tt >= g.nt) continue;
+    const Elem *col = cells + (dpk * EPP) * kCellPitch + trow;
+    Words w;
+    if constexpr (ES == 2) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        w[c] = (uint32_t)col[(2 * c) * kCellPitch] | ((uint32_t)col[(2 * c + 1) * kCellPitch] << 16);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        w[c] = (uint32_t)col[(4 * c) * kCellPitch] | ((uint32_t)col[(4 * c + 1) * kCellPitch] << 8) |
+               ((uint32_t)col[(4 * c + 2) * kCellPitch] << 16) | ((uint32_t)col[(4 * c + 3) * kCellPitch] << 24);
+    }
+    __builtin_nontemporal_store(w, reinterpret_cast<Words *>(out + (off_o + tt * g.st[0] + d0) * ES));
+  }
+}
+
+// A copy whose input has its unit stride along dimension t >= 1 while the output has it along
+// dimension 0, elements of 1 or 2 bytes.  Returns TWG_E_UNSUPPORTED unless every 16-byte pack of
+// both sides is aligned (pointers, extents of the two dimensions, every other stride).
+inline int launch_tile_narrow(void *out, const void *in, int es, const Geom &g, hipStream_t s) {
+  if ((es != 1 && es != 2) || g.ndim < 2 || g.stride[0][0] != 1 || g.stride[1][0] == 1)
+    return TWG_E_UNSUPPORTED;
+  int t = -1;
+  for (int d = 1; d < g.ndim && t < 0; ++d)
+    if (g.stride[1][d] == 1) t = d;
+  if (t < 0) return TWG_E_UNSUPPORTED;
+  const int64_t epp = 16 / es;
+  if (!aligned_to(out, 16) || !aligned_to(in, 16) || g.shape[0] % epp || g.shape[t] % epp)
+    return TWG_E_UNSUPPORTED;
+  if (g.shape[0] < 32 || g.shape[t] < 32) return TWG_E_UNSUPPORTED;  // (tiles mostly empty)
+  for (int d = 0; d < g.ndim; ++d) {
+    if (d != 0 && g.stride[0][d] % epp) return TWG_E_UNSUPPORTED;
+    if (d != t && g.stride[1][d] % epp) return TWG_E_UNSUPPORTED;
+  }
+  TileGeom tg{};
+  tg.n0 = g.shape[0];
+  tg.nt = g.shape[t];
+  tg.psplit = 1;
+  for (int o = 0; o < 2; ++o) {
+    tg.s0[o] = g.stride[o][0];
+    tg.st[o] = g.stride[o][t];
+  }
+  int64_t batch = 1;
+  for (int d = 1; d < g.ndim; ++d) {
+    if (d == t) continue;
+    tg.bshape[tg.nbatch] = g.shape[d];
+    for (int o = 0; o < 2; ++o) tg.bstride[o][tg.nbatch] = g.stride[o][d];
+    tg.nbatch++;
+    batch *= g.shape[d];
+  }
+  constexpr int kTd0 = 128;
+  const int tt = es == 2 ? 64 : 128;
+  const int64_t tiles0 = (tg.n0 + kTd0 - 1) / kTd0, tilest = (tg.nt + tt - 1) / tt;
+  const int64_t blocks = tile_grid(tiles0, tilest, batch, false, &tg.ngroups);
+  if (blocks == 0) return TWG_E_UNSUPPORTED;
+  tg.tiles0 = (uint32_t)tiles0;
+  tg.tilest = (uint32_t)tilest;
+  if (es == 2)
+    ew_tile_narrow<2, kTd0, 64><<<(unsigned)blocks, kThreads, 0, s>>>(
+        static_cast<unsigned char *>(out), static_cast<const unsigned char *>(in), tg);
+  else
+    ew_tile_narrow<1, kTd0, 128><<<(unsigned)blocks, kThreads, 0, s>>>(
+        static_cast<unsigned char *>(out), static_cast<const unsigned char *>(in), tg);
+  return (int)hipGetLastError();
+}
+
 }  // namespace
 }  // namespace twg
