@@ -12,12 +12,16 @@
 //   twg_ew_rows.h   ew_rows    - inner dimension unit-stride (or broadcast) for every operand,
 //                                outer dimensions arbitrary (row bias, column bias, slices)
 //                   ew_generic_vec - short or ragged rows: a flat walk over packs, div/mod per pack
+//                   ew_stepped_vec - the same walk for inputs stepped by 2 along their rows
 //                   ew_generic - anything else, one element per lane, div/mod index math with
 //                                dimension 0 fastest
 //   twg_ew_tile.h   ew_tile, ew_tile_vec, ew_tile_any - an input whose unit stride lies along
 //                                another dimension than the output's: tiles staged through LDS so
 //                                that both sides of the transpose stay coalesced
-//                   ew_deint   - an input stored [.., x, c] with a short c against [.., c, x]
+//                   ew_tile_narrow - the same for copies of 1- and 2-byte elements
+//   twg_ew_strips.h ew_deint   - an input stored [.., x, c] with a short c against [.., c, x]
+//                   ew_inter   - its mirror image: a planar input against an output [.., x, c]
+//                   ew_pix     - a short c innermost everywhere, two outer dimensions swapped
 // This file: launch_ew, which canonicalizes the caller's geometry and picks the kernel.
 //
 // Replaces the two WGSL templates of the reference and their host drivers:
@@ -29,6 +33,7 @@
 #include "twg_ew_dense.h"
 #include "twg_ew_rows.h"
 #include "twg_ew_tile.h"
+#include "twg_ew_strips.h"
 
 namespace twg {
 namespace {
