@@ -1096,6 +1096,10 @@ def test_copy_strided_every_element_size_and_layout(twg, dtype):
     check(rnd(16 + 320 * 256)[16:].view(320, 256).t(), what="transposed, storage offset of 16")
     check(rnd(3 + 320 * 256)[3:].view(320, 256).t(), what="transposed, storage offset of 3")
     check(rnd(256, 512).t(), out=torch.zeros(512, 512, dtype=dtype)[:, :256], what="transposed into a wider output")
+    if dtype == torch.uint8:  # from 2^26 elements on, 1-byte elements take wider tiles
+        big = torch.randint(0, 256, (8192 + 144, 8192), generator=g, dtype=torch.uint8)
+        check(big.t(), what="transposed, 2^26 elements and a ragged last tile")
+        del big
     check(rnd(1027, 260).t(), what="transposed, ragged")
     check(rnd(4, 30, 40, 3).permute(0, 3, 1, 2), what="NHWC viewed as NCHW")
     check(rnd(4, 3, 30, 40).permute(0, 2, 3, 1), what="NCHW viewed as NHWC")
