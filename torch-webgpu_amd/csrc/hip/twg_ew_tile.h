@@ -542,8 +542,8 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
 }
 
 // ------------------------------------------------------- ew_tile_narrow
-// Transposing copies of 1- and 2-byte elements (bool masks, half and bfloat16 tensors) with
-// 16-byte accesses on both sides.  One element per lane and instruction (ew_tile) moves as
+// Transposing copies of 1-, 2- and 8-byte elements (bool masks, half and bfloat16 tensors,
+// int64 and float64) with 16-byte accesses on both sides.  One element per lane and instruction (ew_tile) moves as
 // many elements per second as the float32 tile kernel moves, which for these widths is a
 // quarter or half of its bytes.  Here a tile of TD0 x TT elements is read as 16-byte packs
 // along t, the input's unit-stride dimension, and parked in LDS as it lies in memory; each
@@ -555,14 +555,16 @@ int launch_tile(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_
 template <int ES, int TD0, int TT>
 __global__ __launch_bounds__(kThreads) void ew_tile_narrow(unsigned char *out, const unsigned char *in,
                                                            TileGeom g) {
-  static_assert(ES == 1 || ES == 2, "1- and 2-byte elements");
+  static_assert(ES == 1 || ES == 2 || ES == 8, "1-, 2- and 8-byte elements");
   constexpr int EPP = 16 / ES;             // elements per pack
   constexpr int kRowWords = TT * ES / 4;   // a tile row of the input, in words
-  constexpr int kPitch = kRowWords + 1;    // odd
+  // odd, or for 8-byte elements (which must stay 8-byte aligned) 8 modulo 32: the 8 rows a
+  // store instruction gathers from then start 16 banks apart
+  constexpr int kPitch = kRowWords + (ES == 8 ? 8 : 1);
   constexpr int kPacksT = TT / EPP, kPacks0 = TD0 / EPP;
   static_assert(kRowWords % 4 == 0 && TT % 8 == 0 && TD0 % EPP == 0 && kPacks0 >= 8, "tile shape");
   typedef uint32_t Words __attribute__((ext_vector_type(4)));
-  using Elem = typename std::conditional<ES == 1, uint8_t, uint16_t>::type;
+  using Elem = typename std::conditional<ES == 1, uint8_t, typename std::conditional<ES == 2, uint16_t, uint64_t>::type>::type;
   __shared__ uint32_t lds[TD0 * kPitch];
 
   uint32_t t0i, tti;
@@ -611,6 +613,12 @@ __global__ __launch_bounds__(kThreads) void ew_tile_narrow(unsigned char *out, c
 #pragma unroll
       for (int c = 0; c < 4; ++c)
         w[c] = (uint32_t)col[(2 * c) * kCellPitch] | ((uint32_t)col[(2 * c + 1) * kCellPitch] << 16);
+    } else if constexpr (ES == 8) {
+      const uint64_t e0 = col[0], e1 = col[kCellPitch];
+      w[0] = (uint32_t)e0;
+      w[1] = (uint32_t)(e0 >> 32);
+      w[2] = (uint32_t)e1;
+      w[3] = (uint32_t)(e1 >> 32);
     } else {
 #pragma unroll
       for (int c = 0; c < 4; ++c)
@@ -622,10 +630,10 @@ __global__ __launch_bounds__(kThreads) void ew_tile_narrow(unsigned char *out, c
 }
 
 // A copy whose input has its unit stride along dimension t >= 1 while the output has it along
-// dimension 0, elements of 1 or 2 bytes.  Returns TWG_E_UNSUPPORTED unless every 16-byte pack of
+// dimension 0, elements of 1, 2 or 8 bytes.  Returns TWG_E_UNSUPPORTED unless every 16-byte pack of
 // both sides is aligned (pointers, extents of the two dimensions, every other stride).
 inline int launch_tile_narrow(void *out, const void *in, int es, const Geom &g, hipStream_t s) {
-  if ((es != 1 && es != 2) || g.ndim < 2 || g.stride[0][0] != 1 || g.stride[1][0] == 1)
+  if ((es != 1 && es != 2 && es != 8) || g.ndim < 2 || g.stride[0][0] != 1 || g.stride[1][0] == 1)
     return TWG_E_UNSUPPORTED;
   int t = -1;
   for (int d = 1; d < g.ndim && t < 0; ++d)
@@ -659,8 +667,9 @@ inline int launch_tile_narrow(void *out, const void *in, int es, const Geom &g, 
   // on a transposed [16384, 8192] of 2-byte elements against 55% with 128, 68% against 62% on
   // [128, 56, 56, 96] stored NCHW; 1-byte elements gain from 2^26 elements on (56% against 49%)
   // and lose a point or two below.
+  // (8-byte elements: 64 x 64, runs of 512 bytes on both sides)
   const bool wide = es == 2 || g.numel >= (int64_t(1) << 26);
-  const int td0 = wide ? 256 : 128, tt = es == 2 ? 64 : 128;
+  const int td0 = es == 8 ? 64 : wide ? 256 : 128, tt = es == 1 ? 128 : 64;
   const int64_t tiles0 = (tg.n0 + td0 - 1) / td0, tilest = (tg.nt + tt - 1) / tt;
   const int64_t blocks = tile_grid(tiles0, tilest, batch, false, &tg.ngroups);
   if (blocks == 0) return TWG_E_UNSUPPORTED;
@@ -668,7 +677,9 @@ inline int launch_tile_narrow(void *out, const void *in, int es, const Geom &g, 
   tg.tilest = (uint32_t)tilest;
   unsigned char *o = static_cast<unsigned char *>(out);
   const unsigned char *i = static_cast<const unsigned char *>(in);
-  if (es == 2)
+  if (es == 8)
+    ew_tile_narrow<8, 64, 64><<<(unsigned)blocks, kThreads, 0, s>>>(o, i, tg);
+  else if (es == 2)
     ew_tile_narrow<2, 256, 64><<<(unsigned)blocks, kThreads, 0, s>>>(o, i, tg);
   else if (wide)
     ew_tile_narrow<1, 256, 128><<<(unsigned)blocks, kThreads, 0, s>>>(o, i, tg);
