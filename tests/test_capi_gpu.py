@@ -341,6 +341,8 @@ def test_add_transposed_operand(twg, rows, cols):
     ((4, 30, 40, 3), (0, 3, 1, 2)), ((2, 1000, 3), (0, 2, 1)), ((1027, 4), (1, 0)), ((3, 700, 16), (0, 2, 1)),
     ((2, 301, 31), (0, 2, 1)), ((5000, 2), (1, 0)), ((3, 2051, 7), (0, 2, 1)), ((2, 4099, 24), (0, 2, 1)),
     ((2, 3, 255, 5), (0, 1, 3, 2)), ((2, 2, 260, 8), (1, 0, 3, 2)), ((300, 32), (1, 0)),
+    # 32 to 63 channels take the same strips (32 values of x each)
+    ((2, 301, 33), (0, 2, 1)), ((3, 700, 48), (0, 2, 1)), ((2, 40, 50, 63), (0, 3, 1, 2)), ((1027, 36), (1, 0)),
     # a short x: several strips per block (groups of the next dimension, the last group shorter)
     ((7, 5, 40, 3), (0, 1, 3, 2)), ((3, 11, 100, 2), (0, 1, 3, 2)), ((2, 9, 33, 31), (0, 1, 3, 2)),
     ((2, 23, 56, 3), (1, 0, 3, 2)), ((40, 112, 3), (0, 2, 1)), ((1, 3, 32, 4), (0, 1, 3, 2)),

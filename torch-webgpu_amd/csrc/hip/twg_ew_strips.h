@@ -273,7 +273,7 @@ int launch_deint(TO *out, const TA *a, const TB *b, const Geom &g, int pd, bool 
 
 // ------------------------------------------------------------ ew_inter
 // The mirror of ew_deint: the OUTPUT is laid out [.., x, c] with a short innermost extent c
-// (dimension 0, 2..31 elements; x is dimension 1, output stride c) and an input is stored
+// (dimension 0, 2..63 elements; x is dimension 1, output stride c) and an input is stored
 // planar, [.., c, x] (unit stride along x): NCHW -> NHWC with a few channels, coordinate arrays
 // stacked into points.  A block takes a strip of TX values of x: it reads the planar operands'
 // c runs of TX elements with 16-byte loads straight into LDS (one run per channel, the pitch
@@ -435,7 +435,7 @@ int launch_inter(TO *out, const TA *a, const TB *b, const Geom &g, bool a_p, boo
     if (!out_packs_aligned(out, g, 2)) return TWG_E_UNSUPPORTED;
     if (g.ndim < 2) return TWG_E_UNSUPPORTED;
     const int64_t P = g.shape[0];
-    if (P < 2 || P >= 32 || g.stride[0][0] != 1 || g.stride[0][1] != P) return TWG_E_UNSUPPORTED;
+    if (P < 2 || P >= 64 || g.stride[0][0] != 1 || g.stride[0][1] != P) return TWG_E_UNSUPPORTED;
     auto like_out = [&](int o) { return g.stride[o][0] == 1 && g.stride[o][1] == P; };
     auto planar = [&](int o) { return g.stride[o][1] == 1 && g.stride[o][0] != 0; };
     if (a_p ? !planar(1) : !like_out(1)) return TWG_E_UNSUPPORTED;
