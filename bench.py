@@ -582,7 +582,8 @@ def op_chain(capi, L):
 def geometry_families(capi, L):
     """add.Tensor on ~2^25 fp32 elements with (a) the second operand broadcast in every possible
     way over a set of 2- to 4-dimensional shapes, (b) the first operand stored in every
-    permutation of its dimensions and (c) one or both operands slices of a larger storage.  Reports algorithmic bytes / time as % of the HBM peak: the
+    permutation of its dimensions and (c) one or both operands slices of a larger storage; and
+    (d) copies of permuted tensors of 1-, 2- and 8-byte elements (twg_copy_strided).  Reports algorithmic bytes / time as % of the HBM peak: the
     slowest patterns and the median of each family.  Median of three batches of 12 launches,
     each batch between one pair of events on the library's stream, consecutive launches on
     three sets of operands in turn."""
@@ -730,11 +731,46 @@ def geometry_families(capi, L):
                               "slowest": rows_[:5], "all": rows_}
     log(f"slice family: {len(rows_)} patterns, median {rows_[len(rows_) // 2]['pct_hbm_peak']}%, "
         f"slowest {rows_[0]['pct_hbm_peak']}%")
+    # (d) copies (what .contiguous() runs) of permuted tensors whose elements are not 4 bytes
+    # wide: bool masks, half / bfloat16, int64 / float64.  Bytes: 2 x the element size per element.
+    def timed_copy(shape, a_st, es):
+        n = 1
+        for s_ in shape:
+            n *= s_
+        sets = [(capi.DeviceBuffer(es * n), capi.DeviceBuffer(es * n)) for _ in range(kSets)]
+        it = capi.make_iter(shape, contig(shape), a_st)
+
+        def run(i):
+            da, do = sets[i]
+            capi.check(L.twg_copy_strided(do.ptr, da.ptr, es, ctypes.byref(it), None))
+        t = median_launch_seconds(run)
+        return round(2 * es * n / t / 1e9 / HBM_PEAK_GBS * 100, 1), round(t * 1e3, 4)
+
+    rows_ = []
+    for es in (1, 2, 8):
+        for shape, perm in (([8192, 4096], [1, 0]), ([16384, 8192], [1, 0]), ([128, 56, 56, 96], [0, 3, 1, 2]),
+                            ([256, 224, 224, 3], [0, 3, 1, 2]), ([256, 197, 768], [0, 2, 1]),
+                            ([64, 128, 64, 64], [0, 2, 1, 3]), ([2048, 96, 192], [0, 2, 1])):
+            nd = len(shape)
+            phys = contig([shape[p_] for p_ in perm])
+            a_st = [0] * nd
+            for pos, p_ in enumerate(perm):
+                a_st[p_] = phys[pos]
+            pct, ms = timed_copy(shape, a_st, es)
+            rows_.append({"pct_hbm_peak": pct, "ms": ms, "shape": shape, "a_memory_order": perm,
+                          "element_bytes": es, "launch_order": launches[0]})
+    rows_.sort(key=lambda r: r["pct_hbm_peak"])
+    fam["permuted_copies_of_1_2_8_byte_elements"] = {
+        "patterns": len(rows_), "median_pct": rows_[len(rows_) // 2]["pct_hbm_peak"], "slowest": rows_[:5],
+        "all": rows_}
+    log(f"copies of 1-, 2- and 8-byte elements: {len(rows_)} patterns, median "
+        f"{rows_[len(rows_) // 2]['pct_hbm_peak']}%, slowest {rows_[0]['pct_hbm_peak']}%")
     return {"geometry_families": fam, "elements_per_pattern": "about 2^25", "op": "add.Tensor fp32",
             "operand_sets_in_rotation": kSets,
             "launches_per_pattern": kSets + 3 * 12,
             "bytes": "4 B per element read per full operand + 4 B written; a broadcast operand counts its own size; "
-                     "a stepped operand counts the elements used, not the lines touched"}
+                     "a stepped operand counts the elements used, not the lines touched; the copies of the last family "
+                     "(twg_copy_strided, not add) move 2 x their element size per element"}
 
 
 def sweep(args, capi, W, L, torch, n, rows, cols, K, Wm, time_launches, summarize,
