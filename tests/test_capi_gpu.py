@@ -1098,6 +1098,18 @@ def test_copy_strided_every_element_size_and_layout(twg, dtype):
     check(rnd(16 + 320 * 256)[16:].view(320, 256).t(), what="transposed, storage offset of 16")
     check(rnd(3 + 320 * 256)[3:].view(320, 256).t(), what="transposed, storage offset of 3")
     check(rnd(256, 512).t(), out=torch.zeros(512, 512, dtype=dtype)[:, :256], what="transposed into a wider output")
+    # planar <-> interleaved with few channels (image batches between NCHW and NHWC): 1- and
+    # 2-byte elements take strips through LDS; several strips per row with a shorter last one,
+    # 2 to 32 channels, a batch, and a row length that is no whole number of packs (the gather)
+    check(rnd(2, 3, 224, 224).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, 3 channels")
+    check(rnd(2, 224, 224, 3).permute(0, 3, 1, 2), what="NHWC viewed as NCHW, 3 channels")
+    check(rnd(3, 16, 48, 48).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, 16 channels")
+    check(rnd(3, 48, 48, 16).permute(0, 3, 1, 2), what="NHWC viewed as NCHW, 16 channels")
+    check(rnd(2, 5, 64, 80).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, 5 channels")
+    check(rnd(2, 64, 80, 31).permute(0, 3, 1, 2), what="NHWC viewed as NCHW, 31 channels")
+    check(rnd(2, 32, 40, 40).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, 32 channels")
+    check(rnd(2, 1, 4096 + 272).expand(2, 7, 4096 + 272).transpose(1, 2), what="one plane for all 7 channels")
+    check(rnd(2, 3, 17, 19).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, ragged rows")
     if dtype == torch.uint8:  # from 2^26 elements on, 1-byte elements take wider tiles
         big = torch.randint(0, 256, (8192 + 144, 8192), generator=g, dtype=torch.uint8)
         check(big.t(), what="transposed, 2^26 elements and a ragged last tile")

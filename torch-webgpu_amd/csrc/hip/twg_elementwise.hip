@@ -141,6 +141,11 @@ int twg_copy_strided(void *out, const void *in, int32_t elem_size, const twg_ite
       rc = launch_tile_narrow(out, in, elem_size, g, resolve_stream(stream));
       if (rc != TWG_E_UNSUPPORTED) return rc;
     }
+    // ... and so have copies between planar and interleaved layouts with few channels
+    if (g.numel >= 4096) {
+      rc = launch_strip_narrow(out, in, elem_size, g, resolve_stream(stream));
+      if (rc != TWG_E_UNSUPPORTED) return rc;
+    }
   }
   switch (elem_size) {
     case 1:

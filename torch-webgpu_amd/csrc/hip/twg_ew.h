@@ -22,6 +22,7 @@
 //   twg_ew_strips.h ew_deint   - an input stored [.., x, c] with a short c against [.., c, x]
 //                   ew_inter   - its mirror image: a planar input against an output [.., x, c]
 //                   ew_pix     - a short c innermost everywhere, two outer dimensions swapped
+//                   ew_strip_narrow - planar <-> interleaved copies of 1- and 2-byte elements
 // This file: launch_ew, which canonicalizes the caller's geometry and picks the kernel.
 //
 // Replaces the two WGSL templates of the reference and their host drivers:

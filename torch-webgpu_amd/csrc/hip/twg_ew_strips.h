@@ -696,5 +696,174 @@ int launch_pix(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t
   }
 }
 
+// ------------------------------------------------------ ew_strip_narrow
+// Copies between planar and interleaved layouts ([.., c, x] <-> [.., x, c], 2..32 channels) for
+// elements of 1 and 2 bytes: uint8 and half image batches between NCHW and NHWC.  The strip
+// kernels above move 4-byte elements; one element per lane ran these at 11-17% of peak.  A
+// block takes a strip of TX values of x, parks what it reads in LDS as it lies in memory (16-byte
+// packs: c runs of TX elements, or one run of TX * c elements) and gathers each 16-byte output
+// pack element by element with narrow LDS reads.  TO_INTERLEAVED: the output is [.., x, c].
+// Offsets and strides in elements; every pack aligned (the launcher checks).
+struct StripNarrow {
+  int64_t nx;            // extent of x
+  int64_t cs_in, cs_out; // stride of c in the planar operand (input or output)
+  uint32_t P, tx, tiles; // channels, x per strip, strips per row
+  SmallDiv by_p;
+  int32_t nbatch;
+  int64_t bshape[TWG_MAX_DIMS - 2];
+  int64_t bstride[2][TWG_MAX_DIMS - 2];
+};
+
+template <int ES, bool TO_INTERLEAVED>
+__global__ __launch_bounds__(kThreads) void ew_strip_narrow(unsigned char *out, const unsigned char *in,
+                                                            StripNarrow g) {
+  constexpr uint32_t EPP = 16 / ES;
+  typedef uint32_t Words __attribute__((ext_vector_type(4)));
+  using Elem = typename std::conditional<ES == 1, uint8_t, uint16_t>::type;
+  extern __shared__ __attribute__((aligned(16))) unsigned char strip_lds[];
+  const Elem *cells = reinterpret_cast<const Elem *>(strip_lds);
+
+  uint32_t rem = blockIdx.x / g.tiles;
+  const uint32_t ti = blockIdx.x - rem * g.tiles;
+  int64_t off_o = 0, off_i = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = rem / extent;
+    const int64_t i = rem - q * extent;
+    rem = q;
+    off_o += i * g.bstride[0][d];
+    off_i += i * g.bstride[1][d];
+  }
+  const int64_t x0 = (int64_t)ti * g.tx;
+  const uint32_t nx = (uint32_t)(g.nx - x0 < (int64_t)g.tx ? g.nx - x0 : (int64_t)g.tx);  // a multiple of EPP
+  const uint32_t P = g.P, xpacks = nx / EPP;
+  // LDS: planar rows of pitch elements (one per channel; 16 bytes more than a full strip's run,
+  // so that rows start 4 banks apart), or the interleaved strip as it is
+  const uint32_t pitch = g.tx + EPP;
+
+  if constexpr (TO_INTERLEAVED) {
+    for (uint32_t i = threadIdx.x; i < P * xpacks; i += kThreads) {
+      const uint32_t c = i / xpacks, p = i - c * xpacks;
+      const Words v = __builtin_nontemporal_load(
+          reinterpret_cast<const Words *>(in + (off_i + (int64_t)c * g.cs_in + x0 + (int64_t)p * EPP) * ES));
+      *reinterpret_cast<Words *>(strip_lds + ((size_t)c * pitch + (size_t)p * EPP) * ES) = v;
+    }
+  } else {
+    for (uint32_t i = threadIdx.x; i < P * xpacks; i += kThreads) {  // nx * P elements, P * xpacks packs
+      const Words v = __builtin_nontemporal_load(
+          reinterpret_cast<const Words *>(in + (off_i + x0 * (int64_t)P + (int64_t)i * EPP) * ES));
+      *reinterpret_cast<Words *>(strip_lds + (size_t)i * 16) = v;
+    }
+  }
+  __syncthreads();
+
+  for (uint32_t i = threadIdx.x; i < P * xpacks; i += kThreads) {
+    Elem e[EPP];
+    unsigned char *dst;
+    if constexpr (TO_INTERLEAVED) {
+      // pack i of the strip as it lies in the output: elements j .. j + EPP - 1, (x, c) = (j / P, j % P)
+      const uint32_t j = i * EPP;
+      uint32_t x = div_by(j, g.by_p), c = j - x * P;
+#pragma unroll
+      for (uint32_t k = 0; k < EPP; ++k) {
+        e[k] = cells[c * pitch + x];
+        if (++c == P) {
+          c = 0;
+          ++x;
+        }
+      }
+      dst = out + (off_o + x0 * (int64_t)P + j) * ES;
+    } else {
+      // pack p of channel c: x = p * EPP .. + EPP - 1, out of the interleaved strip.  With an
+      // even channel count, lanes that follow one another take the channels of one p, so that
+      // their reads are neighbouring bytes: the packs of one channel lie EPP * P elements apart,
+      // which for 16 channels of bytes is one bank for all of them (14% of peak that way, 58%
+      // this way).  With an odd count they take the packs of one channel, which keeps their
+      // stores together (3 channels of 2-byte elements: 72% against 67%).
+      uint32_t c, p;
+      if (P & 1u) {
+        c = i / xpacks;
+        p = i - c * xpacks;
+      } else {
+        p = div_by(i, g.by_p);
+        c = i - p * P;
+      }
+#pragma unroll
+      for (uint32_t k = 0; k < EPP; ++k) e[k] = cells[(p * EPP + k) * P + c];
+      dst = out + (off_o + (int64_t)c * g.cs_out + x0 + (int64_t)p * EPP) * ES;
+    }
+    Words w;
+    if constexpr (ES == 2) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[q] = (uint32_t)e[2 * q] | ((uint32_t)e[2 * q + 1] << 16);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        w[q] = (uint32_t)e[4 * q] | ((uint32_t)e[4 * q + 1] << 8) | ((uint32_t)e[4 * q + 2] << 16) |
+               ((uint32_t)e[4 * q + 3] << 24);
+    }
+    __builtin_nontemporal_store(w, reinterpret_cast<Words *>(dst));
+  }
+}
+
+// A copy of 1- or 2-byte elements between [.., c, x] and [.., x, c] with 2..32 channels.  Returns
+// TWG_E_UNSUPPORTED unless the geometry is of that kind with every 16-byte pack aligned.
+inline int launch_strip_narrow(void *out, const void *in, int es, const Geom &g, hipStream_t s) {
+  if ((es != 1 && es != 2) || g.ndim < 2 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
+  const int64_t epp = 16 / es;
+  if (!aligned_to(out, 16) || !aligned_to(in, 16)) return TWG_E_UNSUPPORTED;
+  StripNarrow sg{};
+  int xd = -1, cd = -1;
+  bool to_interleaved;
+  if (g.shape[0] >= 2 && g.shape[0] <= 32 && g.stride[0][1] == g.shape[0] && g.stride[1][1] == 1 &&
+      g.stride[1][0] != 0 && g.stride[1][0] != 1) {
+    // output [.., x, c] (dimension 0 = c, dimension 1 = x), input planar
+    to_interleaved = true;
+    cd = 0;
+    xd = 1;
+    sg.cs_in = g.stride[1][0];
+  } else {
+    // output planar (dimension 0 = x), input [.., x, c]: the dimension with unit input stride is c
+    to_interleaved = false;
+    xd = 0;
+    for (int d = 1; d < g.ndim && cd < 0; ++d)
+      if (g.stride[1][d] == 1 && g.shape[d] >= 2 && g.shape[d] <= 32 && g.stride[1][0] == g.shape[d]) cd = d;
+    if (cd < 0) return TWG_E_UNSUPPORTED;
+    sg.cs_out = g.stride[0][cd];
+  }
+  const int64_t P = g.shape[cd];
+  sg.nx = g.shape[xd];
+  if (sg.nx % epp || sg.nx < 256) return TWG_E_UNSUPPORTED;
+  if ((to_interleaved ? sg.cs_in : sg.cs_out) % epp) return TWG_E_UNSUPPORTED;
+  int64_t batch = 1;
+  for (int d = 0; d < g.ndim; ++d) {
+    if (d == xd || d == cd) continue;
+    if (g.stride[0][d] % epp || g.stride[1][d] % epp) return TWG_E_UNSUPPORTED;
+    sg.bshape[sg.nbatch] = g.shape[d];
+    sg.bstride[0][sg.nbatch] = g.stride[0][d];
+    sg.bstride[1][sg.nbatch] = g.stride[1][d];
+    sg.nbatch++;
+    batch *= g.shape[d];
+  }
+  // about 8 KiB per strip, a power of two of x values
+  uint32_t tx = 4096;
+  while (tx > 64 && (int64_t)tx * P * es > 8192) tx /= 2;
+  sg.P = (uint32_t)P;
+  sg.tx = tx;
+  const int64_t tiles = (sg.nx + tx - 1) / tx;
+  if (tiles > INT32_MAX || batch > INT32_MAX || tiles * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+  sg.tiles = (uint32_t)tiles;
+  sg.by_p = small_div((uint32_t)P);
+  const size_t lds = to_interleaved ? (size_t)P * (tx + epp) * es : (size_t)P * tx * es;
+  const unsigned grid = (unsigned)(tiles * batch);
+  unsigned char *o = static_cast<unsigned char *>(out);
+  const unsigned char *i = static_cast<const unsigned char *>(in);
+  if (es == 1 && to_interleaved) ew_strip_narrow<1, true><<<grid, kThreads, lds, s>>>(o, i, sg);
+  else if (es == 1) ew_strip_narrow<1, false><<<grid, kThreads, lds, s>>>(o, i, sg);
+  else if (to_interleaved) ew_strip_narrow<2, true><<<grid, kThreads, lds, s>>>(o, i, sg);
+  else ew_strip_narrow<2, false><<<grid, kThreads, lds, s>>>(o, i, sg);
+  return (int)hipGetLastError();
+}
+
 }  // namespace
 }  // namespace twg
