@@ -141,7 +141,8 @@ int twg_copy_strided(void *out, const void *in, int32_t elem_size, const twg_ite
       rc = launch_tile_narrow(out, in, elem_size, g, resolve_stream(stream));
       if (rc != TWG_E_UNSUPPORTED) return rc;
     }
-    // ... and so have copies between planar and interleaved layouts with few channels
+    // ... and so have copies between planar and interleaved layouts with few channels (8-byte
+    // elements: 77-80% of peak against 28-63% as pairs of words)
     if (g.numel >= 4096) {
       rc = launch_strip_narrow(out, in, elem_size, g, resolve_stream(stream));
       if (rc != TWG_E_UNSUPPORTED) return rc;

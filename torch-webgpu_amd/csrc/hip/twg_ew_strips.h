@@ -698,7 +698,7 @@ int launch_pix(TO *out, const TA *a, const TB *b, const Geom &g, int t, bool a_t
 
 // ------------------------------------------------------ ew_strip_narrow
 // Copies between planar and interleaved layouts ([.., c, x] <-> [.., x, c], 2..32 channels) for
-// elements of 1 and 2 bytes: uint8 and half image batches between NCHW and NHWC.  The strip
+// elements of 1, 2 and 8 bytes: uint8 and half image batches between NCHW and NHWC.  The strip
 // kernels above move 4-byte elements; one element per lane ran these at 11-17% of peak.  A
 // block takes a strip of TX values of x, parks what it reads in LDS as it lies in memory (16-byte
 // packs: c runs of TX elements, or one run of TX * c elements) and gathers each 16-byte output
@@ -719,7 +719,7 @@ __global__ __launch_bounds__(kThreads) void ew_strip_narrow(unsigned char *out, 
                                                             StripNarrow g) {
   constexpr uint32_t EPP = 16 / ES;
   typedef uint32_t Words __attribute__((ext_vector_type(4)));
-  using Elem = typename std::conditional<ES == 1, uint8_t, uint16_t>::type;
+  using Elem = typename std::conditional<ES == 1, uint8_t, typename std::conditional<ES == 2, uint16_t, uint64_t>::type>::type;
   extern __shared__ __attribute__((aligned(16))) unsigned char strip_lds[];
   const Elem *cells = reinterpret_cast<const Elem *>(strip_lds);
 
@@ -793,7 +793,12 @@ __global__ __launch_bounds__(kThreads) void ew_strip_narrow(unsigned char *out, 
       dst = out + (off_o + (int64_t)c * g.cs_out + x0 + (int64_t)p * EPP) * ES;
     }
     Words w;
-    if constexpr (ES == 2) {
+    if constexpr (ES == 8) {
+      w[0] = (uint32_t)e[0];
+      w[1] = (uint32_t)(e[0] >> 32);
+      w[2] = (uint32_t)e[1];
+      w[3] = (uint32_t)(e[1] >> 32);
+    } else if constexpr (ES == 2) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) w[q] = (uint32_t)e[2 * q] | ((uint32_t)e[2 * q + 1] << 16);
     } else {
@@ -806,10 +811,10 @@ __global__ __launch_bounds__(kThreads) void ew_strip_narrow(unsigned char *out, 
   }
 }
 
-// A copy of 1- or 2-byte elements between [.., c, x] and [.., x, c] with 2..32 channels.  Returns
+// A copy of 1-, 2- or 8-byte elements between [.., c, x] and [.., x, c] with 2..32 channels.  Returns
 // TWG_E_UNSUPPORTED unless the geometry is of that kind with every 16-byte pack aligned.
 inline int launch_strip_narrow(void *out, const void *in, int es, const Geom &g, hipStream_t s) {
-  if ((es != 1 && es != 2) || g.ndim < 2 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
+  if ((es != 1 && es != 2 && es != 8) || g.ndim < 2 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
   const int64_t epp = 16 / es;
   if (!aligned_to(out, 16) || !aligned_to(in, 16)) return TWG_E_UNSUPPORTED;
   StripNarrow sg{};
@@ -858,7 +863,9 @@ inline int launch_strip_narrow(void *out, const void *in, int es, const Geom &g,
   const unsigned grid = (unsigned)(tiles * batch);
   unsigned char *o = static_cast<unsigned char *>(out);
   const unsigned char *i = static_cast<const unsigned char *>(in);
-  if (es == 1 && to_interleaved) ew_strip_narrow<1, true><<<grid, kThreads, lds, s>>>(o, i, sg);
+  if (es == 8 && to_interleaved) ew_strip_narrow<8, true><<<grid, kThreads, lds, s>>>(o, i, sg);
+  else if (es == 8) ew_strip_narrow<8, false><<<grid, kThreads, lds, s>>>(o, i, sg);
+  else if (es == 1 && to_interleaved) ew_strip_narrow<1, true><<<grid, kThreads, lds, s>>>(o, i, sg);
   else if (es == 1) ew_strip_narrow<1, false><<<grid, kThreads, lds, s>>>(o, i, sg);
   else if (to_interleaved) ew_strip_narrow<2, true><<<grid, kThreads, lds, s>>>(o, i, sg);
   else ew_strip_narrow<2, false><<<grid, kThreads, lds, s>>>(o, i, sg);
