@@ -1110,6 +1110,22 @@ def test_copy_strided_every_element_size_and_layout(twg, dtype):
     check(rnd(2, 32, 40, 40).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, 32 channels")
     check(rnd(2, 1, 4096 + 272).expand(2, 7, 4096 + 272).transpose(1, 2), what="one plane for all 7 channels")
     check(rnd(2, 3, 17, 19).permute(0, 2, 3, 1), what="NCHW viewed as NHWC, ragged rows")
+    # output rows that are no whole number of packs, the output dense across them (1- and 2-byte
+    # elements: blocks write whole rows as one run of aligned packs with a head and a tail)
+    check(rnd(3, 197, 768).transpose(1, 2), what="rows of 197")
+    check(rnd(2, 33, 640).transpose(1, 2), what="rows of 33")
+    check(rnd(511, 256).t(), what="rows of 511, two dimensions")
+    check(rnd(5, 9, 128).transpose(1, 2), what="rows of 9")
+    check(rnd(1 + 2 * 77 * 192)[1:].view(2, 77, 192).transpose(1, 2), what="rows of 77, storage offset of 1")
+    check(rnd(2, 77, 192).transpose(1, 2), out=torch.zeros(1 + 2 * 192 * 77, dtype=dtype)[1:].view(2, 192, 77),
+          what="rows of 77 into an output that starts off a pack")
+    # the mirror image: input rows that are no whole number of packs, the input dense across them
+    check(rnd(3, 768, 197).transpose(1, 2), what="input rows of 197")
+    check(rnd(2, 640, 33).transpose(1, 2), what="input rows of 33")
+    check(rnd(256, 511).t(), what="input rows of 511, two dimensions")
+    check(rnd(5, 128, 9).transpose(1, 2), what="input rows of 9")
+    check(rnd(1 + 2 * 192 * 77)[1:].view(2, 192, 77).transpose(1, 2), what="input rows of 77, storage offset of 1")
+    check(rnd(2, 1000, 77).transpose(1, 2), what="input rows of 77, a last block of 40 rows")
     if dtype == torch.uint8:  # from 2^26 elements on, 1-byte elements take wider tiles
         big = torch.randint(0, 256, (8192 + 144, 8192), generator=g, dtype=torch.uint8)
         check(big.t(), what="transposed, 2^26 elements and a ragged last tile")

@@ -147,6 +147,13 @@ int twg_copy_strided(void *out, const void *in, int32_t elem_size, const twg_ite
       rc = launch_strip_narrow(out, in, elem_size, g, resolve_stream(stream));
       if (rc != TWG_E_UNSUPPORTED) return rc;
     }
+    // ... and transposes whose output rows, or whose input rows, are no whole number of packs
+    if (g.numel >= 4096) {
+      rc = launch_rowtile_narrow(out, in, elem_size, g, resolve_stream(stream));
+      if (rc != TWG_E_UNSUPPORTED) return rc;
+      rc = launch_coltile_narrow(out, in, elem_size, g, resolve_stream(stream));
+      if (rc != TWG_E_UNSUPPORTED) return rc;
+    }
   }
   switch (elem_size) {
     case 1:

@@ -688,5 +688,259 @@ inline int launch_tile_narrow(void *out, const void *in, int es, const Geom &g, 
   return (int)hipGetLastError();
 }
 
+// ----------------------------------------------------- ew_rowtile_narrow
+// Transposing copies of 1- and 2-byte elements whose output rows are no whole number of
+// 16-byte packs (a [B, 197, 768] tensor of half viewed as [B, 768, 197]): ew_tile_narrow needs
+// every output row to start on a pack.  Here the output is dense across dimensions 0 (x, any
+// extent up to 512) and 1 (y), so a block's share, TY whole rows, is one contiguous run of
+// TY * X elements: it is written as aligned 16-byte packs that may span two rows, with the few
+// elements before the first and after the last aligned pack stored one by one.  The input's
+// runs (TY elements along y for each x, aligned packs) are parked in LDS as they lie in memory
+// and every output element is picked up with a narrow LDS read.  Offsets and strides in elements.
+struct RowTileNarrow {
+  uint32_t X, ty, tiles;      // extent of x, rows per block, blocks per batch entry
+  int64_t Y, sx;              // extent of y, input stride along x
+  SmallDiv by_x;
+  int32_t nbatch;
+  int64_t bshape[TWG_MAX_DIMS - 2];
+  int64_t bstride[2][TWG_MAX_DIMS - 2];
+};
+
+template <int ES>
+__global__ __launch_bounds__(kThreads) void ew_rowtile_narrow(unsigned char *out, const unsigned char *in,
+                                                              RowTileNarrow g) {
+  constexpr uint32_t EPP = 16 / ES;
+  typedef uint32_t Words __attribute__((ext_vector_type(4)));
+  using Elem = typename std::conditional<ES == 1, uint8_t, uint16_t>::type;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rowtile_lds[];
+  const Elem *cells = reinterpret_cast<const Elem *>(rowtile_lds);
+
+  uint32_t rem = blockIdx.x / g.tiles;
+  const uint32_t ti = blockIdx.x - rem * g.tiles;
+  int64_t off_o = 0, off_i = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = rem / extent;
+    const int64_t i = rem - q * extent;
+    rem = q;
+    off_o += i * g.bstride[0][d];
+    off_i += i * g.bstride[1][d];
+  }
+  const int64_t y0 = (int64_t)ti * g.ty;
+  const uint32_t ny = (uint32_t)(g.Y - y0 < (int64_t)g.ty ? g.Y - y0 : (int64_t)g.ty);  // a multiple of EPP
+  const uint32_t X = g.X, ypacks = ny / EPP;
+  const uint32_t pitch = g.ty + 4 / ES;  // elements between two x in LDS: an odd number of words
+
+  // the input: for each x, ny elements along y
+  for (uint32_t i = threadIdx.x; i < X * ypacks; i += kThreads) {
+    const uint32_t x = i / ypacks, p = i - x * ypacks;
+    const Words v = __builtin_nontemporal_load(
+        reinterpret_cast<const Words *>(in + (off_i + (int64_t)x * g.sx + y0 + (int64_t)p * EPP) * ES));
+    uint32_t *dst = reinterpret_cast<uint32_t *>(rowtile_lds + ((size_t)x * pitch + (size_t)p * EPP) * ES);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) dst[c] = v[c];
+  }
+  __syncthreads();
+
+  // the output: ny * X consecutive elements from `first` on
+  Elem *first = reinterpret_cast<Elem *>(out) + off_o + y0 * (int64_t)X;
+  const uint32_t total = ny * X;
+  uint32_t head = (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(first) & 15u)) & 15u) / ES;
+  if (head > total) head = total;
+  const uint32_t npacks = (total - head) / EPP, tail0 = head + npacks * EPP;
+  auto cell_of = [&](uint32_t j) {  // element j of the run: row j / X, column j % X
+    const uint32_t y = div_by(j, g.by_x), x = j - y * X;
+    return cells[x * pitch + y];
+  };
+  if (threadIdx.x < head) first[threadIdx.x] = cell_of(threadIdx.x);
+  if (threadIdx.x < total - tail0) first[tail0 + threadIdx.x] = cell_of(tail0 + threadIdx.x);
+  for (uint32_t i = threadIdx.x; i < npacks; i += kThreads) {
+    const uint32_t j = head + i * EPP;
+    uint32_t y = div_by(j, g.by_x), x = j - y * X;
+    Elem e[EPP];
+#pragma unroll
+    for (uint32_t k = 0; k < EPP; ++k) {
+      e[k] = cells[x * pitch + y];
+      if (++x == X) {
+        x = 0;
+        ++y;
+      }
+    }
+    Words w;
+    if constexpr (ES == 2) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[q] = (uint32_t)e[2 * q] | ((uint32_t)e[2 * q + 1] << 16);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        w[q] = (uint32_t)e[4 * q] | ((uint32_t)e[4 * q + 1] << 8) | ((uint32_t)e[4 * q + 2] << 16) |
+               ((uint32_t)e[4 * q + 3] << 24);
+    }
+    __builtin_nontemporal_store(w, reinterpret_cast<Words *>(first + j));
+  }
+}
+
+// The output dense across dimensions 0 and 1 (rows of X <= 512 elements, X no multiple of the
+// pack), the input with unit stride along dimension 1 and aligned packs there.  Returns
+// TWG_E_UNSUPPORTED for anything else.
+inline int launch_rowtile_narrow(void *out, const void *in, int es, const Geom &g, hipStream_t s) {
+  if ((es != 1 && es != 2) || g.ndim < 2 || g.stride[0][0] != 1 || g.stride[0][1] != g.shape[0] ||
+      g.stride[1][1] != 1 || g.stride[1][0] == 1)
+    return TWG_E_UNSUPPORTED;
+  const int64_t epp = 16 / es, X = g.shape[0], Y = g.shape[1];
+  if (X < 8 || X > 512 || Y < 64 || Y % epp || g.stride[1][0] % epp || g.stride[1][0] == 0 ||
+      !aligned_to(in, 16) || reinterpret_cast<uintptr_t>(out) % es)
+    return TWG_E_UNSUPPORTED;
+  RowTileNarrow rg{};
+  int64_t batch = 1;
+  for (int d = 2; d < g.ndim; ++d) {
+    if (g.stride[1][d] % epp) return TWG_E_UNSUPPORTED;
+    rg.bshape[rg.nbatch] = g.shape[d];
+    rg.bstride[0][rg.nbatch] = g.stride[0][d];
+    rg.bstride[1][rg.nbatch] = g.stride[1][d];
+    rg.nbatch++;
+    batch *= g.shape[d];
+  }
+  // rows per block: 128 bytes of each input run (a whole line) while the tile fits 32 KiB of
+  // LDS, down to 16 rows
+  uint32_t ty = 128 / es;
+  while (ty > 16 && (int64_t)X * (ty + 4 / es) * es > 32768) ty /= 2;
+  if ((int64_t)X * (ty + 4 / es) * es > 49152) return TWG_E_UNSUPPORTED;
+  rg.X = (uint32_t)X;
+  rg.Y = Y;
+  rg.sx = g.stride[1][0];
+  rg.ty = ty;
+  rg.by_x = small_div((uint32_t)X);
+  const int64_t tiles = (Y + ty - 1) / ty;
+  if (tiles > INT32_MAX || batch > INT32_MAX || tiles * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+  rg.tiles = (uint32_t)tiles;
+  const size_t lds = (size_t)X * (ty + 4 / es) * es;
+  const unsigned grid = (unsigned)(tiles * batch);
+  unsigned char *o = static_cast<unsigned char *>(out);
+  const unsigned char *i = static_cast<const unsigned char *>(in);
+  if (es == 1) ew_rowtile_narrow<1><<<grid, kThreads, lds, s>>>(o, i, rg);
+  else ew_rowtile_narrow<2><<<grid, kThreads, lds, s>>>(o, i, rg);
+  return (int)hipGetLastError();
+}
+
+// The mirror image: the INPUT's rows are no whole number of packs (a [B, 768, 197] tensor of
+// half viewed as [B, 197, 768]) and the input is dense across them, so a block's share of it,
+// TX rows of Y elements, is one contiguous run: read as aligned packs, with the few elements
+// before the first and after the last aligned pack fetched one by one, and parked in LDS as it
+// lies in memory.  The output's rows (TX elements along dimension 0 for each y) are whole packs.
+struct ColTileNarrow {
+  uint32_t Y, tx, tiles;      // extent of y, input rows per block, blocks per batch entry
+  int64_t X, sy;              // extent of dimension 0, output stride along y
+  int32_t nbatch;
+  int64_t bshape[TWG_MAX_DIMS - 2];
+  int64_t bstride[2][TWG_MAX_DIMS - 2];
+};
+
+template <int ES>
+__global__ __launch_bounds__(kThreads) void ew_coltile_narrow(unsigned char *out, const unsigned char *in,
+                                                              ColTileNarrow g) {
+  constexpr uint32_t EPP = 16 / ES;
+  typedef uint32_t Words __attribute__((ext_vector_type(4)));
+  using Elem = typename std::conditional<ES == 1, uint8_t, uint16_t>::type;
+  extern __shared__ __attribute__((aligned(16))) unsigned char coltile_lds[];
+  Elem *cells = reinterpret_cast<Elem *>(coltile_lds);
+
+  uint32_t rem = blockIdx.x / g.tiles;
+  const uint32_t ti = blockIdx.x - rem * g.tiles;
+  int64_t off_o = 0, off_i = 0;
+  for (int d = 0; d < g.nbatch; ++d) {
+    const uint32_t extent = (uint32_t)g.bshape[d];
+    const uint32_t q = rem / extent;
+    const int64_t i = rem - q * extent;
+    rem = q;
+    off_o += i * g.bstride[0][d];
+    off_i += i * g.bstride[1][d];
+  }
+  const int64_t x0 = (int64_t)ti * g.tx;
+  const uint32_t nx = (uint32_t)(g.X - x0 < (int64_t)g.tx ? g.X - x0 : (int64_t)g.tx);  // a multiple of EPP
+  const uint32_t Y = g.Y, total = nx * Y;
+
+  // the input: total consecutive elements from `first` on.  Element j is parked at cells[shift + j],
+  // shift chosen so that the aligned packs of memory are aligned packs of LDS.
+  const Elem *first = reinterpret_cast<const Elem *>(in) + off_i + x0 * (int64_t)Y;
+  uint32_t head = (uint32_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(first) & 15u)) & 15u) / ES;
+  if (head > total) head = total;
+  const uint32_t shift = (EPP - head % EPP) % EPP;
+  const uint32_t npacks = (total - head) / EPP, tail0 = head + npacks * EPP;
+  if (threadIdx.x < head) cells[shift + threadIdx.x] = first[threadIdx.x];
+  if (threadIdx.x < total - tail0) cells[shift + tail0 + threadIdx.x] = first[tail0 + threadIdx.x];
+  for (uint32_t i = threadIdx.x; i < npacks; i += kThreads) {
+    const uint32_t j = head + i * EPP;
+    const Words v = __builtin_nontemporal_load(reinterpret_cast<const Words *>(first + j));
+    *reinterpret_cast<Words *>(cells + shift + j) = v;
+  }
+  __syncthreads();
+
+  // the output: for each y, nx elements along dimension 0; lane -> (y within a group of 8, pack)
+  const uint32_t xpacks = nx / EPP, ygroups = (Y + 7) / 8;
+  for (uint32_t i = threadIdx.x; i < ygroups * 8 * xpacks; i += kThreads) {
+    const uint32_t ys = i & 7u, r = i >> 3, yg = r / xpacks, xp = r - yg * xpacks, y = yg * 8 + ys;
+    if (y >= Y) continue;
+    const Elem *col = cells + shift + (size_t)(xp * EPP) * Y + y;
+    Words w;
+    if constexpr (ES == 2) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[q] = (uint32_t)col[(2 * q) * Y] | ((uint32_t)col[(2 * q + 1) * Y] << 16);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        w[q] = (uint32_t)col[(4 * q) * Y] | ((uint32_t)col[(4 * q + 1) * Y] << 8) |
+               ((uint32_t)col[(4 * q + 2) * Y] << 16) | ((uint32_t)col[(4 * q + 3) * Y] << 24);
+    }
+    __builtin_nontemporal_store(
+        w, reinterpret_cast<Words *>(out + (off_o + (int64_t)y * g.sy + x0 + (int64_t)xp * EPP) * ES));
+  }
+}
+
+// The input dense across dimension t (unit stride, Y <= 512 elements, no multiple of the pack)
+// and dimension 0, the output with unit stride along dimension 0 and aligned packs there.
+// Returns TWG_E_UNSUPPORTED for anything else.
+inline int launch_coltile_narrow(void *out, const void *in, int es, const Geom &g, hipStream_t s) {
+  if ((es != 1 && es != 2) || g.ndim < 2 || g.stride[0][0] != 1) return TWG_E_UNSUPPORTED;
+  int t = -1;
+  for (int d = 1; d < g.ndim && t < 0; ++d)
+    if (g.stride[1][d] == 1 && g.stride[1][0] == g.shape[d]) t = d;
+  if (t < 0) return TWG_E_UNSUPPORTED;
+  const int64_t epp = 16 / es, X = g.shape[0], Y = g.shape[t];
+  if (Y < 8 || Y > 512 || X < 64 || X % epp || !aligned_to(out, 16) ||
+      reinterpret_cast<uintptr_t>(in) % es)
+    return TWG_E_UNSUPPORTED;
+  ColTileNarrow cg{};
+  int64_t batch = 1;
+  for (int d = 1; d < g.ndim; ++d) {
+    if (g.stride[0][d] % epp) return TWG_E_UNSUPPORTED;
+    if (d == t) continue;
+    cg.bshape[cg.nbatch] = g.shape[d];
+    cg.bstride[0][cg.nbatch] = g.stride[0][d];
+    cg.bstride[1][cg.nbatch] = g.stride[1][d];
+    cg.nbatch++;
+    batch *= g.shape[d];
+  }
+  // input rows per block: 128 bytes of each output run (a whole line) while the tile fits
+  // 32 KiB of LDS, down to 16 rows
+  uint32_t tx = 128 / es;
+  while (tx > 16 && ((int64_t)tx * Y + epp) * es > 32768) tx /= 2;
+  if (((int64_t)tx * Y + epp) * es > 49152) return TWG_E_UNSUPPORTED;
+  cg.Y = (uint32_t)Y;
+  cg.X = X;
+  cg.sy = g.stride[0][t];
+  cg.tx = tx;
+  const int64_t tiles = (X + tx - 1) / tx;
+  if (tiles > INT32_MAX || batch > INT32_MAX || tiles * batch > INT32_MAX) return TWG_E_UNSUPPORTED;
+  cg.tiles = (uint32_t)tiles;
+  const size_t lds = (size_t)(tx * Y + epp) * es;
+  const unsigned grid = (unsigned)(tiles * batch);
+  unsigned char *o = static_cast<unsigned char *>(out);
+  const unsigned char *i = static_cast<const unsigned char *>(in);
+  if (es == 1) ew_coltile_narrow<1><<<grid, kThreads, lds, s>>>(o, i, cg);
+  else ew_coltile_narrow<2><<<grid, kThreads, lds, s>>>(o, i, cg);
+  return (int)hipGetLastError();
+}
+
 }  // namespace
 }  // namespace twg
