@@ -18,7 +18,8 @@
 //   twg_ew_tile.h   ew_tile, ew_tile_vec, ew_tile_any - an input whose unit stride lies along
 //                                another dimension than the output's: tiles staged through LDS so
 //                                that both sides of the transpose stay coalesced
-//                   ew_tile_narrow - the same for copies of 1- and 2-byte elements
+//                   ew_tile_narrow, ew_rowtile_narrow, ew_coltile_narrow - the same for copies of
+//                                1-, 2- and 8-byte elements (aligned packs; ragged rows on one side)
 //   twg_ew_strips.h ew_deint   - an input stored [.., x, c] with a short c against [.., c, x]
 //                   ew_inter   - its mirror image: a planar input against an output [.., x, c]
 //                   ew_pix     - a short c innermost everywhere, two outer dimensions swapped

@@ -1,6 +1,7 @@
 // Elementwise kernels for an operand whose unit stride lies along another dimension than the
-// output's: tiles transposed through LDS (ew_tile, ew_tile_vec, ew_tile_any; ew_tile_narrow for
-// copies of 1- and 2-byte elements), with their launchers.
+// output's: tiles transposed through LDS (ew_tile, ew_tile_vec, ew_tile_any; ew_tile_narrow,
+// ew_rowtile_narrow and ew_coltile_narrow for copies of 1-, 2- and 8-byte elements), with their
+// launchers.
 #pragma once
 
 #include "twg_ew_packs.h"
