@@ -719,7 +719,8 @@ __global__ __launch_bounds__(kThreads) void ew_strip_narrow(unsigned char *out, 
                                                             StripNarrow g) {
   constexpr uint32_t EPP = 16 / ES;
   typedef uint32_t Words __attribute__((ext_vector_type(4)));
-  using Elem = typename std::conditional<ES == 1, uint8_t, typename std::conditional<ES == 2, uint16_t, uint64_t>::type>::type;
+  using Wide = typename std::conditional<ES == 2, uint16_t, uint64_t>::type;
+  using Elem = typename std::conditional<ES == 1, uint8_t, Wide>::type;
   extern __shared__ __attribute__((aligned(16))) unsigned char strip_lds[];
   const Elem *cells = reinterpret_cast<const Elem *>(strip_lds);
 

@@ -565,7 +565,8 @@ __global__ __launch_bounds__(kThreads) void ew_tile_narrow(unsigned char *out, c
   constexpr int kPacksT = TT / EPP, kPacks0 = TD0 / EPP;
   static_assert(kRowWords % 4 == 0 && TT % 8 == 0 && TD0 % EPP == 0 && kPacks0 >= 8, "tile shape");
   typedef uint32_t Words __attribute__((ext_vector_type(4)));
-  using Elem = typename std::conditional<ES == 1, uint8_t, typename std::conditional<ES == 2, uint16_t, uint64_t>::type>::type;
+  using Wide = typename std::conditional<ES == 2, uint16_t, uint64_t>::type;
+  using Elem = typename std::conditional<ES == 1, uint8_t, Wide>::type;
   __shared__ uint32_t lds[TD0 * kPitch];
 
   uint32_t t0i, tti;
